@@ -1,0 +1,125 @@
+/*
+ * libsfbert_hip -- C ABI of the MI355X (gfx950) block-sparse attention path.
+ *
+ * Plain pointers and sizes only.  Device pointers are marked [dev], host pointers [host].  Every
+ * device entry point enqueues work on the given HIP stream and returns without synchronising; it
+ * allocates nothing and keeps no state.  Tensors Q/K/V/O are [batch, ctx, heads, head_state]
+ * contiguous (element offset b*ctx*H*d + token*H*d + h*d + k), sparse S/P tensors are
+ * [batch][heads][blocks][bs][bs], exactly as the reference lays them out
+ * (openai_blocksparse.h:40-41,148).  Each declaration cites the reference interface it replaces.
+ *
+ * All functions return an sfb_status (0 = ok) unless stated otherwise.
+ */
+#ifndef SFBERT_HIP_H
+#define SFBERT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The reference's CUDA uint2 LUT entry (openai_blocksparse.h:203) as a plain POD. */
+typedef struct { uint32_t x, y; } sfb_uint2;
+
+/* hipStream_t, passed as an opaque pointer (the reference passes CUstream, openai_blocksparse.h:202). */
+typedef void* sfb_stream_t;
+
+typedef enum {
+    SFB_OK = 0,
+    SFB_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    SFB_ERR_BLOCK_SIZE = 2,     /* block size not supported by this entry point */
+    SFB_ERR_HEAD_STATE = 3,     /* head_state (d) not supported */
+    SFB_ERR_SHAPE = 4,          /* zero / inconsistent dimensions */
+    SFB_ERR_DTYPE = 5,          /* unknown or unsupported element type */
+    SFB_ERR_ALIGNMENT = 6,      /* a tensor pointer is not 16-byte aligned */
+    SFB_ERR_LAUNCH = 7,         /* hipGetLastError() reported a failure after the launch */
+    SFB_ERR_ARGUMENT = 8,       /* other invalid argument (op code, pattern parameter ...) */
+    SFB_ERR_WORKSPACE = 9       /* workspace missing or too small */
+} sfb_status;
+
+typedef enum { SFB_F32 = 0, SFB_BF16 = 1 } sfb_dtype;
+
+/* NT_OP / NN_OP / TN_OP of gpu_types.h:135-137 */
+enum { SFB_NT_OP = 0, SFB_NN_OP = 1, SFB_TN_OP = 2 };
+
+const char* sfb_status_string(int status);
+/* 1 when the library was built for gfx950 and a HIP device is usable, else 0. */
+int sfb_device_available(void);
+
+/* ================================================================================================
+ * Host-side descriptors (integer work on [host] arrays; bit-exact with the reference's formats)
+ * ============================================================================================== */
+
+/* layout[heads][nb][nb], 1 = (query block row, key block column) attended. */
+/* no_fusion_test.cu:47-62 (causal != 0: i >= j; causal == 0: dense). */
+int sfb_layout_full(uint32_t* layout, int nb, int causal);
+/* local_fusion_test.cu:46-63 (bidirectional == 0: the reference's causal band; != 0: |i-j| <= extra_diag). */
+int sfb_layout_local(uint32_t* layout, int nb, int extra_diag, int bidirectional);
+/* fixed_fusion_test.cu:52-106: per-head summary column phase stride-(h+1), own chunk, optional causal cut. */
+int sfb_layout_fixed(uint32_t* layout, int heads, int nb, int stride, int causal);
+/* stride_fusion_test.cu:48-71: j <= i && j + (i % block_chunks) >= i. */
+int sfb_layout_strided_chunks(uint32_t* layout, int nb, int block_chunks);
+/* Block form of the element rule ewops.h:462-503: band of `band` blocks plus (i-j) % stride == 0. */
+int sfb_layout_strided(uint32_t* layout, int nb, int band, int stride, int causal);
+/* big_bird_fusion_test.cu:50-99: window, `nglobal` dense rows+columns (first ones, or split between both
+ * ends), plus rand_cols[nb][nrand] random key blocks per row (-1 = none; NULL = no random blocks). */
+int sfb_layout_bigbird(uint32_t* layout, int nb, int window, int nglobal, int global_both_ends,
+                       const int32_t* rand_cols, int nrand);
+/* Seeded replacement of the reference's unseeded rand()%10 draw (big_bird_fusion_test.cu:81-99):
+ * nrand distinct still-empty columns per block-row, splitmix64 + partial Fisher-Yates. */
+int sfb_bigbird_draw(int32_t* rand_cols, int nb, int window, int nglobal, int global_both_ends,
+                     int nrand, uint64_t seed);
+
+/* local_fusion_test.cu:78-85: number of nonzero blocks of one head's layout. */
+uint32_t sfb_count_blocks(const uint32_t* layout, int nb);
+/* local_fusion_test.cu:89-99: nt_lut[blocks] = {row block, col block}, row-major scan. */
+int sfb_build_nt_lut(sfb_uint2* nt_lut, const uint32_t* layout, int nb);
+/* local_fusion_test.cu:106-133: nn_lut[nb + blocks]; *nn_max is read as the initial value and updated. */
+int sfb_build_nn_lut(sfb_uint2* nn_lut, const sfb_uint2* nt_lut, uint32_t blocks, int nb,
+                     uint32_t* nn_max);
+/* local_fusion_test.cu:229-237: rblk_lut[blocks] = {block id, row block}. */
+int sfb_build_rblk_lut(sfb_uint2* rblk_lut, const sfb_uint2* nn_lut, int nb);
+/* blocksparse.h:1016-1043 */
+void sfb_magicu64(uint32_t d, uint32_t* magic, uint32_t* shift);
+
+/* Element masks, keep[blocks][bs][bs] bytes. kind: 0 all ones; 1 diagonal blocks lower-triangular
+ * (no_fusion_test.cu:124-143); 2 local rule (local_fusion_test.cu:146-175); 3 every block
+ * lower-triangular (stride_fusion_test.cu:141-160). */
+int sfb_element_mask(uint8_t* keep, const sfb_uint2* nt_lut, uint32_t blocks, int bs, int kind,
+                     int local_attn_ctx);
+/* no_fusion_test.cu:145-157: block-major words[blk*bs + row], bit j = keep key column j.
+ * Word type follows blocksparse.h:684-720: uint32 for bs 32, uint64 for bs 64. */
+int sfb_pack_mask(void* words, const uint8_t* keep, uint32_t blocks, int bs);
+/* no_fusion_test.cu:159-163: row-major words[row*blocks + blk] for the unfused softmax. */
+int sfb_transpose_mask(void* row_major, const void* block_major, uint32_t blocks, int bs);
+
+/* MI355X addition (no reference counterpart): launch order of block-rows, longest first, ties by
+ * ascending row; row_order[nb].  Passing it to the fused entry points is optional. */
+int sfb_build_row_order(uint32_t* row_order, const sfb_uint2* nn_lut, int nb);
+
+/* ================================================================================================
+ * Device entry points
+ * ============================================================================================== */
+
+/* Fully fused attention: O = softmax_rows(scale * Q K^T restricted to layout & mask & key<valid_len) V,
+ * one work-group per (batch, head, block-row), no S/P in memory.  Replaces the sequence
+ * bst_sgemm_nt -> BlocksparseMaskedSoftmax -> bst_sgemm_xn (transformer_attention_optimize.cu:728-748)
+ * and the unfinished fusion_attention / fusion_kernel (fusion_blocksparse.h:2518-3050); arithmetic
+ * follows the CPU path (matmul.h:53-78, ewops.h:64-98, matmul.h:6-20).
+ *   q,k,v [dev]  in_dtype (SFB_F32 or SFB_BF16);  o [dev] fp32
+ *   nn_lut [dev] lut_heads * lut_dim entries, lut_dim = ctx_blks + blocks
+ *   mask [dev]   block-major words (uint32 for bs 32, uint64 for bs 64), NULL = all ones
+ *   valid_len [dev] int32[batch] keys >= valid_len[b] are masked, NULL = none (MI355X addition)
+ *   row_order [dev] uint32[ctx_blks] from sfb_build_row_order, NULL = descending row index */
+int sfb_fused_attention(sfb_stream_t stream, const void* q, const void* k, const void* v, float* o,
+                        int in_dtype, const sfb_uint2* nn_lut, const void* mask,
+                        const int32_t* valid_len, const uint32_t* row_order, uint32_t block_size,
+                        uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                        uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
+                        float scale);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SFBERT_HIP_H */

@@ -1,0 +1,47 @@
+"""Builds libsfbert_hip.so (HIP kernels for gfx950 + C ABI + host descriptors) in-tree with hipcc."""
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libsfbert_hip.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32 out of scalar float code.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature",
+                "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def sources():
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip"))) + sorted(glob.glob(os.path.join(CSRC, "*.cpp")))
+
+
+def build(verbose=True, jobs=8):
+    objs, procs = [], []
+    for src in sources():
+        obj = os.path.join(CSRC, os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmd = [HIPCC] + DEVICE_FLAGS + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+        while sum(p.poll() is None for _, p in procs) >= jobs:
+            procs[0][1].wait()
+    for src, p in procs:
+        out, _ = p.communicate()
+        text = "\n".join(l for l in out.decode().splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))
+        if verbose and text.strip():
+            print(text)
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    extra = [l for l in os.environ.get("SFB_EXTRA_LIBS", "").split() if l]
+    subprocess.check_call(link + extra)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,10 @@
+"""Loads the package (its directory name is not a Python identifier)."""
+import importlib
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+sfb = importlib.import_module("sf-bert_amd")

@@ -1,0 +1,112 @@
+"""Host descriptor builders of the library (through the C ABI) against the CPU oracle: bit-exact."""
+import ctypes as C
+import re
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from sfb import sfb, ROOT
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "sfbert_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = sorted(set(re.findall(r"\b(sfb_[a-z0-9_]+)\s*\(", header)))
+    assert declared, "no declarations found"
+    for name in declared:
+        assert hasattr(sfb.lib, name), "missing export " + name
+    assert sorted(sfb.capi.EXPORTED) == declared
+
+
+def test_status_strings():
+    assert sfb.lib.sfb_status_string(0) == b"ok"
+    assert len({sfb.lib.sfb_status_string(i) for i in range(10)}) == 10
+
+
+LAYOUT_CASES = [
+    ("full", (10, True)), ("full", (7, False)),
+    ("local", (16, 1, True)), ("local", (16, 1, False)), ("local", (9, 0, False)), ("local", (12, 3, False)),
+    ("strided_chunks", (32, 1)), ("strided_chunks", (16, 4)),
+    ("strided", (32, 4, 4, False)), ("strided", (32, 4, 4, True)), ("strided", (17, 2, 5, False)),
+]
+
+
+@pytest.mark.parametrize("name,args", LAYOUT_CASES)
+def test_layouts_bit_exact(name, args):
+    got = getattr(sfb, "layout_" + name)(*args)
+    want = getattr(orc, "layout_" + name)(*args)
+    assert got.dtype == np.uint32 and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("heads,nb,stride,causal", [(4, 10, 4, True), (1, 32, 4, False), (4, 33, 4, True),
+                                                     (3, 8, 2, False)])
+def test_fixed_layout_bit_exact(heads, nb, stride, causal):
+    assert np.array_equal(sfb.layout_fixed(heads, nb, stride, causal), orc.layout_fixed(heads, nb, stride, causal))
+
+
+@pytest.mark.parametrize("nb,window,nglobal,both,nrand,seed", [(64, 1, 2, True, 3, 1234), (10, 1, 2, False, 1, 0),
+                                                               (20, 2, 3, True, 4, 99), (6, 1, 2, True, 3, 5),
+                                                               (5, 0, 0, False, 7, 1)])
+def test_bigbird_bit_exact(nb, window, nglobal, both, nrand, seed):
+    rc = sfb.bigbird_draw(nb, window, nglobal, both, nrand, seed)
+    assert np.array_equal(rc, orc.bigbird_draw(nb, window, nglobal, both, nrand, seed))
+    assert np.array_equal(sfb.layout_bigbird(nb, window, nglobal, both, rc),
+                          orc.layout_bigbird(nb, window, nglobal, both, rc))
+    assert np.array_equal(sfb.layout_bigbird(nb, window, nglobal, both), orc.layout_bigbird(nb, window, nglobal, both))
+
+
+def _random_layouts():
+    rng = np.random.default_rng(0)
+    for nb in (1, 2, 7, 16, 64):
+        lay = (rng.random((nb, nb)) < 0.3).astype(np.uint32)
+        if nb > 3:
+            lay[3] = 0
+        yield lay
+    yield orc.layout_full(10)
+    yield orc.layout_bigbird(64, 1, 2, True, orc.bigbird_draw(64, 1, 2, True, 3, 1234))
+    yield np.zeros((4, 4), np.uint32)
+
+
+@pytest.mark.parametrize("layout", list(_random_layouts()))
+def test_luts_bit_exact(layout):
+    for init in (0, 2):
+        got, want = sfb.build_luts(layout, init), orc.build_luts(layout, init)
+        for key in ("nt_lut", "nn_lut", "rblk_lut"):
+            assert np.array_equal(got[key], want[key]), key
+        assert got["nn_max"] == want["nn_max"] and got["blocks"] == want["blocks"]
+    counts = layout.sum(axis=1)
+    order = got["row_order"]
+    assert sorted(order.tolist()) == list(range(layout.shape[0]))
+    assert all((counts[a] > counts[b]) or (counts[a] == counts[b] and a < b)
+               for a, b in zip(order[:-1], order[1:]))
+
+
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+def test_masks_bit_exact(bs, kind):
+    luts = orc.build_luts(orc.layout_local(6, 2))
+    keep = sfb.element_mask(luts["nt_lut"], bs, kind, local_attn_ctx=bs + 5)
+    assert np.array_equal(keep, orc.element_mask(luts["nt_lut"], bs, kind, local_attn_ctx=bs + 5))
+    words = sfb.pack_mask(keep)
+    assert words.dtype == (np.uint64 if bs == 64 else np.uint32)
+    assert np.array_equal(words, orc.pack_mask(keep))
+    blocks = keep.shape[0]
+    assert np.array_equal(sfb.transpose_mask(words, blocks, bs), orc.transpose_mask(words, blocks, bs))
+    rnd = (np.random.default_rng(bs + kind).random(keep.shape) < 0.5).astype(np.uint8)
+    assert np.array_equal(sfb.pack_mask(rnd), orc.pack_mask(rnd))
+
+
+def test_magicu64_bit_exact():
+    for d in list(range(1, 300)) + [1000, 4096, 65537, 2 ** 20 + 3]:
+        assert sfb.magicu64(d) == orc.magicu64(d), d
+
+
+def test_error_codes():
+    lay = np.zeros((4, 4), np.uint32)
+    assert sfb.lib.sfb_layout_full(None, 4, 1) == 1
+    assert sfb.lib.sfb_layout_full(lay.ctypes.data_as(C.c_void_p), 0, 1) == 4
+    assert sfb.lib.sfb_pack_mask(lay.ctypes.data_as(C.c_void_p), lay.ctypes.data_as(C.c_void_p), 1, 16) == 2
+    with pytest.raises(sfb.capi.SfbError):
+        sfb.layout_local(4, -1)

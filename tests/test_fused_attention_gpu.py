@@ -1,0 +1,164 @@
+"""Parity of the fused HIP attention (through the C ABI) against the CPU oracle, on the workload
+configurations and on edge cases; bit-level properties at full size."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_common import PATTERNS, TOL_BF16, TOL_F32, dev, elementwise_err, qkv, rel_err, run_fused
+from sfb import sfb
+
+pytestmark = pytest.mark.gpu
+THREADS = 16
+
+
+def check(got, want, tol):
+    err = rel_err(got, want)
+    ew = elementwise_err(got, want, floor=1e-2 * np.abs(want).max())
+    print("rel_err %.3e elementwise(floor 1%% of max) %.3e" % (err, ew), flush=True)
+    assert np.isfinite(got).all()
+    assert err <= tol, err
+    assert ew <= 10 * tol, ew
+
+
+def test_c1_local_fp32():
+    B, H, L, d, bs = 1, 12, 512, 64, 32
+    luts = sfb.build_luts(PATTERNS["local"](L // bs))
+    assert luts["blocks"] == 46
+    Q, K, V = qkv(B, L, H, d, seed=1)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    check(run_fused(Q, K, V, luts, bs, 0.125), want, TOL_F32)
+
+
+def test_c2_fixed_padding_fp32():
+    B, H, L, d, bs = 8, 12, 1024, 64, 32
+    luts = sfb.build_luts(PATTERNS["fixed"](L // bs))
+    assert luts["blocks"] == 352
+    Q, K, V = qkv(B, L, H, d, seed=2)
+    valid = orc.fill_uniform_int((B,), 22, 768, 1024)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, valid_len=valid, nthreads=THREADS)
+    check(run_fused(Q, K, V, luts, bs, 0.125, valid_len=valid), want, TOL_F32)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_c3_strided(bf16):
+    B, H, L, d, bs = 2, 12, 2048, 64, 64  # batch 2 of the configuration's 8: the oracle stays in seconds
+    luts = sfb.build_luts(PATTERNS["strided"](L // bs))
+    assert luts["blocks"] == 346
+    Q, K, V = qkv(B, L, H, d, seed=3, bf16=bf16)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    check(run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16), want, TOL_BF16 if bf16 else TOL_F32)
+
+
+@pytest.mark.parametrize("bf16", [True, False])
+def test_c4_bigbird(bf16):
+    B, H, L, d, bs = 1, 3, 4096, 64, 64  # 3 of the 48 (batch, head) pairs against the oracle
+    luts = sfb.build_luts(PATTERNS["bigbird"](L // bs))
+    assert luts["blocks"] == 622 and luts["nn_max"] == 64
+    Q, K, V = qkv(B, L, H, d, seed=4, bf16=bf16)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    check(run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16), want, TOL_BF16 if bf16 else TOL_F32)
+
+
+def test_c4_full_size_properties():
+    """B4 H12 L4096: closed form on all-ones inputs, batch/head independence, fp32 vs bf16 kernels."""
+    B, H, L, d, bs = 4, 12, 4096, 64, 64
+    lay = PATTERNS["bigbird"](L // bs)
+    luts = sfb.build_luts(lay)
+    ones = np.ones((B, L, H, d), np.float32)
+    for bf16 in (True, False):
+        O = run_fused(ones, ones, ones, luts, bs, 0.125, bf16=bf16)
+        n_keys = (lay.sum(axis=1) * bs).astype(np.float32)
+        want = np.repeat(n_keys / (n_keys + np.float32(1e-6)), bs)[None, :, None, None]
+        assert np.abs(O - want).max() <= 1e-6
+    Q, K, V = qkv(1, L, 2, d, seed=44, bf16=True)
+    tile = lambda x: np.ascontiguousarray(np.tile(x, (B, 1, H // 2, 1)))
+    Ob = run_fused(tile(Q), tile(K), tile(V), luts, bs, 0.125, bf16=True)
+    assert np.array_equal(Ob, np.tile(Ob[:1, :, :2], (B, 1, H // 2, 1)))  # every (b,h) copy identical
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    check(Ob[:1, :, :2], want, TOL_BF16)
+    Of = run_fused(tile(Q), tile(K), tile(V), luts, bs, 0.125, bf16=False)
+    check(Of[:1, :, :2], want, TOL_F32)
+
+
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("pattern", ["causal", "local_causal", "bigbird", "full"])
+def test_masks_and_padding(pattern, bs, bf16):
+    nb, B, H, d = 8, 3, 2, 64
+    L = nb * bs
+    luts = sfb.build_luts(PATTERNS[pattern](nb))
+    kind = {"causal": sfb.MASK_CAUSAL_DIAG, "local_causal": sfb.MASK_LOCAL}.get(pattern, sfb.MASK_ALL)
+    mask = sfb.pack_mask(sfb.element_mask(luts["nt_lut"], bs, kind, local_attn_ctx=bs)) if kind else None
+    if pattern == "full":  # a random element mask, so every bit position is exercised
+        keep = (np.random.default_rng(bs).random((luts["blocks"], bs, bs)) < 0.7).astype(np.uint8)
+        mask = sfb.pack_mask(keep)
+    valid = np.array([L, L - bs - 7, 5], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=50 + bs, bf16=bf16)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, mask=mask, valid_len=valid, nthreads=THREADS)
+    got = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, mask=mask, valid_len=valid)
+    check(got, want, TOL_BF16 if bf16 else TOL_F32)
+    # same result without the launch-order table
+    got2 = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, mask=mask, valid_len=valid, use_order=False)
+    assert np.array_equal(got, got2)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_empty_rows_and_fully_masked_rows(bf16):
+    bs, nb, B, H, d = 32, 6, 2, 3, 64
+    L = bs * nb
+    lay = PATTERNS["local"](nb).copy()
+    lay[2] = 0
+    luts = sfb.build_luts(lay)
+    Q, K, V = qkv(B, L, H, d, seed=70, bf16=bf16)
+    valid = np.array([L, 0], np.int32)
+    got = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, valid_len=valid)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, valid_len=valid)
+    assert (got[:, 2 * bs:3 * bs] == 0).all() and (got[1] == 0).all()
+    check(got, want, TOL_BF16 if bf16 else TOL_F32)
+
+
+def test_per_head_luts_and_masks():
+    bs, nb, B, H, d = 32, 8, 2, 4, 64
+    L = bs * nb
+    lay = sfb.layout_fixed(H, nb, 4, causal=True)
+    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
+    blocks = per_head[0]["blocks"]
+    assert all(p["blocks"] == blocks for p in per_head)
+    nn = np.concatenate([p["nn_lut"] for p in per_head])
+    masks = np.concatenate([sfb.pack_mask(sfb.element_mask(p["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG))
+                            for p in per_head])
+    Q, K, V = qkv(B, L, H, d, seed=80)
+    want = orc.attention(Q, K, V, nn, bs, 0.125, mask=masks, lut_heads=H, mask_heads=H, blocks=blocks)
+    got = run_fused(Q, K, V, per_head[0], bs, 0.125, mask=masks, lut_heads=H, mask_heads=H, nn_lut=nn,
+                    blocks=blocks, use_order=False)
+    check(got, want, TOL_F32)
+
+
+def test_scale_and_large_scores():
+    # scores far from zero: the running maximum and the 1e-6 term must still follow the oracle
+    bs, nb, B, H, d = 64, 4, 1, 2, 64
+    L = bs * nb
+    luts = sfb.build_luts(PATTERNS["full"](nb))
+    Q, K, V = qkv(B, L, H, d, seed=90)
+    Q *= 6.0
+    for scale in (0.125, 1.0, 0.01):
+        want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale)
+        check(run_fused(Q, K, V, luts, bs, scale), want, TOL_F32)
+
+
+def test_argument_errors():
+    q = torch.zeros((1, 64, 1, 64), device="cuda")
+    lut = sfb.to_device(np.zeros((3, 2), np.uint32))
+    call = lambda **kw: sfb.lib.sfb_fused_attention(
+        None, kw.get("q", C.c_void_p(q.data_ptr())), C.c_void_p(q.data_ptr()), C.c_void_p(q.data_ptr()),
+        C.c_void_p(q.data_ptr()), kw.get("dtype", 0), C.c_void_p(lut.data_ptr()), None, None, None,
+        C.c_uint32(kw.get("bs", 64)), C.c_uint32(1), C.c_uint32(1), C.c_uint32(1), C.c_uint32(1),
+        C.c_uint32(kw.get("d", 64)), C.c_uint32(1), C.c_uint32(2), C.c_uint32(1), C.c_float(0.125))
+    assert call(q=None) == 1
+    assert call(bs=16) == 2
+    assert call(d=48) == 3
+    assert call(dtype=7) == 5
+    assert call(q=C.c_void_p(q.data_ptr() + 4)) == 6
