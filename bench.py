@@ -1,0 +1,147 @@
+"""Benchmark of the fused block-sparse attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c3|c2|c1] [--dtype bf16|f32]
+
+One step = one fused attention call over the whole batch of the workload (default: the BigBird
+configuration B4 H12 L4096 d64 block 64, bf16 inputs, fp32 accumulation and output).  Inputs are
+synthetic N(0,1) tensors already resident in HBM when the timed region starts.  Prints ONE JSON line:
+metric/value = effective TFLOP/s over the nonzero blocks (nnz*B*H*4*bs^2*d flops per call), plus
+`roofline` (MFMA bound, measured with HIP events on the launch stream) and `cpu_baseline` (the CPU
+oracle timed on this host's cores on a bounded sample of the same workload).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (pattern, B, H, L, d, bs, default dtype)
+    "c1": ("local", 1, 12, 512, 64, 32, "f32"),
+    "c2": ("fixed", 8, 12, 1024, 64, 32, "f32"),
+    "c3": ("strided", 8, 12, 2048, 64, 64, "bf16"),
+    "c4": ("bigbird", 4, 12, 4096, 64, 64, "bf16"),
+}
+
+
+def make_layout(sfb, pattern, nb):
+    if pattern == "local":
+        return sfb.layout_local(nb, 1, bidirectional=True)
+    if pattern == "fixed":
+        return sfb.layout_fixed(1, nb, 4, causal=False)[0]
+    if pattern == "strided":
+        return sfb.layout_strided(nb, 4, 4)
+    return sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234))
+
+
+def cpu_baseline(luts, B, H, L, d, bs, bf16, flops_per_bh):
+    """Times the CPU oracle (a port of the reference CPU path) on one batch element of the workload."""
+    import numpy as np
+    import oracle_lib as orc
+    threads = max(1, min(16, os.cpu_count() or 1))
+    sample_b = 1
+    Q, K, V = (orc.fill_normal((sample_b, L, H, d), 900 + i) for i in range(3))
+    if bf16:
+        Q, K, V = (orc.round_bf16(x) for x in (Q, K, V))
+    t0 = time.perf_counter()
+    orc.attention(Q, K, V, luts["nn_lut"], bs, 1.0 / np.sqrt(d), nthreads=threads)
+    dt = time.perf_counter() - t0
+    tflops = flops_per_bh * sample_b * H / dt / 1e12
+    return {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "CPU oracle (fp32 port of matmul.h/ewops.h loops, OpenMP over block-rows) on "
+                      "batch 1 of %d of the same workload: %.2f s, scaled by flops" % (B, dt),
+            "seconds": dt, "ms_per_call_extrapolated": dt * B * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--dtype", default=None, choices=["bf16", "f32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the path shards over (batch, head) with no exchange and "
+              "this build has no multi-GPU leg; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    sfb = importlib.import_module("sf-bert_amd")
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(1)
+
+    pattern, B, H, L, d, bs, default_dtype = WORKLOADS[args.workload]
+    dtype = args.dtype or default_dtype
+    bf16 = dtype == "bf16"
+    nb = L // bs
+    luts = sfb.build_luts(make_layout(sfb, pattern, nb))
+    blocks = luts["blocks"]
+    flops_per_bh = blocks * 4.0 * bs * bs * d
+    flops = flops_per_bh * B * H
+    elem = 2 if bf16 else 4
+    algo_bytes = B * L * H * d * (3 * elem + 4)
+
+    torch.manual_seed(0)
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    q, k, v = (torch.randn((B, L, H, d), device="cuda", dtype=torch.float32).to(tdt) for _ in range(3))
+    out = torch.empty((B, L, H, d), device="cuda", dtype=torch.float32)
+    nn_lut = sfb.to_device(luts["nn_lut"])
+    order = sfb.to_device(luts["row_order"])
+    scale = 1.0 / (d ** 0.5)
+
+    def step():
+        sfb.fused_attention(q, k, v, nn_lut, bs, blocks, scale, row_order=order, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    kernel_ms = start.elapsed_time(stop) / args.steps   # HIP events on the launch stream
+    ms_per_step = wall_ms / args.steps
+    assert torch.isfinite(out).all()
+
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dtype]
+    result = {
+        "metric": "fused block-sparse attn effective TFLOP/s + ms/layer at L=4096, 1 MI355X",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": "%s: %s block-sparse attention B%d H%d L%d d%d block %d, %d nonzero "
+                               "blocks, %s inputs, fp32 accumulate/output" %
+                               (args.workload, pattern, B, H, L, d, bs, blocks, dtype)},
+        "ms_per_attention_call": kernel_ms,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+                     "frac": achieved / peak, "traffic": None,
+                     "kernel": "fused_attention_%s_kernel<%d,%d>" % (dtype if bf16 else "f32", bs, d),
+                     "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms,
+                     "hbm_algorithmic_bytes_per_launch": algo_bytes,
+                     "hbm_achieved_GBs": algo_bytes / (kernel_ms * 1e-3) / 1e9,
+                     "hbm_frac": algo_bytes / (kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops_per_bh)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libsfbert_hip.so")
+# SFBERT_HIP_LIB points at an alternative build of the same library (e.g. an experimental kernel variant)
+LIB_PATH = os.environ.get("SFBERT_HIP_LIB") or os.path.join(_HERE, "libsfbert_hip.so")
 
 F32, BF16 = 0, 1
 NT_OP, NN_OP, TN_OP = 0, 1, 2

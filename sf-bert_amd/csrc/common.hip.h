@@ -22,6 +22,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kMaxSeed = -1000000.0f;
 // Score given to a masked key: far below any real score, finite so that (s - max) never makes NaN.
 constexpr float kMaskedScore = -3.0e38f;
+// Probabilities are kept relative to a reference maximum that may lag the true one by this many
+// powers of two before the accumulators are rescaled.
+constexpr float kLazyRescaleLog2 = 8.0f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -29,6 +32,12 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     f32x2 f = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// acc + lo(pair) + hi(pair) for a packed bf16 pair (v_dot2c_f32_bf16 against packed ones).
+__device__ __forceinline__ float dot2_bf16_ones(uint32_t pair, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair),
+                                           __builtin_bit_cast(bf16x2, 0x3f803f80u), acc, false);
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {

@@ -33,6 +33,7 @@ struct FusedParams {
     uint32_t mask_stride;  // words between heads' masks (0 = shared)
     uint32_t groups;       // ceil(batch*heads / 8)
     float scale_log2e;
+    float slack;           // raw-score distance a block maximum may exceed the reference maximum
 };
 
 // Keep-bits of one lane's query row for one key block, with key padding folded in.
@@ -49,11 +50,25 @@ __device__ __forceinline__ uint64_t load_keep_word(const void* mask, size_t word
 
 // Online-softmax step on one key block.  s[kt][i] holds, for this lane's query, the raw score of key
 //   kt*32 + (i/4)*8 + half*4 + i%4      (half = lane / 32)
-// and is overwritten by the unnormalised probability.  m, l: running maximum (raw units) and this
-// lane's partial row sum; o: output accumulators, rescaled when the maximum moves.
-template <int KT, int NO>
-__device__ __forceinline__ void softmax_block(f32x16 (&s)[KT], f32x16 (&o)[NO], float& m, float& l,
-                                              float c, bool masked, uint64_t keep, uint32_t half) {
+// and is overwritten by the unnormalised probability (PACK: pk[kt*8 + i/2] receives the pair
+// (i, i+1) rounded to bf16, and the row sum is taken over those rounded values, i.e. over exactly
+// what the P.V product uses).
+//
+// The probabilities are taken relative to a reference maximum m_used that is only moved when a
+// block's maximum exceeds it by more than `slack` (raw-score units; 2^8 in probability), so the
+// rescaling of the output accumulators is rare.  m_true tracks the exact running maximum; the final
+// normalisation uses both, which keeps the result identical to softmax relative to the true maximum
+// including the +1e-6 term of the denominator.
+struct RowState {
+    float m_used;   // reference maximum the stored probabilities are relative to (raw units)
+    float m_true;   // exact running maximum over kept keys, seeded like the CPU path
+    float l;        // this lane's partial sum of probabilities relative to m_used
+};
+
+template <int KT, int NO, bool PACK>
+__device__ __forceinline__ void softmax_block(f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], f32x16 (&o)[NO],
+                                              RowState& st, float c, float slack, bool masked,
+                                              uint64_t keep, uint32_t half) {
     if (masked) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -65,40 +80,61 @@ __device__ __forceinline__ void softmax_block(f32x16 (&s)[KT], f32x16 (&o)[NO], 
             }
         }
     }
-    float mloc = s[0][0];
+    float mx0 = s[0][0], mx1 = s[0][1];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) mloc = fmaxf(fmaxf(mloc, s[kt][i]), s[kt][i + 1]);
+        for (int i = 0; i < 16; i += 4) {
+            mx0 = fmaxf(fmaxf(mx0, s[kt][i]), s[kt][i + 1]);
+            mx1 = fmaxf(fmaxf(mx1, s[kt][i + 2]), s[kt][i + 3]);
+        }
     }
+    float mloc = fmaxf(mx0, mx1);
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-    const float m_new = fmaxf(m, mloc);
-    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
-        const float alpha = exp2_fast((m - m_new) * c);
-        l *= alpha;
+    st.m_true = fmaxf(st.m_true, mloc);
+    if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
+        const float m_new = fmaxf(st.m_used, mloc);
+        const float alpha = exp2_fast((st.m_used - m_new) * c);
+        st.m_used = m_new;
+        st.l *= alpha;
 #pragma unroll
         for (int n = 0; n < NO; ++n) o[n] *= alpha;
     }
-    m = m_new;
-    const float mc = m_new * c;
-    float sum = 0.f;
+    const float mc = st.m_used * c;
+    float sum0 = 0.f, sum1 = 0.f;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float p = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc));
-            s[kt][i] = p;
-            sum += p;
+        for (int i = 0; i < 16; i += 4) {
+            const float p0 = exp2_fast(__builtin_fmaf(s[kt][i + 0], c, -mc));
+            const float p1 = exp2_fast(__builtin_fmaf(s[kt][i + 1], c, -mc));
+            const float p2 = exp2_fast(__builtin_fmaf(s[kt][i + 2], c, -mc));
+            const float p3 = exp2_fast(__builtin_fmaf(s[kt][i + 3], c, -mc));
+            if (PACK) {
+                const uint32_t a = pack_bf16(p0, p1), b = pack_bf16(p2, p3);
+                pk[kt * 8 + i / 2] = a;
+                pk[kt * 8 + i / 2 + 1] = b;
+                sum0 = dot2_bf16_ones(a, sum0);
+                sum1 = dot2_bf16_ones(b, sum1);
+            } else {
+                s[kt][i + 0] = p0; s[kt][i + 1] = p1; s[kt][i + 2] = p2; s[kt][i + 3] = p3;
+                sum0 += p0 + p1;
+                sum1 += p2 + p3;
+            }
         }
     }
-    l += sum;
+    st.l += sum0 + sum1;
 }
 
 // Normalise and store this lane's part of O: o[mt][i] is output column mt*32 + (i/4)*8 + half*4 + i%4.
 template <int NO>
-__device__ __forceinline__ void store_output(float* o_row, f32x16 (&o)[NO], float l, uint32_t half) {
-    const float total = l + __shfl_xor(l, 32);
-    const float inv = 1.0f / (total + 1e-6f);
+__device__ __forceinline__ void store_output(float* o_row, f32x16 (&o)[NO], const RowState& st, float c,
+                                             uint32_t half) {
+    // sum relative to the true maximum = total / f with f = 2^((m_true - m_used) c); hence
+    // O = acc / (total + 1e-6 f)  (ewops.h:93 divides by sum + 1e-6).
+    const float total = st.l + __shfl_xor(st.l, 32);
+    const float f = exp2_fast((st.m_true - st.m_used) * c);
+    const float inv = 1.0f / (total + 1e-6f * f);
 #pragma unroll
     for (int mt = 0; mt < NO; ++mt) {
 #pragma unroll
@@ -120,7 +156,7 @@ __device__ __forceinline__ void store_output(float* o_row, f32x16 (&o)[NO], floa
 // Two buffers, one barrier per key block: block j+1 is fetched into registers while block j is
 // multiplied, written to the other buffer afterwards.
 template <int BS, int D>
-__global__ __launch_bounds__(BS * 2) void fused_attention_bf16_kernel(FusedParams p) {
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
     constexpr int NT = BS * 2;
     constexpr int KT = BS / 32;      // 32-key tiles per block
     constexpr int NO = D / 32;       // 32-column tiles of O
@@ -228,8 +264,8 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_bf16_kernel(FusedParam
     for (int n = 0; n < NO; ++n)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
-    float m_run = kMaxSeed, l_run = 0.f;
-    const float c = p.scale_log2e;
+    RowState st = {kMaxSeed, kMaxSeed, 0.f};
+    const float c = p.scale_log2e, slack = p.slack;
 
     sfb_uint2 entry = lut[lut_off];
     fetch(entry.y);
@@ -264,17 +300,13 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_bf16_kernel(FusedParam
         const bool masked = (mask != nullptr) || (limit < BS);
         uint64_t keep = ~0ull;
         if (masked) keep = load_keep_word<BS>(mask, (size_t)here.x * BS + wave * 32 + qn, limit);
-        softmax_block<KT, NO>(s, o_acc, m_run, l_run, c, masked, keep, half);
+        uint32_t pk[KT * 8];
+        softmax_block<KT, NO, true>(s, pk, o_acc, st, c, slack, masked, keep, half);
 
         // O^T += V^T . P^T
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
-            const int kt = u / 2, i0 = (u % 2) * 8;
-            u32x4 pb;
-            pb.x = pack_bf16(s[kt][i0 + 0], s[kt][i0 + 1]);
-            pb.y = pack_bf16(s[kt][i0 + 2], s[kt][i0 + 3]);
-            pb.z = pack_bf16(s[kt][i0 + 4], s[kt][i0 + 5]);
-            pb.w = pack_bf16(s[kt][i0 + 6], s[kt][i0 + 7]);
+            const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
             const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
             for (int mt = 0; mt < NO; ++mt) {
@@ -287,7 +319,7 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_bf16_kernel(FusedParam
         __syncthreads();
     }
 
-    store_output<NO>(o_row, o_acc, l_run, half);
+    store_output<NO>(o_row, o_acc, st, c, half);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -300,7 +332,7 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_bf16_kernel(FusedParam
 // fp32: MFMA step (kt, i) consumes key kt*32 + (i/4)*8 + half*4 + i%4, whose V row is read as 32
 // consecutive floats.
 template <int BS, int D>
-__global__ __launch_bounds__(BS * 2) void fused_attention_f32_kernel(FusedParams p) {
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedParams p) {
     constexpr int NT = BS * 2;
     constexpr int KT = BS / 32;
     constexpr int NO = D / 32;
@@ -371,8 +403,8 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_f32_kernel(FusedParams
     for (int n = 0; n < NO; ++n)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
-    float m_run = kMaxSeed, l_run = 0.f;
-    const float c = p.scale_log2e;
+    RowState st = {kMaxSeed, kMaxSeed, 0.f};
+    const float c = p.scale_log2e, slack = p.slack;
 
     sfb_uint2 entry = lut[lut_off];
     fetch(entry.y);
@@ -404,7 +436,8 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_f32_kernel(FusedParams
         const bool masked = (mask != nullptr) || (limit < BS);
         uint64_t keep = ~0ull;
         if (masked) keep = load_keep_word<BS>(mask, (size_t)here.x * BS + wave * 32 + qn, limit);
-        softmax_block<KT, NO>(s, o_acc, m_run, l_run, c, masked, keep, half);
+        uint32_t pk_unused[KT * 8];
+        softmax_block<KT, NO, false>(s, pk_unused, o_acc, st, c, slack, masked, keep, half);
 
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -421,7 +454,7 @@ __global__ __launch_bounds__(BS * 2) void fused_attention_f32_kernel(FusedParams
         __syncthreads();
     }
 
-    store_output<NO>(o_row, o_acc, l_run, half);
+    store_output<NO>(o_row, o_acc, st, c, half);
 }
 
 template <int BS, int D>
@@ -448,6 +481,7 @@ extern "C" int sfb_fused_attention(sfb_stream_t stream, const void* q, const voi
     if (in_dtype != SFB_F32 && in_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (batch_dim == 0 || ctx_blks == 0 || head_dim == 0 || lut_heads == 0 || mask_heads == 0)
         return SFB_ERR_SHAPE;
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
@@ -464,6 +498,7 @@ extern "C" int sfb_fused_attention(sfb_stream_t stream, const void* q, const voi
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
     p.groups = bh_groups(batch_dim * head_dim);
     p.scale_log2e = scale * kLog2e;
+    p.slack = kLazyRescaleLog2 / p.scale_log2e;
     hipStream_t s = (hipStream_t)stream;
     if (block_size == 64) return launch_fused<64, 64>(s, p, in_dtype);
     return launch_fused<32, 64>(s, p, in_dtype);
