@@ -69,6 +69,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["bf16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--max-blocks", type=int, default=16,
+                    help="split block-rows longer than this many key blocks (0 = one work-group per row)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path shards over (batch, head) with no exchange and "
@@ -100,8 +102,17 @@ def main():
     order = sfb.to_device(luts["row_order"])
     scale = 1.0 / (d ** 0.5)
 
-    def step():
-        sfb.fused_attention(q, k, v, nn_lut, bs, blocks, scale, row_order=order, out=out)
+    if args.max_blocks > 0:
+        sched = sfb.build_schedule(luts["nn_lut"], nb, args.max_blocks)
+        items = sfb.to_device(sched["items"])
+        workspace = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256),
+                                dtype=torch.uint8, device="cuda")
+
+        def step():
+            sfb.fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, bs, blocks, scale, out=out)
+    else:
+        def step():
+            sfb.fused_attention(q, k, v, nn_lut, bs, blocks, scale, row_order=order, out=out)
 
     for _ in range(args.warmup):
         step()

@@ -13,6 +13,7 @@
 #ifndef SFBERT_HIP_H
 #define SFBERT_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -98,6 +99,29 @@ int sfb_transpose_mask(void* row_major, const void* block_major, uint32_t blocks
  * ascending row; row_order[nb].  Passing it to the fused entry points is optional. */
 int sfb_build_row_order(uint32_t* row_order, const sfb_uint2* nn_lut, int nb);
 
+/* MI355X addition (no reference counterpart): work items of a scheduled fused launch.  Block-rows
+ * with more than max_blocks key blocks (BigBird's global rows) are cut into ceil(count/max_blocks)
+ * chunks of near-equal length so that no work-group walks a long row alone; the chunks' partial
+ * results are merged by whichever chunk finishes last.  Items are sorted longest first. */
+typedef struct {
+    uint32_t row;      /* query block row */
+    uint32_t first;    /* first key block of this item, relative to the row's NN-LUT segment */
+    uint32_t count;    /* number of key blocks of this item */
+    uint32_t nchunks;  /* chunks the row was cut into (1 = whole row) */
+    uint32_t chunk;    /* index of this chunk within the row */
+    uint32_t slot;     /* index of the row among split rows (arrival counter), 0 if not split */
+    uint32_t part;     /* index of the row's first partial-result record, 0 if not split */
+    uint32_t reserved;
+} sfb_work_item;
+/* items may be NULL to query the counts; otherwise it must hold *n_items entries as returned by a
+ * query call.  n_slots = number of split rows, n_parts = total chunks of split rows. */
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_slots, uint32_t* n_parts,
+                       const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
+/* Bytes of the [dev] workspace a scheduled launch needs: arrival counters + partial records.  The
+ * workspace must be zero-filled once before its first use; launches leave the counters at zero. */
+size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
+                                    uint32_t head_dim, uint32_t block_size, uint32_t state_dim);
+
 /* ================================================================================================
  * Device entry points
  * ============================================================================================== */
@@ -118,6 +142,19 @@ int sfb_fused_attention(sfb_stream_t stream, const void* q, const void* k, const
                         uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
                         uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
                         float scale);
+
+/* The same operation launched over sfb_build_schedule's work items (one layout shared by all heads).
+ *   items [dev] n_items entries;  workspace [dev] 256-byte aligned, sfb_schedule_workspace_bytes()
+ *   bytes, zero-filled before first use (may be NULL when n_parts == 0).  Launches that share a
+ *   workspace must be ordered on one stream. */
+int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k, const void* v,
+                                  float* o, int in_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                  const int32_t* valid_len, const sfb_work_item* items,
+                                  uint32_t n_items, uint32_t n_slots, uint32_t n_parts,
+                                  void* workspace, size_t workspace_bytes, uint32_t block_size,
+                                  uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                  uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
+                                  float scale);
 
 #ifdef __cplusplus
 }

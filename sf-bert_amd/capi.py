@@ -39,6 +39,7 @@ lib.sfb_status_string.restype = C.c_char_p
 lib.sfb_status_string.argtypes = [C.c_int]
 lib.sfb_count_blocks.restype = C.c_uint32
 lib.sfb_magicu64.restype = None
+lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -47,7 +48,8 @@ EXPORTED = [
     "sfb_layout_strided", "sfb_layout_bigbird", "sfb_bigbird_draw", "sfb_count_blocks",
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
-    "sfb_fused_attention",
+    "sfb_build_schedule", "sfb_schedule_workspace_bytes",
+    "sfb_fused_attention", "sfb_fused_attention_scheduled",
 ]
 
 
@@ -163,6 +165,29 @@ def transpose_mask(words, blocks, bs):
     return out
 
 
+WORK_ITEM_DTYPE = np.dtype([(n, np.uint32) for n in
+                            ("row", "first", "count", "nchunks", "chunk", "slot", "part", "reserved")])
+
+
+def build_schedule(nn_lut, nb, max_blocks=16):
+    """Work items of a scheduled fused launch: dict(items structured array, n_slots, n_parts)."""
+    nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
+    n_items, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    _check(lib.sfb_build_schedule(None, C.byref(n_items), C.byref(n_slots), C.byref(n_parts),
+                                  _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
+    items = np.zeros(n_items.value, WORK_ITEM_DTYPE)
+    _check(lib.sfb_build_schedule(_np(items), C.byref(n_items), C.byref(n_slots), C.byref(n_parts),
+                                  _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
+    return Luts(items=items, n_items=int(n_items.value), n_slots=int(n_slots.value),
+                n_parts=int(n_parts.value))
+
+
+def schedule_workspace_bytes(sched, batch, heads, block_size, d):
+    return int(lib.sfb_schedule_workspace_bytes(C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]),
+                                                C.c_uint32(batch), C.c_uint32(heads),
+                                                C.c_uint32(block_size), C.c_uint32(d)))
+
+
 def magicu64(d):
     m, s = C.c_uint32(0), C.c_uint32(0)
     lib.sfb_magicu64(C.c_uint32(d), C.byref(m), C.byref(s))
@@ -209,4 +234,26 @@ def fused_attention(q, k, v, nn_lut, block_size, blocks, scale, mask=None, valid
                                    C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d), C.c_uint32(lut_heads),
                                    C.c_uint32(nb + blocks), C.c_uint32(mask_heads), C.c_float(scale)),
            "sfb_fused_attention")
+    return out
+
+
+def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_size, blocks, scale,
+                              mask=None, valid_len=None, mask_heads=1, out=None):
+    """fused_attention over sfb_build_schedule's work items; `items` and `workspace` are device buffers
+    (workspace: zero-filled uint8 tensor of schedule_workspace_bytes(), or None if nothing is split)."""
+    import torch
+    B, L, H, d = q.shape
+    if out is None:
+        out = torch.empty((B, L, H, d), dtype=torch.float32, device=q.device)
+    nb = L // block_size
+    for t in (q, k, v, out):
+        if not t.is_contiguous():
+            raise SfbError(4, "non-contiguous tensor")
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(lib.sfb_fused_attention_scheduled(
+        _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dtype_code(q), _dev(nn_lut), _dev(mask),
+        _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_slots"]),
+        C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes), C.c_uint32(block_size),
+        C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d),
+        C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled")
     return out

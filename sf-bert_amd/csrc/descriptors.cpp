@@ -285,4 +285,40 @@ int sfb_build_row_order(uint32_t* row_order, const sfb_uint2* nn_lut, int nb) {
     return SFB_OK;
 }
 
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_slots, uint32_t* n_parts,
+                       const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
+    if (!n_items || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
+    if (nb <= 0) return SFB_ERR_SHAPE;
+    if (max_blocks == 0) return SFB_ERR_ARGUMENT;
+    std::vector<sfb_work_item> all;
+    uint32_t slots = 0, parts = 0;
+    for (int r = 0; r < nb; ++r) {
+        const uint32_t count = nn_lut[r].y;
+        const uint32_t chunks = count > max_blocks ? (count + max_blocks - 1) / max_blocks : 1;
+        if (chunks == 1) {
+            all.push_back(sfb_work_item{(uint32_t)r, 0u, count, 1u, 0u, 0u, 0u, 0u});
+            continue;
+        }
+        const uint32_t base = count / chunks, extra = count % chunks;
+        uint32_t first = 0;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const uint32_t len = base + (c < extra ? 1u : 0u);
+            all.push_back(sfb_work_item{(uint32_t)r, first, len, chunks, c, slots, parts, 0u});
+            first += len;
+        }
+        ++slots;
+        parts += chunks;
+    }
+    std::stable_sort(all.begin(), all.end(),
+                     [](const sfb_work_item& a, const sfb_work_item& b) { return a.count > b.count; });
+    if (items) {
+        if (*n_items < all.size()) return SFB_ERR_ARGUMENT;
+        std::copy(all.begin(), all.end(), items);
+    }
+    *n_items = (uint32_t)all.size();
+    *n_slots = slots;
+    *n_parts = parts;
+    return SFB_OK;
+}
+
 }  // extern "C"

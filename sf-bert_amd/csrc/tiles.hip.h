@@ -1,0 +1,197 @@
+// LDS tile staging and MFMA fragment access shared by the attention kernels.
+//
+// A work-group of NT = 2*BS threads (BS/32 waves, each owning 32 query rows) walks key blocks of BS
+// keys.  Lane l of a wave is query column qn = l % 32 and half = l / 32 of the 32x32 MFMA shapes.
+//
+// Score tile, transposed:  S^T[key][query] = sum_k K[key][k] Q[query][k]      (A = K, B = Q^T)
+//   accumulator element i of key tile kt is key  kt*32 + (i/4)*8 + half*4 + i%4  of query qn.
+// Output tile, transposed: O^T[col][query] += sum_key V[key][col] P[query][key] (A = V^T, B = P^T)
+//   accumulator element i of column tile mt is column  mt*32 + (i/4)*8 + half*4 + i%4.
+// Because both accumulators keep one query per lane, the softmax is lane-local and P feeds the
+// second product without leaving its registers.
+#pragma once
+
+#include "common.hip.h"
+
+namespace sfb {
+
+// ------------------------------------------------------------------------------------------------
+// bf16 operands, v_mfma_f32_32x32x16_bf16 (8 bf16 per lane per step: k-slots half*8 .. half*8+7)
+// ------------------------------------------------------------------------------------------------
+// K tile in LDS: [BS keys][D + 8] bf16 row-major; the 16-byte pad makes the 128-bit fragment reads
+//   conflict-free.  Score k-slot (ks, half, j) is head-dimension index (2ks + half)*8 + j.
+// V tile in LDS: transposed, [D][BS + 8] bf16, and inside a row the 4-key groups are stored in the
+//   order the P^T operand holds them: product step u, half hf, slot j is key 16u + 8(j/4) + 4hf + j%4,
+//   i.e. group g = 4u + 2a + hf (a = j/4) lives at byte (2u + hf)*16 + a*8.
+template <int BS, int D>
+struct Bf16Tiles {
+    static constexpr int NT = BS * 2;
+    static constexpr int K_STRIDE = (D + 8) * 2;   // bytes
+    static constexpr int V_STRIDE = (BS + 8) * 2;  // bytes
+    static constexpr int K_BYTES = BS * K_STRIDE;
+    static constexpr int V_BYTES = D * V_STRIDE;
+    static constexpr int K_CHUNKS = D / 16;         // 16-byte chunks of K per thread
+    static constexpr int V_ITEMS = D / 64;          // (4 keys x 8 columns) items of V per thread
+    static_assert(D % 64 == 0, "head state must be a multiple of 64");
+
+    struct KRegs { u32x4 g[K_CHUNKS]; };
+    struct VRegs { u32x4 g[V_ITEMS][4]; };
+
+    // base: element offset of (b, first token of the key block, h, 0); row_stride = heads * D.
+    static __device__ __forceinline__ void fetch_k(KRegs& r, const __bf16* K, size_t base,
+                                                   uint32_t row_stride, uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < K_CHUNKS; ++i) {
+            const uint32_t cid = i * NT + t, row = cid / (D / 8), c = cid % (D / 8);
+            r.g[i] = *(const u32x4*)(K + base + (size_t)(row * row_stride + c * 8));
+        }
+    }
+    static __device__ __forceinline__ void stage_k(uint8_t* k_lds, const KRegs& r, uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < K_CHUNKS; ++i) {
+            const uint32_t cid = i * NT + t, row = cid / (D / 8), c = cid % (D / 8);
+            *(u32x4*)(k_lds + row * K_STRIDE + c * 16) = r.g[i];
+        }
+    }
+    static __device__ __forceinline__ void fetch_v(VRegs& r, const __bf16* V, size_t base,
+                                                   uint32_t row_stride, uint32_t t) {
+#pragma unroll
+        for (int ii = 0; ii < V_ITEMS; ++ii) {
+            const uint32_t id = ii * NT + t, g = id % (BS / 4), c = id / (BS / 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                r.g[ii][e] = *(const u32x4*)(V + base + (size_t)((4 * g + e) * row_stride + c * 8));
+        }
+    }
+    // 4 keys x 8 columns per item -> 8 (column, 4-key group) pairs of 8 bytes.
+    static __device__ __forceinline__ void stage_v(uint8_t* v_lds, const VRegs& r, uint32_t t) {
+#pragma unroll
+        for (int ii = 0; ii < V_ITEMS; ++ii) {
+            const uint32_t id = ii * NT + t, g = id % (BS / 4), c = id / (BS / 4);
+            const uint32_t pos = (2 * (g / 4) + (g & 1)) * 16 + ((g & 3) >> 1) * 8;
+#pragma unroll
+            for (int dd = 0; dd < 8; ++dd) {
+                const uint32_t x0 = r.g[ii][0][dd / 2], x1 = r.g[ii][1][dd / 2];
+                const uint32_t x2 = r.g[ii][2][dd / 2], x3 = r.g[ii][3][dd / 2];
+                u32x2 out;
+                if (dd & 1) {
+                    out.x = (x0 >> 16) | (x1 & 0xffff0000u);
+                    out.y = (x2 >> 16) | (x3 & 0xffff0000u);
+                } else {
+                    out.x = (x0 & 0xffffu) | (x1 << 16);
+                    out.y = (x2 & 0xffffu) | (x3 << 16);
+                }
+                *(u32x2*)(v_lds + (c * 8 + dd) * V_STRIDE + pos) = out;
+            }
+        }
+    }
+    static __device__ __forceinline__ bf16x8 k_frag(const uint8_t* k_lds, int kt, int ks, uint32_t qn,
+                                                    uint32_t half) {
+        return *(const bf16x8*)(k_lds + (kt * 32 + qn) * K_STRIDE + (2 * ks + half) * 16);
+    }
+    static __device__ __forceinline__ bf16x8 v_frag(const uint8_t* v_lds, int mt, int u, uint32_t qn,
+                                                    uint32_t half) {
+        return *(const bf16x8*)(v_lds + (mt * 32 + qn) * V_STRIDE + (2 * u + half) * 16);
+    }
+    // Q^T operand of one query row, kept in registers: D/16 steps of 8 bf16.
+    static __device__ __forceinline__ void load_q(bf16x8 (&qf)[D / 16], const __bf16* q_row,
+                                                  uint32_t half) {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) qf[ks] = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// fp32 operands, v_mfma_f32_32x32x2_f32 (one float per lane per step: k-slot = half)
+// ------------------------------------------------------------------------------------------------
+// K tile in LDS: [BS][D + 4] floats; score k-slot (step, half) is head-dimension index
+//   8*(step/4) + 4*half + step%4, so one 128-bit read feeds four steps.
+// V tile in LDS: [BS][D + 8] floats, row-major (no transposition needed: product step (kt, i)
+//   consumes key kt*32 + (i/4)*8 + half*4 + i%4 and reads 32 consecutive floats of that row).
+template <int BS, int D>
+struct F32Tiles {
+    static constexpr int NT = BS * 2;
+    static constexpr int K_STRIDE = D + 4;  // floats
+    static constexpr int V_STRIDE = D + 8;  // floats
+    static constexpr int K_FLOATS = BS * K_STRIDE;
+    static constexpr int V_FLOATS = BS * V_STRIDE;
+    static constexpr int CHUNKS = D / 8;    // float4 chunks per thread per tile
+    static_assert(D % 32 == 0, "head state must be a multiple of 32");
+
+    struct Regs { f32x4 g[CHUNKS]; };
+
+    static __device__ __forceinline__ void fetch(Regs& r, const float* X, size_t base,
+                                                 uint32_t row_stride, uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const uint32_t cid = i * NT + t, row = cid / (D / 4), cc = cid % (D / 4);
+            r.g[i] = *(const f32x4*)(X + base + (size_t)(row * row_stride + cc * 4));
+        }
+    }
+    template <int STRIDE>
+    static __device__ __forceinline__ void stage(float* lds, const Regs& r, uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const uint32_t cid = i * NT + t, row = cid / (D / 4), cc = cid % (D / 4);
+            *(f32x4*)(lds + row * STRIDE + cc * 4) = r.g[i];
+        }
+    }
+    static __device__ __forceinline__ f32x4 k_frag(const float* k_lds, int kt, int g, uint32_t qn,
+                                                   uint32_t half) {
+        return *(const f32x4*)(k_lds + (kt * 32 + qn) * K_STRIDE + 8 * g + 4 * half);
+    }
+    static __device__ __forceinline__ float v_elem(const float* v_lds, int kt, int i, int mt,
+                                                   uint32_t qn, uint32_t half) {
+        const uint32_t key = kt * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+        return v_lds[key * V_STRIDE + mt * 32 + qn];
+    }
+    static __device__ __forceinline__ void load_q(f32x4 (&qf)[D / 8], const float* q_row, uint32_t half) {
+#pragma unroll
+        for (int g = 0; g < D / 8; ++g) qf[g] = *(const f32x4*)(q_row + 8 * g + 4 * half);
+    }
+};
+
+// Keep-bits of one lane's query row for one key block (block-major mask words), key padding folded in.
+template <int BS>
+__device__ __forceinline__ uint64_t load_keep_word(const void* mask, size_t word_index, int limit) {
+    uint64_t w = ~0ull;
+    if (mask) {
+        if (BS == 64) w = ((const uint64_t*)mask)[word_index];
+        else w = ((const uint32_t*)mask)[word_index];
+    }
+    if (limit < BS) w &= (limit <= 0) ? 0ull : ((1ull << limit) - 1ull);
+    return w;
+}
+
+// Replace the scores of masked keys by kMaskedScore.  keep bit k = key k of the block is kept.
+template <int KT>
+__device__ __forceinline__ void apply_keep(f32x16 (&s)[KT], uint64_t keep, uint32_t half) {
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        const uint32_t w = (uint32_t)(keep >> (kt * 32)) >> (half * 4);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t bit = (i / 4) * 8 + (i % 4);
+            s[kt][i] = ((w >> bit) & 1u) ? s[kt][i] : kMaskedScore;
+        }
+    }
+}
+
+// Maximum over this lane's scores of one block and over the partner lane (the other 16 keys of each
+// 32-key tile of the same query).
+template <int KT>
+__device__ __forceinline__ float block_row_max(const f32x16 (&s)[KT]) {
+    float mx0 = s[0][0], mx1 = s[0][1];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int i = 0; i < 16; i += 4) {
+            mx0 = fmaxf(fmaxf(mx0, s[kt][i]), s[kt][i + 1]);
+            mx1 = fmaxf(fmaxf(mx1, s[kt][i + 2]), s[kt][i + 3]);
+        }
+    }
+    const float m = fmaxf(mx0, mx1);
+    return fmaxf(m, __shfl_xor(m, 32));
+}
+
+}  // namespace sfb

@@ -46,11 +46,25 @@ PATTERNS = {
 
 
 def run_fused(Q, K, V, luts, bs, scale, bf16=False, mask=None, valid_len=None, use_order=True,
-              lut_heads=1, mask_heads=1, nn_lut=None, blocks=None):
+              lut_heads=1, mask_heads=1, nn_lut=None, blocks=None, max_blocks=None, workspace=None):
+    """max_blocks != None runs the scheduled entry point (rows longer than max_blocks are split)."""
     q, k, v = (dev(x, bf16) for x in (Q, K, V))
     nn = sfb.to_device(luts["nn_lut"] if nn_lut is None else nn_lut)
     m = None if mask is None else sfb.to_device(mask)
     vl = None if valid_len is None else sfb.to_device(np.asarray(valid_len, np.int32))
+    if max_blocks is not None:
+        B, L, H, d = Q.shape
+        sched = sfb.build_schedule(luts["nn_lut"], L // bs, max_blocks)
+        if workspace is None:
+            nbytes = sfb.schedule_workspace_bytes(sched, B, H, bs, d)
+            workspace = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device="cuda")
+        o = sfb.fused_attention_scheduled(q, k, v, nn, sfb.to_device(sched["items"]), sched, workspace, bs,
+                                          luts["blocks"], scale, mask=m, valid_len=vl,
+                                          mask_heads=mask_heads)
+        torch.cuda.synchronize()
+        assert int(workspace[:max(4 * B * H * sched["n_slots"], 4)].view(torch.int32).abs().sum()) == 0, \
+            "arrival counters must be left at zero"
+        return o.cpu().numpy()
     order = sfb.to_device(luts["row_order"]) if use_order else None
     o = sfb.fused_attention(q, k, v, nn, bs, luts["blocks"] if blocks is None else blocks, scale,
                             mask=m, valid_len=vl, row_order=order, lut_heads=lut_heads,

@@ -110,3 +110,37 @@ def test_error_codes():
     assert sfb.lib.sfb_pack_mask(lay.ctypes.data_as(C.c_void_p), lay.ctypes.data_as(C.c_void_p), 1, 16) == 2
     with pytest.raises(sfb.capi.SfbError):
         sfb.layout_local(4, -1)
+
+
+@pytest.mark.parametrize("max_blocks", [1, 3, 8, 100])
+def test_schedule_covers_every_block_once(max_blocks):
+    lay = orc.layout_bigbird(64, 1, 2, True, orc.bigbird_draw(64, 1, 2, True, 3, 1234))
+    lay[5] = 0
+    luts = sfb.build_luts(lay)
+    sched = sfb.build_schedule(luts["nn_lut"], 64, max_blocks)
+    items = sched["items"]
+    counts = lay.sum(axis=1)
+    assert sched["n_items"] == len(items)
+    assert (items["count"] <= max(max_blocks, 1)).all()
+    assert (np.diff(items["count"].astype(np.int64)) <= 0).all()  # longest first
+    split_rows = [r for r in range(64) if counts[r] > max_blocks]
+    assert sched["n_slots"] == len(split_rows)
+    assert sched["n_parts"] == sum(-(-int(counts[r]) // max_blocks) for r in split_rows)
+    slots, parts = set(), []
+    for r in range(64):
+        mine = np.sort(items[items["row"] == r], order="first")
+        assert len(mine) >= 1 and (mine["nchunks"] == len(mine)).all()
+        assert mine["first"][0] == 0 and mine["count"].sum() == counts[r]
+        assert (mine["first"][1:] == np.cumsum(mine["count"])[:-1]).all()
+        assert sorted(mine["chunk"].tolist()) == list(range(len(mine)))
+        if len(mine) > 1:
+            assert mine["count"].max() - mine["count"].min() <= 1
+            assert len(set(mine["slot"].tolist())) == 1 and len(set(mine["part"].tolist())) == 1
+            slots.add(int(mine["slot"][0]))
+            parts.append((int(mine["part"][0]), len(mine)))
+    assert slots == set(range(sched["n_slots"]))
+    parts.sort()
+    assert all(parts[i][0] + parts[i][1] == parts[i + 1][0] for i in range(len(parts) - 1))
+    assert not parts or (parts[0][0] == 0 and parts[-1][0] + parts[-1][1] == sched["n_parts"])
+    nbytes = sfb.schedule_workspace_bytes(sched, 4, 12, 64, 64)
+    assert nbytes == (4 * 12 * sched["n_slots"] * 4 + 255) // 256 * 256 + 4 * 12 * sched["n_parts"] * (64 * 64 + 256) * 4

@@ -139,6 +139,44 @@ def test_per_head_luts_and_masks():
     check(got, want, TOL_F32)
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("max_blocks", [8, 3, 1])
+def test_scheduled_split_rows(bf16, max_blocks):
+    """Rows cut into chunks whose partials are merged by the last chunk to finish: same result as the
+    oracle, masks and padding included, and the workspace is reusable launch after launch."""
+    bs, nb, B, H, d = 64, 16, 2, 3, 64
+    L = bs * nb
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    keep = (np.random.default_rng(7).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
+    mask = sfb.pack_mask(keep)
+    valid = np.array([L, L - 100], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=95, bf16=bf16)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, mask=mask, valid_len=valid, nthreads=THREADS)
+    sched = sfb.build_schedule(luts["nn_lut"], nb, max_blocks)
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        got = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, mask=mask, valid_len=valid,
+                        max_blocks=max_blocks, workspace=ws)
+        check(got, want, TOL_BF16 if bf16 else TOL_F32)
+
+
+def test_c4_scheduled_full_size():
+    B, H, L, d, bs = 4, 12, 4096, 64, 64
+    luts = sfb.build_luts(PATTERNS["bigbird"](L // bs))
+    Q, K, V = qkv(1, L, 2, d, seed=44, bf16=True)
+    tile = lambda x: np.ascontiguousarray(np.tile(x, (B, 1, H // 2, 1)))
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    got = run_fused(tile(Q), tile(K), tile(V), luts, bs, 0.125, bf16=True, max_blocks=8)
+    for b in range(B):
+        for h in range(0, H, 2):
+            assert rel_err(got[b:b + 1, :, h:h + 2], want) <= TOL_BF16
+    plain = run_fused(tile(Q), tile(K), tile(V), luts, bs, 0.125, bf16=True)
+    unsplit = [r for r in range(L // bs) if luts["nn_lut"][r, 1] <= 8]
+    rows = np.concatenate([np.arange(r * bs, (r + 1) * bs) for r in unsplit])
+    assert np.array_equal(got[:, rows], plain[:, rows])  # unsplit rows take the identical code path
+    assert rel_err(got, plain) <= 5e-3  # split rows: probabilities are rounded to bf16 relative to per-chunk maxima
+
+
 def test_scale_and_large_scores():
     # scores far from zero: the running maximum and the 1e-6 term must still follow the oracle
     bs, nb, B, H, d = 64, 4, 1, 2, 64
