@@ -156,6 +156,52 @@ int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
 
+/* ---- the unfused trio (kept as the no_fusion comparison) ------------------------------------ */
+
+/* bst_sgemm_nt (openai_blocksparse.h:202-233; blocksparse.h:425): S_blk = A_rowblk . B_colblk^T for
+ * every entry of the NT LUT.  a, b [dev] [batch, ctx, heads, state] of in_dtype; c [dev] sparse
+ * [batch][heads][blocks][bs][bs] of out_dtype (the reference stores bf16; fp32 is offered so the fp32
+ * configurations keep fp32 scores).  lut_dim = blocks.  Unsupported block sizes are an error, not the
+ * reference's silent no-op (openai_blocksparse.h:225-232). */
+int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, void* c,
+               int in_dtype, int out_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+               uint32_t ctx_blks_a, uint32_t ctx_blks_b, uint32_t head_dim, uint32_t state_dim,
+               uint32_t lut_heads, uint32_t lut_dim);
+
+/* BlocksparseMaskedSoftmax<T,V> (blocksparse.h:649-722): y = softmax over each sparse row of x.
+ * lut = NN LUT, lut_dim = ctx_blks + blocks; mask [dev] ROW-major words[row*blocks + blk] (uint32 for
+ * bs 32, uint64 for bs 64) or NULL; valid_len [dev] int32[batch] or NULL (MI355X addition); scale is
+ * the raw 1/sqrt(d) -- log2(e) is folded inside, as blocksparse.h:669 does.  max_lut is accepted for
+ * signature compatibility.  Numerics follow the CPU softmax (ewops.h:64-98), not the reference GPU
+ * kernel's approximations. */
+int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, const void* mask, const void* x,
+                       void* y, int x_dtype, int y_dtype, const int32_t* valid_len, uint32_t block_size,
+                       uint32_t blocks, uint32_t batch_dim, uint32_t head_dim, uint32_t ctx_blks,
+                       uint32_t lut_heads, uint32_t lut_dim, uint32_t max_lut, uint32_t mask_heads,
+                       float scale);
+
+/* bst_sgemm_xn (blocksparse.h:965-1014), op = SFB_NN_OP: C_rowblk = sum over the row's blocks of
+ * A_blk . B_colblk.  a [dev] sparse P of a_dtype; b [dev] V [batch, ctx_b, heads, state] of b_dtype;
+ * c [dev] fp32 [batch, ctx_c, heads, state]; block-rows without blocks are zero-filled
+ * (blocksparse.h:949-962).  The product runs on bf16 MFMA when b is bf16, on fp32 MFMA otherwise.
+ * SFB_TN_OP (the backward product) returns SFB_ERR_ARGUMENT.  magic/shift/max_lut are accepted for
+ * signature compatibility. */
+int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
+               int a_dtype, int b_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+               uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim,
+               uint32_t lut_heads, uint32_t lut_dim, uint32_t op, uint32_t magic, uint32_t shift,
+               uint32_t max_lut);
+
+/* fusion_attention1 / fusion_attention2 (fusion_blocksparse.h:400-455, 1212-1268): sdd + masked
+ * softmax in one kernel, y = P in the sparse layout (fp32 or bf16).  One work-group owns a whole
+ * block-row, so the reference's rblk_flag / rblk_flag1 / Max / Sum scratch and its spin-waits are not
+ * needed.  mask is BLOCK-major here (fusion_blocksparse.h:690). */
+int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const void* a, const void* b,
+                          void* y, int in_dtype, int y_dtype, const void* mask,
+                          const int32_t* valid_len, uint32_t block_size, uint32_t blocks,
+                          uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                          uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -50,6 +50,7 @@ EXPORTED = [
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled",
+    "sfb_sdd_nt", "sfb_masked_softmax", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
 ]
 
 
@@ -257,3 +258,73 @@ def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_si
         C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d),
         C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled")
     return out
+
+
+# ------------------------------------------------------------------------------------ unfused trio
+def _torch_dtype(code):
+    import torch
+    return torch.bfloat16 if code == BF16 else torch.float32
+
+
+def bst_sgemm_nt(lut, a, b, block_size, blocks, out_dtype=None, lut_heads=1, c=None):
+    """sdd: S [B, H, blocks, bs, bs] = a_rowblk . b_colblk^T per NT-LUT entry (openai_blocksparse.h:202)."""
+    import torch
+    B, L, H, d = a.shape
+    if c is None:
+        c = torch.empty((B, H, blocks, block_size, block_size), device=a.device,
+                        dtype=_torch_dtype(F32 if out_dtype is None else out_dtype))
+    _check(lib.sfb_sdd_nt(_stream(), _dev(lut), _dev(a), _dev(b), _dev(c), _dtype_code(a), _dtype_code(c),
+                          C.c_uint32(block_size), C.c_uint32(blocks), C.c_uint32(B),
+                          C.c_uint32(L // block_size), C.c_uint32(b.shape[1] // block_size), C.c_uint32(H),
+                          C.c_uint32(d), C.c_uint32(lut_heads), C.c_uint32(blocks)), "sfb_sdd_nt")
+    return c
+
+
+def BlocksparseMaskedSoftmax(lut, mask, x, ctx_blks, scale, out_dtype=None, valid_len=None, lut_heads=1,
+                             mask_heads=1, max_lut=0, y=None):
+    """Row softmax over the sparse scores (blocksparse.h:649); mask is ROW-major (transpose_mask)."""
+    import torch
+    B, H, blocks, bs, _ = x.shape
+    if y is None:
+        y = torch.empty_like(x, dtype=_torch_dtype(_dtype_code(x) if out_dtype is None else out_dtype))
+    _check(lib.sfb_masked_softmax(_stream(), _dev(lut), _dev(mask), _dev(x), _dev(y), _dtype_code(x),
+                                  _dtype_code(y), _dev(valid_len), C.c_uint32(bs), C.c_uint32(blocks),
+                                  C.c_uint32(B), C.c_uint32(H), C.c_uint32(ctx_blks), C.c_uint32(lut_heads),
+                                  C.c_uint32(ctx_blks + blocks), C.c_uint32(max_lut),
+                                  C.c_uint32(mask_heads), C.c_float(scale)), "sfb_masked_softmax")
+    return y
+
+
+def bst_sgemm_xn(lut, a, b, ctx_blks_c, op=NN_OP, lut_heads=1, magic=1, shift=0, max_lut=0, c=None):
+    """dsd: O [B, L, H, d] = sum_blk P_blk . V_colblk (blocksparse.h:965)."""
+    import torch
+    B, H, blocks, bs, _ = a.shape
+    _, Lb, _, d = b.shape
+    if c is None:
+        c = torch.empty((B, ctx_blks_c * bs, H, d), device=b.device, dtype=torch.float32)
+    _check(lib.sfb_dsd_xn(_stream(), _dev(lut), _dev(a), _dev(b), _dev(c), _dtype_code(a), _dtype_code(b),
+                          C.c_uint32(bs), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(Lb // bs),
+                          C.c_uint32(ctx_blks_c), C.c_uint32(H), C.c_uint32(d), C.c_uint32(lut_heads),
+                          C.c_uint32(ctx_blks_c + blocks), C.c_uint32(op), C.c_uint32(magic),
+                          C.c_uint32(shift), C.c_uint32(max_lut)), "sfb_dsd_xn")
+    return c
+
+
+def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_len=None, out_dtype=None,
+                      lut_heads=1, mask_heads=1, y=None):
+    """sdd + masked softmax in one kernel -> P (fusion_blocksparse.h:1212); mask is BLOCK-major."""
+    import torch
+    B, L, H, d = a.shape
+    if y is None:
+        y = torch.empty((B, H, blocks, block_size, block_size), device=a.device,
+                        dtype=_torch_dtype(F32 if out_dtype is None else out_dtype))
+    nb = L // block_size
+    _check(lib.sfb_fused_sdd_softmax(_stream(), _dev(nn_lut), _dev(a), _dev(b), _dev(y), _dtype_code(a),
+                                     _dtype_code(y), _dev(mask), _dev(valid_len), C.c_uint32(block_size),
+                                     C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H),
+                                     C.c_uint32(d), C.c_uint32(lut_heads), C.c_uint32(nb + blocks),
+                                     C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_sdd_softmax")
+    return y
+
+
+fusion_attention1 = fusion_attention2

@@ -1,0 +1,461 @@
+// The unfused block-sparse attention trio, kept as the comparison path for the fused kernel:
+//   sdd  : S_blk = Q_rowblk . K_colblk^T for every block of the NT look-up table   (sfb_sdd_nt)
+//   softmax over the sparse row (scaled, masked)                                    (sfb_masked_softmax)
+//   dsd  : O_rowblk = sum_blk P_blk . V_colblk                                      (sfb_dsd_xn)
+// S and P live in memory as [batch][heads][blocks][bs][bs] (openai_blocksparse.h:148), fp32 or bf16.
+// Also here: the two-stage fusion  sdd + softmax -> P  of the reference's fusion_attention1/2
+// (sfb_fused_sdd_softmax), done by one work-group per block-row without any inter-group exchange.
+//
+// Arithmetic follows the CPU path of the reference (matmul.h:53-78, ewops.h:64-98, matmul.h:6-20).
+#include "tiles.hip.h"
+
+namespace sfb {
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ f32x4 load4(const float* p) { return *(const f32x4*)p; }
+    static __device__ __forceinline__ void store4(float* p, f32x4 v) { *(f32x4*)p = v; }
+    static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Elem<__bf16> {
+    static __device__ __forceinline__ float load(const __bf16* p) {
+        return bf16_bits_to_f32(*(const uint16_t*)p);
+    }
+    static __device__ __forceinline__ f32x4 load4(const __bf16* p) {
+        const u32x2 r = *(const u32x2*)p;
+        const f32x4 v = {bf16_bits_to_f32(r.x & 0xffffu), bf16_bits_to_f32(r.x >> 16),
+                         bf16_bits_to_f32(r.y & 0xffffu), bf16_bits_to_f32(r.y >> 16)};
+        return v;
+    }
+    static __device__ __forceinline__ void store4(__bf16* p, f32x4 v) {
+        const u32x2 r = {pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+        *(u32x2*)p = r;
+    }
+    static __device__ __forceinline__ void store(__bf16* p, float v) {
+        *(uint16_t*)p = (uint16_t)(pack_bf16(v, 0.f) & 0xffffu);
+    }
+};
+
+// Transposed score tile of one wave (32 queries x BS keys), operands read straight from memory.
+// Accumulator element i of key tile kt is key kt*32 + (i/4)*8 + half*4 + i%4 of query qn.
+template <int BS, int D, typename TIn>
+__device__ __forceinline__ void score_tile_direct(f32x16 (&s)[BS / 32], const TIn* q_row, const TIn* k_blk,
+                                                  uint32_t row_stride, uint32_t qn, uint32_t half) {
+    constexpr int KT = BS / 32;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+    if constexpr (sizeof(TIn) == 2) {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+            const bf16x8 b = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const bf16x8 a = *(const bf16x8*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + (2 * ks + half) * 8);
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, s[kt], 0, 0, 0);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int g = 0; g < D / 8; ++g) {
+            const f32x4 b = *(const f32x4*)(q_row + 8 * g + 4 * half);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const f32x4 a = *(const f32x4*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + 8 * g + 4 * half);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], s[kt], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// Store this lane's part of a BS x BS block (row = its query): groups of 4 consecutive keys.
+template <int BS, typename TOut>
+__device__ __forceinline__ void store_block_row(TOut* row_ptr, const f32x16 (&s)[BS / 32], uint32_t half) {
+#pragma unroll
+    for (int kt = 0; kt < BS / 32; ++kt)
+#pragma unroll
+        for (int ig = 0; ig < 4; ++ig) {
+            const f32x4 v = {s[kt][ig * 4 + 0], s[kt][ig * 4 + 1], s[kt][ig * 4 + 2], s[kt][ig * 4 + 3]};
+            Elem<TOut>::store4(row_ptr + kt * 32 + ig * 8 + half * 4, v);
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// sdd: grid (blocks, batch, heads), one BS x BS block per work-group (openai_blocksparse.h:224)
+// ---------------------------------------------------------------------------------------------
+struct SddParams {
+    const sfb_uint2* lut;
+    const void* a;
+    const void* b;
+    void* c;
+    uint32_t blocks, heads, ctx_a, ctx_b, lut_stride;
+};
+
+template <int BS, int D, typename TIn, typename TOut>
+__global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
+    const uint32_t blk = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const sfb_uint2 e = p.lut[(size_t)h * p.lut_stride + blk];
+    const uint32_t row_stride = p.heads * D;
+    const TIn* q_row = (const TIn*)p.a + token_offset(b, e.x * BS + wave * 32 + qn, h, p.ctx_a, p.heads, D);
+    const TIn* k_blk = (const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, D);
+    f32x16 s[BS / 32];
+    score_tile_direct<BS, D, TIn>(s, q_row, k_blk, row_stride, qn, half);
+    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32 + qn) * BS;
+    store_block_row<BS, TOut>(out, s, half);
+}
+
+// ---------------------------------------------------------------------------------------------
+// masked softmax: one wave per query row, lanes = keys (64/BS blocks per step)
+// (blocksparse.h:459-722 keeps one CTA per query row; the row-major mask order is the same)
+// ---------------------------------------------------------------------------------------------
+struct SoftmaxParams {
+    const sfb_uint2* lut;     // NN LUT
+    const void* mask;         // row-major words[row*blocks + blk], or nullptr
+    const int32_t* valid_len;
+    const void* x;
+    void* y;
+    uint32_t blocks, batch, heads, nb, lut_stride, mask_stride;
+    float scale_log2e;
+};
+
+template <int BS, typename TX, typename TY>
+__global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
+    constexpr int PER = 64 / BS;  // blocks covered by one wave step
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint64_t row_id = (uint64_t)blockIdx.x * 4 + wave;        // over batch*heads*nb*BS
+    const uint64_t total_rows = (uint64_t)p.batch * p.heads * p.nb * BS;
+    if (row_id >= total_rows) return;
+    const uint32_t qi = (uint32_t)(row_id % BS);
+    const uint32_t r = (uint32_t)((row_id / BS) % p.nb);
+    const uint32_t bh = (uint32_t)(row_id / ((uint64_t)BS * p.nb));
+    const uint32_t b = bh / p.heads, h = bh % p.heads;
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
+    const uint32_t off = lut[r].x, count = lut[r].y;
+    const uint32_t sub = lane / BS, key = lane % BS;
+    const TX* x = (const TX*)p.x + (size_t)bh * p.blocks * BS * BS;
+    TY* y = (TY*)p.y + (size_t)bh * p.blocks * BS * BS;
+    const int valid = p.valid_len ? p.valid_len[b] : (int)(p.nb * BS);
+    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    const float c = p.scale_log2e;
+
+    auto kept = [&](const sfb_uint2 e) -> bool {
+        bool k = (int)(e.y * BS + key) < valid;
+        if (mask) {
+            const size_t w = (size_t)qi * p.blocks + e.x;
+            const uint64_t word = (BS == 64) ? ((const uint64_t*)mask)[w] : ((const uint32_t*)mask)[w];
+            k = k && ((word >> key) & 1ull);
+        }
+        return k;
+    };
+
+    // pass 1: row maximum over kept keys (seed as ewops.h:70), then the sum relative to it
+    float m = kMaxSeed;
+    for (uint32_t j = sub; j < count; j += PER) {
+        const sfb_uint2 e = lut[off + j];
+        const float v = Elem<TX>::load(x + ((size_t)e.x * BS + qi) * BS + key);
+        if (kept(e)) m = fmaxf(m, v);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+    float l = 0.f;
+    for (uint32_t j = sub; j < count; j += PER) {
+        const sfb_uint2 e = lut[off + j];
+        const float v = Elem<TX>::load(x + ((size_t)e.x * BS + qi) * BS + key);
+        if (kept(e)) l += exp2_fast((v - m) * c);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+    const float inv = 1.0f / (l + 1e-6f);
+    // pass 2: normalised probabilities, zeros at masked keys (ewops.h:82)
+    for (uint32_t j = sub; j < count; j += PER) {
+        const sfb_uint2 e = lut[off + j];
+        const size_t at = ((size_t)e.x * BS + qi) * BS + key;
+        const float v = Elem<TX>::load(x + at);
+        Elem<TY>::store(y + at, kept(e) ? exp2_fast((v - m) * c) * inv : 0.f);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dsd: one work-group per (batch, head, block-row), V staged through LDS, P read in operand layout
+// ---------------------------------------------------------------------------------------------
+struct DsdParams {
+    const sfb_uint2* lut;   // NN LUT
+    const void* a;          // P
+    const void* b;          // V
+    float* c;               // O
+    uint32_t blocks, batch, heads, nb_b, nb_c, lut_stride, groups;
+};
+
+template <int BS, int D, typename TP, typename TV>
+__global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
+    constexpr int KT = BS / 32, NO = D / 32;
+    constexpr bool kBf16 = sizeof(TV) == 2;
+    using TB = Bf16Tiles<BS, D>;
+    using TF = F32Tiles<BS, D>;
+    constexpr int LDS_BYTES = kBf16 ? TB::V_BYTES : TF::V_FLOATS * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t smem[LDS_BYTES];
+
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.groups);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t r = p.nb_c - 1 - work.rank;   // long rows of causal layouts first (blocksparse.h:746-748)
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t row_stride = p.heads * D;
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
+    const uint32_t off = lut[r].x, count = lut[r].y;
+    float* o_row = p.c + token_offset(b, r * BS + q_in_block, h, p.nb_c * BS, p.heads, D);
+    const TP* P = (const TP*)p.a + (size_t)work.bh * p.blocks * BS * BS;
+    const TV* V = (const TV*)p.b;
+
+    f32x16 o_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
+
+    for (uint32_t j = 0; j < count; ++j) {
+        const sfb_uint2 e = lut[off + j];
+        const size_t base = token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
+        const TP* p_row = P + ((size_t)e.x * BS + q_in_block) * BS;
+        if constexpr (kBf16) {
+            typename TB::VRegs gv;
+            TB::fetch_v(gv, (const __bf16*)V, base, row_stride, t);
+            TB::stage_v(smem, gv, t);
+            __syncthreads();
+#pragma unroll
+            for (int u = 0; u < BS / 16; ++u) {
+                // slots j: key 16u + 8(j/4) + 4*half + j%4
+                const f32x4 lo = Elem<TP>::load4(p_row + 16 * u + 4 * half);
+                const f32x4 hi = Elem<TP>::load4(p_row + 16 * u + 8 + 4 * half);
+                const u32x4 pb = {pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y),
+                                  pack_bf16(hi.z, hi.w)};
+                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TB::v_frag(smem, mt, u, qn, half), bfrag,
+                                                                        o_acc[mt], 0, 0, 0);
+            }
+        } else {
+            float* v_lds = (float*)smem;
+            typename TF::Regs gv;
+            TF::fetch(gv, (const float*)V, base, row_stride, t);
+            TF::template stage<TF::V_STRIDE>(v_lds, gv, t);
+            __syncthreads();
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ig = 0; ig < 4; ++ig) {
+                    const f32x4 pv = Elem<TP>::load4(p_row + kt * 32 + ig * 8 + half * 4);
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4)
+#pragma unroll
+                        for (int mt = 0; mt < NO; ++mt)
+                            o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                TF::v_elem(v_lds, kt, ig * 4 + e4, mt, qn, half), pv[e4], o_acc[mt], 0, 0, 0);
+                }
+        }
+        __syncthreads();
+    }
+    // block-rows without blocks write zeros (blocksparse.h:949-962)
+#pragma unroll
+    for (int mt = 0; mt < NO; ++mt)
+#pragma unroll
+        for (int ig = 0; ig < 4; ++ig) {
+            const f32x4 out = {o_acc[mt][ig * 4 + 0], o_acc[mt][ig * 4 + 1], o_acc[mt][ig * 4 + 2],
+                               o_acc[mt][ig * 4 + 3]};
+            *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// sdd + softmax -> P in one kernel, one work-group per block-row, two passes over the row's key
+// blocks (statistics, then normalised probabilities).  Replaces fusion_attention1/2, whose
+// per-block work-groups exchange row maxima and sums through global flags and spin on them
+// (fusion_blocksparse.h:224-366); a work-group that owns the whole block-row needs neither.
+// ---------------------------------------------------------------------------------------------
+struct SddSoftmaxParams {
+    const sfb_uint2* nn_lut;
+    const void* a;
+    const void* b;
+    void* y;
+    const void* mask;        // block-major words
+    const int32_t* valid_len;
+    uint32_t blocks, batch, heads, nb, lut_stride, mask_stride, groups;
+    float scale_log2e;
+};
+
+template <int BS, int D, typename TIn, typename TOut>
+__global__ __launch_bounds__(BS * 2, 2) void sdd_softmax_kernel(SddSoftmaxParams p) {
+    constexpr int KT = BS / 32;
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.groups);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t r = p.nb - 1 - work.rank;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t L = p.nb * BS, row_stride = p.heads * D;
+    const sfb_uint2* lut = p.nn_lut + (size_t)h * p.lut_stride;
+    const uint32_t off = lut[r].x, count = lut[r].y;
+    const TIn* q_row = (const TIn*)p.a + token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+    const TIn* K = (const TIn*)p.b;
+    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+    const float c = p.scale_log2e;
+    TOut* Y = (TOut*)p.y + (size_t)work.bh * p.blocks * BS * BS;
+
+    float m = kMaxSeed, l = 0.f;   // exact running maximum and the sum relative to it (this lane's keys)
+    for (int pass = 0; pass < 2; ++pass) {
+        float inv = 0.f;
+        if (pass == 1) {
+            const float total = l + __shfl_xor(l, 32);
+            inv = 1.0f / (total + 1e-6f);
+        }
+        for (uint32_t j = 0; j < count; ++j) {
+            const sfb_uint2 e = lut[off + j];
+            f32x16 s[KT];
+            score_tile_direct<BS, D, TIn>(s, q_row, K + token_offset(b, e.y * BS, h, L, p.heads, D), row_stride,
+                                          qn, half);
+            const int limit = valid - (int)(e.y * BS);
+            const bool masked = (mask != nullptr) || (limit < BS);
+            if (masked) apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)e.x * BS + q_in_block, limit), half);
+            if (pass == 0) {
+                const float m_new = fmaxf(m, block_row_max<KT>(s));
+                l *= exp2_fast((m - m_new) * c);
+                m = m_new;
+                const float mc = m * c;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) l += exp2_fast(__builtin_fmaf(s[kt][i], c, -mc));
+            } else {
+                const float mc = m * c;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[kt][i] = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc)) * inv;
+                store_block_row<BS, TOut>(Y + ((size_t)e.x * BS + q_in_block) * BS, s, half);
+            }
+        }
+    }
+}
+
+static int check_dtype(int d) { return (d == SFB_F32 || d == SFB_BF16) ? SFB_OK : SFB_ERR_DTYPE; }
+
+}  // namespace sfb
+
+using namespace sfb;
+
+#define SFB_DISPATCH_2(BSV, T0, T1, CALL)                                                  \
+    do {                                                                                   \
+        if ((T0) == SFB_F32 && (T1) == SFB_F32) { CALL(BSV, float, float); }               \
+        else if ((T0) == SFB_F32 && (T1) == SFB_BF16) { CALL(BSV, float, __bf16); }        \
+        else if ((T0) == SFB_BF16 && (T1) == SFB_F32) { CALL(BSV, __bf16, float); }        \
+        else { CALL(BSV, __bf16, __bf16); }                                                \
+    } while (0)
+
+extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, void* c,
+                          int in_dtype, int out_dtype, uint32_t block_size, uint32_t blocks,
+                          uint32_t batch_dim, uint32_t ctx_blks_a, uint32_t ctx_blks_b, uint32_t head_dim,
+                          uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim) {
+    if (!lut || !a || !b || !c) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(in_dtype) || check_dtype(out_dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks_a || !ctx_blks_b || !lut_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && lut_heads != head_dim) return SFB_ERR_SHAPE;
+    if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
+    if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
+    SddParams p = {lut, a, b, c, blocks, head_dim, ctx_blks_a * block_size, ctx_blks_b * block_size,
+                   lut_heads > 1 ? lut_dim : 0};
+    const dim3 grid(blocks, batch_dim, head_dim);
+    hipStream_t s = (hipStream_t)stream;
+#define SFB_CALL(BSV, TI, TO) sdd_nt_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
+    if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, out_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, in_dtype, out_dtype, SFB_CALL);
+#undef SFB_CALL
+    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
+extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, const void* mask, const void* x,
+                                  void* y, int x_dtype, int y_dtype, const int32_t* valid_len,
+                                  uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t head_dim,
+                                  uint32_t ctx_blks, uint32_t lut_heads, uint32_t lut_dim, uint32_t max_lut,
+                                  uint32_t mask_heads, float scale) {
+    (void)max_lut;  // sizes the reference's shared memory (blocksparse.h:671-686); not needed here
+    if (!lut || !x || !y) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(x_dtype) || check_dtype(y_dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads || !mask_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
+    if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    SoftmaxParams p = {lut, mask, valid_len, x, y, blocks, batch_dim, head_dim, ctx_blks,
+                       lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0, scale * kLog2e};
+    const uint64_t rows = (uint64_t)batch_dim * head_dim * ctx_blks * block_size;
+    if ((rows + 3) / 4 > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const dim3 grid((uint32_t)((rows + 3) / 4));
+    hipStream_t s = (hipStream_t)stream;
+#define SFB_CALL(BSV, TX, TY) masked_softmax_kernel<BSV, TX, TY><<<grid, dim3(256), 0, s>>>(p)
+    if (block_size == 64) SFB_DISPATCH_2(64, x_dtype, y_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, x_dtype, y_dtype, SFB_CALL);
+#undef SFB_CALL
+    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
+extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
+                          int a_dtype, int b_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                          uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim,
+                          uint32_t lut_heads, uint32_t lut_dim, uint32_t op, uint32_t magic, uint32_t shift,
+                          uint32_t max_lut) {
+    (void)magic; (void)shift; (void)max_lut;  // grid decomposition / smem sizing of the reference kernel
+    if (!lut || !a || !b || !c) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(a_dtype) || check_dtype(b_dtype)) return SFB_ERR_DTYPE;
+    if (op != SFB_NN_OP) return SFB_ERR_ARGUMENT;   // TN_OP is the backward product: not part of this path
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks_b || !ctx_blks_c || !lut_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks_c + blocks)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
+    DsdParams p = {lut, a, b, c, blocks, batch_dim, head_dim, ctx_blks_b, ctx_blks_c,
+                   lut_heads > 1 ? lut_dim : 0, bh_groups(batch_dim * head_dim)};
+    const dim3 grid(p.groups * 8u * ctx_blks_c);
+    hipStream_t s = (hipStream_t)stream;
+#define SFB_CALL(BSV, TP, TV) dsd_nn_kernel<BSV, 64, TP, TV><<<grid, dim3(BSV * 2), 0, s>>>(p)
+    if (block_size == 64) SFB_DISPATCH_2(64, a_dtype, b_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, a_dtype, b_dtype, SFB_CALL);
+#undef SFB_CALL
+    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
+extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const void* a,
+                                     const void* b, void* y, int in_dtype, int y_dtype, const void* mask,
+                                     const int32_t* valid_len, uint32_t block_size, uint32_t blocks,
+                                     uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                     uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim,
+                                     uint32_t mask_heads, float scale) {
+    if (!nn_lut || !a || !b || !y) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(in_dtype) || check_dtype(y_dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads || !mask_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
+    if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
+    SddSoftmaxParams p = {nn_lut, a, b, y, mask, valid_len, blocks, batch_dim, head_dim, ctx_blks,
+                          lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0,
+                          bh_groups(batch_dim * head_dim), scale * kLog2e};
+    const dim3 grid(p.groups * 8u * ctx_blks);
+    hipStream_t s = (hipStream_t)stream;
+#define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
+    if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);
+#undef SFB_CALL
+    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+}
