@@ -202,6 +202,58 @@ int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const vo
                           uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                           uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale);
 
+/* ---- encoder-layer ops (one pass over HBM each) ------------------------------------------------ */
+
+/* bias (ewops.h:10-17; cuda_kernels.h:459-489), gelu (ewops.h:32-43; cuda_kernels.h:561-581: the
+ * sigmoid form x/(1+exp(-1.702x))) and tensor_add_tensor (ewops.h:296-301; cuda_kernels.h:449-457)
+ * as one kernel: out = act(in + bias[col]) + residual.  bias, residual may be NULL; act 0 = none,
+ * 1 = GELU; out of out_dtype (fp32, or bf16 to feed a bf16 GEMM / attention); cols % 4 == 0;
+ * out may alias in. */
+int sfb_bias_act(sfb_stream_t stream, void* out, int out_dtype, const float* in, const float* bias,
+                 const float* residual, int act, uint64_t rows, uint32_t cols);
+/* layernorm (layernorm.h:13-38; cuda_kernels.h:334-372): mean and E[x^2] per row, eps 1e-5 inside the
+ * root, affine; mean / rstd [dev] rows floats or NULL; state % 4 == 0. */
+int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, float* mean, float* rstd, const float* in,
+                  const float* gain, const float* bias, uint32_t rows, uint32_t state);
+/* tensor_add_matrix (ewops.h:276-282; cuda_kernels.h:526-535): out[b][i] = a[b][i] + m[i]. */
+int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, const float* m, uint32_t dim0,
+                   uint64_t inner);
+/* embedding_lookup (embedding.h:5-12; cuda_kernels.h:210-221), optionally fused with the position add:
+ * out[t] = table[ids[t]] (+ pos[t % seq_len]); pos may be NULL. */
+int sfb_embedding_lookup(sfb_stream_t stream, float* out, const float* table, const int32_t* ids,
+                         const float* pos, uint64_t tokens, uint32_t state, uint32_t seq_len, uint32_t vocab);
+/* fp32 -> bf16, round to nearest even (the reference's to_bhalf, ew_op_gpu.h:241-254, rounds half
+ * away from zero; inputs of the bf16 configurations are defined as RNE-rounded); n % 4 == 0. */
+int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in, uint64_t n);
+
+/* cblas_sgemm(RowMajor, NoTrans, NoTrans, m, n, k, 1, A, k, W, n, 0, C, n) (transformer.cpp:516-522, 547,
+ * 562, 571; cublasSgemm twins transformer_attention_optimize.cu:693-716): C[m][n] = A[m][k] W[k][n],
+ * a and w of dtype (fp32, or bf16 with fp32 accumulation), c fp32.  Runs on rocBLAS. */
+int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m, uint32_t n,
+             uint32_t k);
+
+/* Weights of one encoder layer, [in][out] row-major (transformer.cpp:98-136): matrices in the compute
+ * dtype (fp32 or bf16), biases and LayerNorm parameters fp32.  All [dev]. */
+typedef struct {
+    const void *wq, *wk, *wv, *wo, *w1, *w2;
+    const float *bq, *bk, *bv, *bo, *b1, *b2;
+    const float *ln1_g, *ln1_b, *ln2_g, *ln2_b;
+} sfb_layer_weights;
+size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim,
+                                         uint32_t state_dim, uint32_t ffn, int dtype);
+/* One post-LN encoder layer forward (op arithmetic and order of transformer.cpp:513-580, no dropout):
+ * x1 = LN1(x + Attn(xWq+bq, xWk+bk, xWv+bv) Wo + bo); y = LN2(x1 + gelu(x1 W1 + b1) W2 + b2).
+ * x, y [dev] fp32 [batch*ctx, heads*state]; dtype selects fp32 or bf16 operands for the GEMMs and the
+ * attention (accumulation, LayerNorm, residuals and y stay fp32).  items may be NULL (one work-group
+ * per block-row); otherwise items / n_* / attn_workspace are those of sfb_fused_attention_scheduled.
+ * workspace [dev] 256-byte aligned, sfb_encoder_layer_workspace_bytes() bytes. */
+int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
+                              int dtype, const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                              const sfb_work_item* items, uint32_t n_items, uint32_t n_slots, uint32_t n_parts,
+                              void* attn_workspace, size_t attn_workspace_bytes, uint32_t block_size,
+                              uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                              uint32_t state_dim, uint32_t ffn, void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

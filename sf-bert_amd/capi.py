@@ -40,6 +40,7 @@ lib.sfb_status_string.argtypes = [C.c_int]
 lib.sfb_count_blocks.restype = C.c_uint32
 lib.sfb_magicu64.restype = None
 lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
+lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -51,6 +52,8 @@ EXPORTED = [
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
+    "sfb_bias_act", "sfb_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
+    "sfb_gemm", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
 ]
 
 
@@ -328,3 +331,136 @@ def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_
 
 
 fusion_attention1 = fusion_attention2
+
+
+# ------------------------------------------------------------------------------------ layer ops
+def bias_act(x, bias=None, residual=None, act=0, out_dtype=F32, out=None):
+    """out = act(x + bias[col]) + residual (bias: ewops.h:10, gelu: ewops.h:32, tensor_add_tensor: ewops.h:296)."""
+    import torch
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if out is None:
+        out = torch.empty(x.shape, device=x.device, dtype=_torch_dtype(out_dtype))
+    _check(lib.sfb_bias_act(_stream(), _dev(out), _dtype_code(out), _dev(x), _dev(bias), _dev(residual),
+                            int(act), C.c_uint64(rows), C.c_uint32(cols)), "sfb_bias_act")
+    return out
+
+
+def bias(x, b):
+    return bias_act(x, bias=b)
+
+
+def gelu(x):
+    return bias_act(x, act=1)
+
+
+def tensor_add_tensor(a, b):
+    return bias_act(a, residual=b)
+
+
+def layernorm(x, gain, beta, out_dtype=F32, return_stats=False):
+    """layernorm.h:13-38; returns out (and mean, rstd)."""
+    import torch
+    state = x.shape[-1]
+    rows = x.numel() // state
+    out = torch.empty(x.shape, device=x.device, dtype=_torch_dtype(out_dtype))
+    mean = torch.empty(rows, device=x.device) if return_stats else None
+    rstd = torch.empty(rows, device=x.device) if return_stats else None
+    _check(lib.sfb_layernorm(_stream(), _dev(out), _dtype_code(out), _dev(mean), _dev(rstd), _dev(x),
+                             _dev(gain), _dev(beta), C.c_uint32(rows), C.c_uint32(state)), "sfb_layernorm")
+    return (out, mean, rstd) if return_stats else out
+
+
+def tensor_add_matrix(a, m):
+    import torch
+    out = torch.empty_like(a)
+    _check(lib.sfb_add_matrix(_stream(), _dev(out), _dev(a), _dev(m), C.c_uint32(a.shape[0]),
+                              C.c_uint64(m.numel())), "sfb_add_matrix")
+    return out
+
+
+def embedding_lookup(table, ids, pos=None):
+    """out[t] = table[ids[t]] (+ pos[t % seq_len]); ids int32 [B, L]."""
+    import torch
+    vocab, state = table.shape
+    out = torch.empty(tuple(ids.shape) + (state,), device=table.device, dtype=torch.float32)
+    seq_len = ids.shape[-1]
+    _check(lib.sfb_embedding_lookup(_stream(), _dev(out), _dev(table), _dev(ids), _dev(pos),
+                                    C.c_uint64(ids.numel()), C.c_uint32(state), C.c_uint32(seq_len),
+                                    C.c_uint32(vocab)), "sfb_embedding_lookup")
+    return out
+
+
+def cast_bf16(x):
+    import torch
+    out = torch.empty(x.shape, device=x.device, dtype=torch.bfloat16)
+    _check(lib.sfb_cast_f32_bf16(_stream(), _dev(out), _dev(x), C.c_uint64(x.numel())), "sfb_cast_f32_bf16")
+    return out
+
+
+def gemm(a, w):
+    """C[m, n] = a[m, k] @ w[k, n], fp32 or bf16 operands, fp32 result (cblas_sgemm call sites, transformer.cpp:516)."""
+    import torch
+    m, k = a.shape
+    n = w.shape[1]
+    c = torch.empty((m, n), device=a.device, dtype=torch.float32)
+    _check(lib.sfb_gemm(_stream(), _dev(c), _dev(a), _dev(w), _dtype_code(a), C.c_uint32(m), C.c_uint32(n),
+                        C.c_uint32(k)), "sfb_gemm")
+    return c
+
+
+class LayerWeights(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "bq", "bk", "bv", "bo", "b1", "b2",
+                                          "ln1_g", "ln1_b", "ln2_g", "ln2_b")]
+
+
+class EncoderLayer:
+    """One post-LN encoder layer with block-sparse attention (sfb_encoder_layer_forward).
+
+    weights: dict of fp32 CUDA tensors (wq..w2 [in, out], bq..b2, ln1_g, ln1_b, ln2_g, ln2_b);
+    dtype BF16 casts the six matrices to bf16 once."""
+
+    def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16):
+        import torch
+        self.dtype, self.bs, self.heads, self.d, self.ffn = dtype, block_size, heads, head_state, ffn
+        self.luts = luts
+        self.tensors = {}
+        for name, t in weights.items():
+            t = t.contiguous()
+            if dtype == BF16 and name in ("wq", "wk", "wv", "wo", "w1", "w2"):
+                t = cast_bf16(t)
+            self.tensors[name] = t
+        self.c_weights = LayerWeights(**{n: t.data_ptr() for n, t in self.tensors.items()})
+        self.nn_lut = to_device(luts["nn_lut"])
+        self.sched = build_schedule(luts["nn_lut"], luts["nb"], max_blocks) if max_blocks else None
+        self.items = to_device(self.sched["items"]) if self.sched else None
+        self._ws = {}
+
+    def _workspaces(self, B, L, device):
+        import torch
+        key = (B, L)
+        if key not in self._ws:
+            nbytes = int(lib.sfb_encoder_layer_workspace_bytes(C.c_uint32(B), C.c_uint32(L), C.c_uint32(self.heads),
+                                                               C.c_uint32(self.d), C.c_uint32(self.ffn), self.dtype))
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            aws = None
+            if self.sched:
+                aws = torch.zeros(max(schedule_workspace_bytes(self.sched, B, self.heads, self.bs, self.d), 256),
+                                  dtype=torch.uint8, device=device)
+            self._ws[key] = (ws, aws)
+        return self._ws[key]
+
+    def forward(self, x, B, L, mask=None, valid_len=None, out=None):
+        import torch
+        if out is None:
+            out = torch.empty_like(x)
+        ws, aws = self._workspaces(B, L, x.device)
+        s = self.sched
+        _check(lib.sfb_encoder_layer_forward(
+            _stream(), _dev(out), _dev(x), C.byref(self.c_weights), self.dtype, _dev(self.nn_lut), _dev(mask),
+            _dev(valid_len), _dev(self.items), C.c_uint32(s["n_items"] if s else 0),
+            C.c_uint32(s["n_slots"] if s else 0), C.c_uint32(s["n_parts"] if s else 0), _dev(aws),
+            C.c_size_t(aws.numel() if aws is not None else 0), C.c_uint32(self.bs), C.c_uint32(self.luts["blocks"]),
+            C.c_uint32(B), C.c_uint32(L // self.bs), C.c_uint32(self.heads), C.c_uint32(self.d),
+            C.c_uint32(self.ffn), _dev(ws), C.c_size_t(ws.numel())), "sfb_encoder_layer_forward")
+        return out

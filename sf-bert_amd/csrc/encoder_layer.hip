@@ -1,0 +1,133 @@
+// Dense GEMM seam (rocBLAS) and the forward pass of one BERT encoder layer with block-sparse
+// attention inside.  Op order is that of the reference's CPU layer (transformer.cpp:513-580: GEMM,
+// bias, attention, out-projection, bias, residual, LayerNorm, FFN GEMM, bias, GELU, GEMM, bias,
+// residual) arranged post-LN and without dropout:
+//     x1 = LN1(x + Attn(x Wq + bq, x Wk + bk, x Wv + bv) Wo + bo)
+//     y  = LN2(x1 + gelu(x1 W1 + b1) W2 + b2)
+// Weights are [in][out] row-major as in the reference (cblas_sgemm(RowMajor, N, N, m, n, k, A, k, W, n,
+// C, n), transformer.cpp:516); the GEMM is issued column-major as C^T = W^T A^T, the same trick as the
+// reference's cuBLAS calls (transformer_attention_optimize.cu:693-716).
+#include <hip/hip_runtime.h>
+#include <rocblas/rocblas.h>
+
+#include <mutex>
+
+#include "../../include/sfbert_hip.h"
+
+namespace {
+
+std::mutex g_mutex;
+rocblas_handle g_handle = nullptr;
+
+rocblas_handle blas_handle() {
+    if (!g_handle) {
+        if (rocblas_create_handle(&g_handle) != rocblas_status_success) g_handle = nullptr;
+    }
+    return g_handle;
+}
+
+inline size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+}  // namespace
+
+extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
+                        uint32_t n, uint32_t k) {
+    if (!c || !a || !w) return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (!m || !n || !k) return SFB_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    rocblas_handle h = blas_handle();
+    if (!h) return SFB_ERR_LAUNCH;
+    if (rocblas_set_stream(h, (hipStream_t)stream) != rocblas_status_success) return SFB_ERR_LAUNCH;
+    const float alpha = 1.0f, beta = 0.0f;
+    const rocblas_datatype in = dtype == SFB_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
+    // row-major C[m][n] = A[m][k] W[k][n]  ==  column-major C^T[n][m] = W^T[n][k] A^T[k][m]
+    const rocblas_status st = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_none, (int)n, (int)m,
+                                              (int)k, &alpha, w, in, (int)n, a, in, (int)k, &beta, c,
+                                              rocblas_datatype_f32_r, (int)n, c, rocblas_datatype_f32_r, (int)n,
+                                              rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
+extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim,
+                                                    uint32_t state_dim, uint32_t ffn, int dtype) {
+    const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
+    const size_t f32 = sizeof(float), act = dtype == SFB_BF16 ? 2 : 4;
+    // t (fp32 GEMM output, m x max(n, ffn)); q, k, v (compute dtype); attn (fp32); x1 (fp32);
+    // bf16 path only: xa (activation in compute dtype, m x max(n, ffn))
+    size_t bytes = align256(m * (ffn > n ? ffn : n) * f32) + 3 * align256(m * n * act) + 2 * align256(m * n * f32);
+    if (dtype == SFB_BF16) bytes += align256(m * (ffn > n ? ffn : n) * act);
+    return bytes;
+}
+
+extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x,
+                                         const sfb_layer_weights* wt, int dtype, const sfb_uint2* nn_lut,
+                                         const void* mask, const int32_t* valid_len,
+                                         const sfb_work_item* items, uint32_t n_items, uint32_t n_slots,
+                                         uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
+                                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                         uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t ffn,
+                                         void* workspace, size_t workspace_bytes) {
+    if (!y || !x || !wt || !nn_lut || !workspace) return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    const uint32_t ctx = ctx_blks * block_size;
+    const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
+    if (!m || !n || !ffn || (n & 3u) || (ffn & 3u)) return SFB_ERR_SHAPE;
+    if (workspace_bytes < sfb_encoder_layer_workspace_bytes(batch_dim, ctx, head_dim, state_dim, ffn, dtype) ||
+        ((uintptr_t)workspace & 255u))
+        return SFB_ERR_WORKSPACE;
+    const bool bf = dtype == SFB_BF16;
+    const size_t act = bf ? 2 : 4, wide = ffn > n ? ffn : n;
+    uint8_t* p = (uint8_t*)workspace;
+    float* t = (float*)p;            p += align256(m * wide * sizeof(float));
+    void* q = p;                     p += align256(m * n * act);
+    void* k = p;                     p += align256(m * n * act);
+    void* v = p;                     p += align256(m * n * act);
+    float* attn = (float*)p;         p += align256(m * n * sizeof(float));
+    float* x1 = (float*)p;           p += align256(m * n * sizeof(float));
+    void* xa = bf ? (void*)p : nullptr;
+    const float scale = 1.0f / sqrtf((float)state_dim);
+    int rc;
+#define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
+
+    // Q, K, V projections (+ bias), stored in the compute dtype for the attention kernel
+    const void* xin = x;
+    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x, m * n)); xin = xa; }
+    SFB_TRY(sfb_gemm(stream, t, xin, wt->wq, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, q, dtype, t, wt->bq, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, xin, wt->wk, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, k, dtype, t, wt->bk, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, xin, wt->wv, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, v, dtype, t, wt->bv, nullptr, 0, m, (uint32_t)n));
+
+    // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
+    if (items)
+        SFB_TRY(sfb_fused_attention_scheduled(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, items, n_items,
+                                              n_slots, n_parts, attn_workspace, attn_workspace_bytes, block_size,
+                                              blocks, batch_dim, ctx_blks, head_dim, state_dim, 1, scale));
+    else
+        SFB_TRY(sfb_fused_attention(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, nullptr, block_size,
+                                    blocks, batch_dim, ctx_blks, head_dim, state_dim, 1, ctx_blks + blocks, 1,
+                                    scale));
+
+    // output projection + bias + residual, LayerNorm 1
+    const void* ain = attn;
+    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, attn, m * n)); ain = xa; }
+    SFB_TRY(sfb_gemm(stream, t, ain, wt->wo, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, t, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_layernorm(stream, x1, SFB_F32, nullptr, nullptr, t, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
+
+    // FFN: GEMM, bias + sigmoid-GELU, GEMM, bias + residual, LayerNorm 2
+    const void* fin = x1;
+    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x1, m * n)); fin = xa; }
+    SFB_TRY(sfb_gemm(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+    void* g = bf ? xa : (void*)t;   // activation after GELU, in the compute dtype (in place for fp32)
+    SFB_TRY(sfb_bias_act(stream, g, dtype, t, wt->b1, nullptr, 1, m, ffn));
+    // the second FFN GEMM reads g and must not write over it: fp32 writes into attn's buffer
+    float* t2 = bf ? t : attn;
+    SFB_TRY(sfb_gemm(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn));
+    SFB_TRY(sfb_bias_act(stream, t2, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_layernorm(stream, y, SFB_F32, nullptr, nullptr, t2, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
+#undef SFB_TRY
+    return SFB_OK;
+}

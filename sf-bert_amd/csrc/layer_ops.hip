@@ -1,0 +1,173 @@
+// Encoder-layer ops around the attention path: LayerNorm, bias (+ sigmoid-GELU) (+ residual),
+// residual / position adds, embedding gather, fp32 -> bf16 casts.  All are one pass over HBM.
+// Arithmetic follows the reference CPU functions (layernorm.h:13-38, ewops.h:10-17, 32-43, 276-301,
+// embedding.h:5-12); their GPU twins are cuda_kernels.h:334-372, 459-489, 561-581, 449-457, 526-535,
+// 210-221.
+#include "common.hip.h"
+
+namespace sfb {
+
+// x * 1/(1 + exp(-1.702 x))  (ewops.h:32-43)
+__device__ __forceinline__ float sigmoid_gelu(float x) {
+    return x * (1.0f / (1.0f + exp2_fast(-1.702f * kLog2e * x)));
+}
+
+__device__ __forceinline__ void store_out(float* p, f32x4 v) { *(f32x4*)p = v; }
+__device__ __forceinline__ void store_out(__bf16* p, f32x4 v) {
+    const u32x2 r = {pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
+    *(u32x2*)p = r;
+}
+
+// out[r][c] = act(in[r][c] + bias[c]) + residual[r][c]; cols % 4 == 0.
+template <typename TOut, int ACT>
+__global__ __launch_bounds__(256) void bias_act_kernel(TOut* out, const float* in, const float* bias,
+                                                       const float* residual, uint64_t vecs,
+                                                       uint32_t cols4) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < vecs;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        f32x4 v = ((const f32x4*)in)[i];
+        if (bias) v += ((const f32x4*)bias)[i % cols4];
+        if (ACT == 1) {
+            v.x = sigmoid_gelu(v.x); v.y = sigmoid_gelu(v.y); v.z = sigmoid_gelu(v.z); v.w = sigmoid_gelu(v.w);
+        }
+        if (residual) v += ((const f32x4*)residual)[i];
+        store_out(out + i * 4, v);
+    }
+}
+
+// One wave per row: mean and E[x^2] over the row, rstd = 1/sqrt(E[x^2] - mean^2 + 1e-5)
+// (layernorm.h:16-30), y = ((x - mean) * rstd) * g + b (layernorm.h:34).  state % 4 == 0.
+template <typename TOut>
+__global__ __launch_bounds__(256) void layernorm_kernel(TOut* out, float* mean_out, float* rstd_out,
+                                                        const float* in, const float* gain,
+                                                        const float* bias, uint32_t rows, uint32_t state) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const f32x4* x = (const f32x4*)(in + (size_t)row * state);
+    const uint32_t vecs = state / 4;
+    float sum = 0.f, sq = 0.f;
+    for (uint32_t i = lane; i < vecs; i += 64) {
+        const f32x4 v = x[i];
+        sum += (v.x + v.y) + (v.z + v.w);
+        sq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        sum += __shfl_xor(sum, d);
+        sq += __shfl_xor(sq, d);
+    }
+    const float mean = sum / (float)state;
+    const float var = sq / (float)state - mean * mean;
+    const float rstd = 1.0f / sqrtf(var + 1e-5f);
+    if (lane == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (rstd_out) rstd_out[row] = rstd;
+    }
+    TOut* y = out + (size_t)row * state;
+    for (uint32_t i = lane; i < vecs; i += 64) {
+        const f32x4 v = x[i], g = ((const f32x4*)gain)[i], b = ((const f32x4*)bias)[i];
+        const f32x4 r = {((v.x - mean) * rstd) * g.x + b.x, ((v.y - mean) * rstd) * g.y + b.y,
+                         ((v.z - mean) * rstd) * g.z + b.z, ((v.w - mean) * rstd) * g.w + b.w};
+        store_out(y + i * 4, r);
+    }
+}
+
+// out[b][i] = a[b][i] + m[i]  (ewops.h:276-282: position embedding broadcast over the batch)
+__global__ __launch_bounds__(256) void add_matrix_kernel(float* out, const float* a, const float* m,
+                                                         uint64_t vecs, uint64_t inner4) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < vecs;
+         i += (uint64_t)gridDim.x * blockDim.x)
+        ((f32x4*)out)[i] = ((const f32x4*)a)[i] + ((const f32x4*)m)[i % inner4];
+}
+
+// out[t][:] = table[ids[t]][:] (+ pos[t % seq_len][:])  (embedding.h:5-12, ewops.h:276-282)
+__global__ __launch_bounds__(256) void embedding_kernel(float* out, const float* table, const int32_t* ids,
+                                                        const float* pos, uint64_t tokens, uint32_t state4,
+                                                        uint32_t seq_len, uint32_t vocab) {
+    const uint64_t total = tokens * state4;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t tok = i / state4;
+        const uint32_t c = (uint32_t)(i % state4);
+        uint32_t id = (uint32_t)ids[tok];
+        if (id >= vocab) id = vocab - 1;   // out-of-range ids read the last row instead of faulting
+        f32x4 v = ((const f32x4*)table)[(size_t)id * state4 + c];
+        if (pos) v += ((const f32x4*)pos)[(size_t)(tok % seq_len) * state4 + c];
+        ((f32x4*)out)[i] = v;
+    }
+}
+
+static inline uint32_t grid_for(uint64_t work_items) {
+    const uint64_t blocks = (work_items + 255) / 256;
+    return (uint32_t)(blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks));
+}
+
+static inline int launched() { return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH; }
+
+}  // namespace sfb
+
+using namespace sfb;
+
+extern "C" int sfb_bias_act(sfb_stream_t stream, void* out, int out_dtype, const float* in, const float* bias,
+                            const float* residual, int act, uint64_t rows, uint32_t cols) {
+    if (!out || !in) return SFB_ERR_NULL_POINTER;
+    if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (act != 0 && act != 1) return SFB_ERR_ARGUMENT;
+    if (rows == 0 || cols == 0 || (cols & 3u)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out | (uintptr_t)in | (uintptr_t)bias | (uintptr_t)residual) & 15u) return SFB_ERR_ALIGNMENT;
+    const uint64_t vecs = rows * (cols / 4);
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(grid_for(vecs));
+#define SFB_BA(T, A) bias_act_kernel<T, A><<<grid, 256, 0, s>>>((T*)out, in, bias, residual, vecs, cols / 4)
+    if (out_dtype == SFB_F32) { if (act) SFB_BA(float, 1); else SFB_BA(float, 0); }
+    else { if (act) SFB_BA(__bf16, 1); else SFB_BA(__bf16, 0); }
+#undef SFB_BA
+    return launched();
+}
+
+extern "C" int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, float* mean, float* rstd,
+                             const float* in, const float* gain, const float* bias, uint32_t rows,
+                             uint32_t state) {
+    if (!out || !in || !gain || !bias) return SFB_ERR_NULL_POINTER;
+    if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (rows == 0 || state == 0 || (state & 3u)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out | (uintptr_t)in | (uintptr_t)gain | (uintptr_t)bias) & 15u) return SFB_ERR_ALIGNMENT;
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((rows + 3) / 4);
+    if (out_dtype == SFB_F32)
+        layernorm_kernel<float><<<grid, 256, 0, s>>>((float*)out, mean, rstd, in, gain, bias, rows, state);
+    else
+        layernorm_kernel<__bf16><<<grid, 256, 0, s>>>((__bf16*)out, mean, rstd, in, gain, bias, rows, state);
+    return launched();
+}
+
+extern "C" int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, const float* m, uint32_t dim0,
+                              uint64_t inner) {
+    if (!out || !a || !m) return SFB_ERR_NULL_POINTER;
+    if (dim0 == 0 || inner == 0 || (inner & 3u)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out | (uintptr_t)a | (uintptr_t)m) & 15u) return SFB_ERR_ALIGNMENT;
+    const uint64_t vecs = dim0 * (inner / 4);
+    add_matrix_kernel<<<dim3(grid_for(vecs)), 256, 0, (hipStream_t)stream>>>(out, a, m, vecs, inner / 4);
+    return launched();
+}
+
+extern "C" int sfb_embedding_lookup(sfb_stream_t stream, float* out, const float* table, const int32_t* ids,
+                                    const float* pos, uint64_t tokens, uint32_t state, uint32_t seq_len,
+                                    uint32_t vocab) {
+    if (!out || !table || !ids) return SFB_ERR_NULL_POINTER;
+    if (tokens == 0 || state == 0 || (state & 3u) || vocab == 0 || (pos && seq_len == 0)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out | (uintptr_t)table | (uintptr_t)pos) & 15u) return SFB_ERR_ALIGNMENT;
+    embedding_kernel<<<dim3(grid_for(tokens * (state / 4))), 256, 0, (hipStream_t)stream>>>(
+        out, table, ids, pos, tokens, state / 4, seq_len ? seq_len : 1, vocab);
+    return launched();
+}
+
+extern "C" int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in, uint64_t n) {
+    if (!out || !in) return SFB_ERR_NULL_POINTER;
+    if (n == 0 || (n & 3u)) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out & 7u) || ((uintptr_t)in & 15u)) return SFB_ERR_ALIGNMENT;
+    bias_act_kernel<__bf16, 0><<<dim3(grid_for(n / 4)), 256, 0, (hipStream_t)stream>>>(
+        (__bf16*)out, in, nullptr, nullptr, n / 4, 1);
+    return launched();
+}

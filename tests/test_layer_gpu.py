@@ -1,0 +1,93 @@
+"""Encoder-layer ops, the GEMM seam and the whole layer against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_common import PATTERNS, rel_err
+from sfb import sfb
+
+pytestmark = pytest.mark.gpu
+T = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_layer_ops_match_oracle():
+    rows, state = 515, 768
+    x = orc.fill_normal((rows, state), 1) * 2 + 0.3
+    g = orc.fill_normal((state,), 2) + 1
+    b = orc.fill_normal((state,), 3)
+    want, mean, rstd = orc.layernorm(x, g, b)
+    got, m2, r2 = sfb.layernorm(T(x), T(g), T(b), return_stats=True)
+    assert rel_err(got.cpu().numpy(), want) <= 1e-5
+    assert rel_err(m2.cpu().numpy(), mean) <= 1e-5 and rel_err(r2.cpu().numpy(), rstd) <= 1e-5
+    assert rel_err(sfb.gelu(T(x)).cpu().numpy(), orc.gelu(x)) <= 1e-6
+    assert np.array_equal(sfb.bias(T(x), T(b)).cpu().numpy(), orc.bias(x, b))
+    y = orc.fill_normal((rows, state), 4)
+    assert np.array_equal(sfb.tensor_add_tensor(T(x), T(y)).cpu().numpy(), x + y)
+    fused = sfb.bias_act(T(x), bias=T(b), residual=T(y), act=1).cpu().numpy()
+    assert rel_err(fused, orc.gelu(orc.bias(x, b)) + y) <= 1e-6
+    as_bf16 = sfb.bias_act(T(x), bias=T(b), out_dtype=sfb.BF16).float().cpu().numpy()
+    assert np.array_equal(as_bf16, orc.round_bf16(orc.bias(x, b)))
+    assert np.array_equal(sfb.cast_bf16(T(x)).float().cpu().numpy(), orc.round_bf16(x))
+    ln_bf16 = sfb.layernorm(T(x), T(g), T(b), out_dtype=sfb.BF16).float().cpu().numpy()
+    assert rel_err(ln_bf16, want) <= 4e-3
+
+
+def test_embedding_and_position_add():
+    vocab, state, B, L = 1000, 768, 3, 64
+    table = orc.fill_normal((vocab, state), 5)
+    pos = orc.fill_normal((L, state), 6)
+    ids = orc.fill_uniform_int((B, L), 7, 0, vocab - 1)
+    got = sfb.embedding_lookup(T(table), T(ids), T(pos)).cpu().numpy()
+    assert np.array_equal(got, table[ids] + pos[None])
+    assert np.array_equal(sfb.embedding_lookup(T(table), T(ids)).cpu().numpy(), table[ids])
+    x = orc.fill_normal((B, L, state), 8)
+    assert np.array_equal(sfb.tensor_add_matrix(T(x), T(pos)).cpu().numpy(), x + pos[None])
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_gemm_matches_oracle(bf16):
+    m, k, n = 200, 768, 3072
+    A = orc.fill_normal((m, k), 9)
+    W = orc.fill_normal((k, n), 10, 0.02)
+    if bf16:
+        A, W = orc.round_bf16(A), orc.round_bf16(W)
+    want = orc.sgemm(A, W, nthreads=16)
+    a, w = T(A), T(W)
+    if bf16:
+        a, w = a.to(torch.bfloat16), w.to(torch.bfloat16)
+    got = sfb.gemm(a, w).cpu().numpy()
+    assert rel_err(got, want) <= 1e-5
+    want64 = A.astype(np.float64) @ W.astype(np.float64)
+    assert rel_err(got, want64) <= 1e-5
+
+
+def layer_weights(n, ffn, seed):
+    shapes = [("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)), ("w2", (ffn, n)),
+              ("bq", (n,)), ("bk", (n,)), ("bv", (n,)), ("bo", (n,)), ("b1", (ffn,)), ("b2", (n,)),
+              ("ln1_g", (n,)), ("ln1_b", (n,)), ("ln2_g", (n,)), ("ln2_b", (n,))]
+    w = {k: orc.fill_normal(s, seed + i, 0.02) for i, (k, s) in enumerate(shapes)}
+    w["ln1_g"] = w["ln1_g"] + 1
+    w["ln2_g"] = w["ln2_g"] + 1
+    return w
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("max_blocks", [0, 4])
+def test_encoder_layer_matches_oracle(bf16, max_blocks):
+    # BERT-base widths (hidden 768, 12 heads, d 64, FFN 3072), BigBird attention, short sequence
+    B, L, H, d, ffn, bs = 2, 1024, 12, 64, 3072, 64
+    n, nb = H * d, L // bs
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    w = layer_weights(n, ffn, 100)
+    x = orc.fill_normal((B * L, n), 300)
+    want = orc.encoder_layer(x, w, luts["nn_lut"], B, L, H, d, ffn, bs, luts["blocks"], operands_bf16=bf16,
+                             nthreads=16)
+    layer = sfb.EncoderLayer({k: T(v) for k, v in w.items()}, luts, bs, H, d, ffn,
+                             dtype=sfb.BF16 if bf16 else sfb.F32, max_blocks=max_blocks)
+    for _ in range(2):
+        got = layer.forward(T(x), B, L).cpu().numpy()
+        torch.cuda.synchronize()
+        err = rel_err(got, want)
+        print("layer rel err", err)
+        assert err <= (1e-2 if bf16 else 1e-4)
