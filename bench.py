@@ -42,23 +42,89 @@ def make_layout(sfb, pattern, nb):
     return sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234))
 
 
-def cpu_baseline(luts, B, H, L, d, bs, bf16, flops_per_bh):
-    """Times the CPU oracle (a port of the reference CPU path) on one batch element of the workload."""
+def cpu_baseline(luts, B, H, L, d, bs, bf16, flops):
+    """Times the CPU oracle (a port of the reference CPU path) on the whole workload, repeated until
+    about ten seconds of wall time have been spent on this host's cores."""
     import numpy as np
     import oracle_lib as orc
     threads = max(1, min(16, os.cpu_count() or 1))
-    sample_b = 1
-    Q, K, V = (orc.fill_normal((sample_b, L, H, d), 900 + i) for i in range(3))
+    Q, K, V = (orc.fill_normal((B, L, H, d), 900 + i) for i in range(3))
     if bf16:
         Q, K, V = (orc.round_bf16(x) for x in (Q, K, V))
-    t0 = time.perf_counter()
-    orc.attention(Q, K, V, luts["nn_lut"], bs, 1.0 / np.sqrt(d), nthreads=threads)
-    dt = time.perf_counter() - t0
-    tflops = flops_per_bh * sample_b * H / dt / 1e12
-    return {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": "CPU oracle (fp32 port of matmul.h/ewops.h loops, OpenMP over block-rows) on "
-                      "batch 1 of %d of the same workload: %.2f s, scaled by flops" % (B, dt),
-            "seconds": dt, "ms_per_call_extrapolated": dt * B * 1e3}
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 30 and time.perf_counter() - t_begin < 10.0:
+        t0 = time.perf_counter()
+        orc.attention(Q, K, V, luts["nn_lut"], bs, 1.0 / np.sqrt(d), nthreads=threads)
+        times.append(time.perf_counter() - t0)
+    dt = sum(times) / len(times)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "CPU oracle (fp32 port of the matmul.h/ewops.h loops over nonzero blocks, OpenMP over "
+                      "block-rows) on the full workload, %d calls, mean %.3f s per call" % (len(times), dt),
+            "ms_per_call": dt * 1e3}
+
+
+def _time(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
+    """sdd -> masked softmax -> dsd with S and P in HBM (bf16 storage for bf16 inputs, else fp32)."""
+    B, L, H, d = q.shape
+    nb = L // bs
+    store = torch.bfloat16 if bf16 else torch.float32
+    nt, nn = sfb.to_device(luts["nt_lut"]), sfb.to_device(luts["nn_lut"])
+    S = torch.empty((B, H, blocks, bs, bs), device="cuda", dtype=store)
+    P = torch.empty_like(S)
+    O = torch.empty((B, L, H, d), device="cuda", dtype=torch.float32)
+
+    def trio():
+        sfb.bst_sgemm_nt(nt, q, k, bs, blocks, c=S)
+        sfb.BlocksparseMaskedSoftmax(nn, None, S, nb, scale, y=P)
+        sfb.bst_sgemm_xn(nn, P, v, nb, c=O)
+
+    ms = _time(torch, trio, 200, 50)
+    parts = {"sdd_ms": _time(torch, lambda: sfb.bst_sgemm_nt(nt, q, k, bs, blocks, c=S), 200, 20),
+             "softmax_ms": _time(torch, lambda: sfb.BlocksparseMaskedSoftmax(nn, None, S, nb, scale, y=P), 200, 20),
+             "dsd_ms": _time(torch, lambda: sfb.bst_sgemm_xn(nn, P, v, nb, c=O), 200, 20)}
+    return dict(ms_per_call=ms, fused_speedup=ms / fused_ms, sp_storage="bf16" if bf16 else "f32", **parts)
+
+
+def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
+    """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
+    B, L, ffn = 8, 4096, 3072
+    n = H * d
+    torch.manual_seed(1)
+    w = {}
+    for name, shape in (("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)),
+                        ("w2", (ffn, n))):
+        w[name] = torch.randn(shape, device="cuda") * 0.02
+    for name, size in (("bq", n), ("bk", n), ("bv", n), ("bo", n), ("b1", ffn), ("b2", n), ("ln1_b", n),
+                       ("ln2_b", n)):
+        w[name] = torch.zeros(size, device="cuda")
+    w["ln1_g"] = torch.ones(n, device="cuda")
+    w["ln2_g"] = torch.ones(n, device="cuda")
+    ids = torch.randint(0, 30522, (B, L), device="cuda", dtype=torch.int32)
+    tok = torch.randn((30522, n), device="cuda") * 0.02
+    pos = torch.randn((L, n), device="cuda") * 0.02
+    x = sfb.embedding_lookup(tok, ids, pos).reshape(B * L, n)
+    out = {"shape": "B8 L4096 hidden 768 heads 12 ffn 3072, BigBird block 64", "gemm_flops": 2.0 * B * L * (4 * n * n + 2 * n * ffn)}
+    y = torch.empty_like(x)
+    for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
+        layer = sfb.EncoderLayer(w, luts, bs, H, d, ffn, dtype=code, max_blocks=max_blocks)
+        out["ms_per_layer_" + name] = _time(torch, lambda: layer.forward(x, B, L, out=y), 20, 5)
+        assert torch.isfinite(y).all()
+        del layer
+    return out
 
 
 def main():
@@ -69,6 +135,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["bf16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-extras", action="store_true",
+                    help="only the fused-attention line: no unfused comparison, no encoder-layer timing")
     ap.add_argument("--max-blocks", type=int, default=16,
                     help="split block-rows longer than this many key blocks (0 = one work-group per row)")
     args = ap.parse_args()
@@ -149,8 +217,12 @@ def main():
                      "hbm_achieved_GBs": algo_bytes / (kernel_ms * 1e-3) / 1e9,
                      "hbm_frac": algo_bytes / (kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
     }
+    if not args.skip_extras:
+        result["unfused"] = time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
+        if args.workload == "c4":
+            result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, args.max_blocks)
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops_per_bh)
+        result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops)
     print(json.dumps(result))
 
 
