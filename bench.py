@@ -64,6 +64,19 @@ def cpu_baseline(luts, B, H, L, d, bs, bf16, flops):
             "ms_per_call": dt * 1e3}
 
 
+def read_traffic(workload, dtype):
+    """HBM bytes per launch of the fused kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+    scaled by a plain copy kernel; recorded in profiles/ (null when no measurement is on file)."""
+    path = os.path.join(ROOT, "profiles", "fused_attention_%s_%s_hbm_traffic.txt" % (workload, dtype))
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def _time(torch, fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -135,8 +148,13 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--dtype", default=None, choices=["bf16", "f32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (reference kernel for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the fused-attention line: no unfused comparison, no encoder-layer timing")
+    ap.add_argument("--heavy", type=int, default=-1,
+                    help="override the schedule's number of leading items launched for all heads first")
     ap.add_argument("--max-blocks", type=int, default=16,
                     help="split block-rows longer than this many key blocks (0 = one work-group per row)")
     args = ap.parse_args()
@@ -172,6 +190,8 @@ def main():
 
     if args.max_blocks > 0:
         sched = sfb.build_schedule(luts["nn_lut"], nb, args.max_blocks)
+        if args.heavy >= 0:
+            sched["n_heavy"] = min(args.heavy, sched["n_items"] - 1)
         items = sfb.to_device(sched["items"])
         workspace = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256),
                                 dtype=torch.uint8, device="cuda")
@@ -181,6 +201,13 @@ def main():
     else:
         def step():
             sfb.fused_attention(q, k, v, nn_lut, bs, blocks, scale, row_order=order, out=out)
+
+    if args.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     for _ in range(args.warmup):
         step()
@@ -197,6 +224,7 @@ def main():
     ms_per_step = wall_ms / args.steps
     assert torch.isfinite(out).all()
 
+    traffic = read_traffic(args.workload, dtype)
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     achieved = flops / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dtype]
@@ -210,7 +238,7 @@ def main():
                                (args.workload, pattern, B, H, L, d, bs, blocks, dtype)},
         "ms_per_attention_call": kernel_ms,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-                     "frac": achieved / peak, "traffic": None,
+                     "frac": achieved / peak, "traffic": traffic,
                      "kernel": "fused_attention_%s_kernel<%d,%d>" % (dtype if bf16 else "f32", bs, d),
                      "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms,
                      "hbm_algorithmic_bytes_per_launch": algo_bytes,

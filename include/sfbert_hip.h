@@ -114,9 +114,11 @@ typedef struct {
     uint32_t reserved;
 } sfb_work_item;
 /* items may be NULL to query the counts; otherwise it must hold *n_items entries as returned by a
- * query call.  n_slots = number of split rows, n_parts = total chunks of split rows. */
-int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_slots, uint32_t* n_parts,
-                       const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
+ * query call.  n_slots = number of split rows, n_parts = total chunks of split rows, n_heavy = number
+ * of leading items with at least twice the median number of key blocks (launched for all heads
+ * before the rest; always < n_items). */
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
 /* Bytes of the [dev] workspace a scheduled launch needs: arrival counters + partial records.  The
  * workspace must be zero-filled once before its first use; launches leave the counters at zero. */
 size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
@@ -150,7 +152,7 @@ int sfb_fused_attention(sfb_stream_t stream, const void* q, const void* k, const
 int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k, const void* v,
                                   float* o, int in_dtype, const sfb_uint2* nn_lut, const void* mask,
                                   const int32_t* valid_len, const sfb_work_item* items,
-                                  uint32_t n_items, uint32_t n_slots, uint32_t n_parts,
+                                  uint32_t n_items, uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts,
                                   void* workspace, size_t workspace_bytes, uint32_t block_size,
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
@@ -249,8 +251,8 @@ size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint3
  * workspace [dev] 256-byte aligned, sfb_encoder_layer_workspace_bytes() bytes. */
 int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
                               int dtype, const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
-                              const sfb_work_item* items, uint32_t n_items, uint32_t n_slots, uint32_t n_parts,
-                              void* attn_workspace, size_t attn_workspace_bytes, uint32_t block_size,
+                              const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                              uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes, uint32_t block_size,
                               uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
                               uint32_t state_dim, uint32_t ffn, void* workspace, size_t workspace_bytes);
 

@@ -176,14 +176,14 @@ WORK_ITEM_DTYPE = np.dtype([(n, np.uint32) for n in
 def build_schedule(nn_lut, nb, max_blocks=16):
     """Work items of a scheduled fused launch: dict(items structured array, n_slots, n_parts)."""
     nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
-    n_items, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
-    _check(lib.sfb_build_schedule(None, C.byref(n_items), C.byref(n_slots), C.byref(n_parts),
+    n_items, n_heavy, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    _check(lib.sfb_build_schedule(None, C.byref(n_items), C.byref(n_heavy), C.byref(n_slots), C.byref(n_parts),
                                   _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
     items = np.zeros(n_items.value, WORK_ITEM_DTYPE)
-    _check(lib.sfb_build_schedule(_np(items), C.byref(n_items), C.byref(n_slots), C.byref(n_parts),
-                                  _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
-    return Luts(items=items, n_items=int(n_items.value), n_slots=int(n_slots.value),
-                n_parts=int(n_parts.value))
+    _check(lib.sfb_build_schedule(_np(items), C.byref(n_items), C.byref(n_heavy), C.byref(n_slots),
+                                  C.byref(n_parts), _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
+    return Luts(items=items, n_items=int(n_items.value), n_heavy=int(n_heavy.value),
+                n_slots=int(n_slots.value), n_parts=int(n_parts.value))
 
 
 def schedule_workspace_bytes(sched, batch, heads, block_size, d):
@@ -256,7 +256,8 @@ def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_si
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _check(lib.sfb_fused_attention_scheduled(
         _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dtype_code(q), _dev(nn_lut), _dev(mask),
-        _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_slots"]),
+        _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]),
+        C.c_uint32(sched["n_slots"]),
         C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes), C.c_uint32(block_size),
         C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d),
         C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled")
@@ -459,7 +460,7 @@ class EncoderLayer:
         _check(lib.sfb_encoder_layer_forward(
             _stream(), _dev(out), _dev(x), C.byref(self.c_weights), self.dtype, _dev(self.nn_lut), _dev(mask),
             _dev(valid_len), _dev(self.items), C.c_uint32(s["n_items"] if s else 0),
-            C.c_uint32(s["n_slots"] if s else 0), C.c_uint32(s["n_parts"] if s else 0), _dev(aws),
+            C.c_uint32(s["n_heavy"] if s else 0), C.c_uint32(s["n_slots"] if s else 0), C.c_uint32(s["n_parts"] if s else 0), _dev(aws),
             C.c_size_t(aws.numel() if aws is not None else 0), C.c_uint32(self.bs), C.c_uint32(self.luts["blocks"]),
             C.c_uint32(B), C.c_uint32(L // self.bs), C.c_uint32(self.heads), C.c_uint32(self.d),
             C.c_uint32(self.ffn), _dev(ws), C.c_size_t(ws.numel())), "sfb_encoder_layer_forward")

@@ -50,25 +50,38 @@ __device__ __forceinline__ size_t token_offset(uint32_t b, uint32_t token, uint3
     return (((size_t)b * L + token) * H + h) * (size_t)d;
 }
 
-// Work-group id -> (batch*head index, rank of the block-row in the launch order).
+// Work-group id -> (batch*head index, rank of the work item in the launch order).
 // Hardware deals consecutive work-group ids round-robin to the 8 XCDs, each with its own L2.  All
-// block-rows of one (batch, head) are given ids of the same residue mod 8, so the K/V blocks they
-// share (window neighbours, global and random blocks) are fetched into one L2 only.  Ranks are the
-// slow index: rank 0 of every head is dispatched before rank 1 of any, which lets the caller put the
-// longest block-rows first.
+// work items of one (batch, head) are given ids of the same residue mod 8, so the K/V blocks they
+// share (window neighbours, global and random blocks) are fetched into one L2 only.  Within an XCD
+// the ranks of one (batch, head) are consecutive and the heads follow one another, so that only a
+// couple of heads' K and V (about 1 MiB each at L = 4096) are live in the 4 MiB L2 at any time.
 struct WorkId {
     uint32_t bh;
     uint32_t rank;
     bool valid;
 };
 
-__device__ __forceinline__ WorkId decode_work(uint32_t wg, uint32_t num_bh, uint32_t groups) {
+// The first `heavy` ranks (items much longer than the rest, sorted to the front) are the exception:
+// they are issued for all heads before anything else, so that they overlap with the short items
+// instead of forming the tail of the launch.
+__device__ __forceinline__ WorkId decode_work(uint32_t wg, uint32_t num_bh, uint32_t ranks,
+                                              uint32_t heavy = 0) {
     constexpr uint32_t kXcds = 8;
-    uint32_t xcd = wg % kXcds;
+    const uint32_t xcd = wg % kXcds;
     uint32_t q = wg / kXcds;
-    uint32_t group = q % groups;
+    const uint32_t groups = (num_bh + kXcds - 1) / kXcds;
     WorkId w;
-    w.rank = q / groups;
+    uint32_t group;
+    if (q < heavy * groups) {
+        w.rank = q / groups;
+        group = q % groups;
+    } else {
+        q -= heavy * groups;
+        const uint32_t light = ranks - heavy;
+        w.rank = heavy + q % light;
+        group = q / light;
+    }
     w.bh = group * kXcds + xcd;
     w.valid = w.bh < num_bh;
     return w;

@@ -285,9 +285,9 @@ int sfb_build_row_order(uint32_t* row_order, const sfb_uint2* nn_lut, int nb) {
     return SFB_OK;
 }
 
-int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_slots, uint32_t* n_parts,
-                       const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
-    if (!n_items || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
+    if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
     if (nb <= 0) return SFB_ERR_SHAPE;
     if (max_blocks == 0) return SFB_ERR_ARGUMENT;
     std::vector<sfb_work_item> all;
@@ -315,6 +315,11 @@ int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_slot
         if (*n_items < all.size()) return SFB_ERR_ARGUMENT;
         std::copy(all.begin(), all.end(), items);
     }
+    // items at least twice as long as the median item are "heavy"
+    const uint32_t median = all[all.size() / 2].count;
+    uint32_t heavy = 0;
+    while (heavy + 1 < all.size() && all[heavy].count >= 2 * median && all[heavy].count > median) ++heavy;
+    *n_heavy = heavy;
     *n_items = (uint32_t)all.size();
     *n_slots = slots;
     *n_parts = parts;

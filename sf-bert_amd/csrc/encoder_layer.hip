@@ -63,8 +63,8 @@ extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t
 extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x,
                                          const sfb_layer_weights* wt, int dtype, const sfb_uint2* nn_lut,
                                          const void* mask, const int32_t* valid_len,
-                                         const sfb_work_item* items, uint32_t n_items, uint32_t n_slots,
-                                         uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
+                                         const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                                         uint32_t n_slots, uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
                                          uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                          uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t ffn,
                                          void* workspace, size_t workspace_bytes) {
@@ -103,7 +103,7 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
     if (items)
         SFB_TRY(sfb_fused_attention_scheduled(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, items, n_items,
-                                              n_slots, n_parts, attn_workspace, attn_workspace_bytes, block_size,
+                                              n_heavy, n_slots, n_parts, attn_workspace, attn_workspace_bytes, block_size,
                                               blocks, batch_dim, ctx_blks, head_dim, state_dim, 1, scale));
     else
         SFB_TRY(sfb_fused_attention(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, nullptr, block_size,

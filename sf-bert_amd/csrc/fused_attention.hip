@@ -36,6 +36,8 @@ struct FusedParams {
     uint32_t lut_stride;            // entries between heads' LUTs (0 = shared)
     uint32_t mask_stride;           // words between heads' masks (0 = shared)
     uint32_t groups;                // ceil(batch*heads / 8)
+    uint32_t ranks;                 // work items per (batch, head)
+    uint32_t heavy;                 // leading items issued for all heads first
     float scale_log2e;
     float slack;                    // raw-score distance a block maximum may exceed the reference maximum
 };
@@ -51,7 +53,7 @@ struct RowWork {
 
 __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
     RowWork w;
-    const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.groups);
+    const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.ranks, p.heavy);
     w.valid = id.valid;
     w.bh = id.bh;
     w.b = id.bh / p.heads;
@@ -243,18 +245,44 @@ __device__ __forceinline__ void store_zero_row(float* o_row, uint32_t half) {
 // ------------------------------------------------------------------------------------------------
 // bf16 inputs, fp32 accumulation: v_mfma_f32_32x32x16_bf16
 // ------------------------------------------------------------------------------------------------
-// Two LDS buffers (K tile + transposed V tile each), one barrier per key block: block j+1 is fetched
-// into registers while block j is multiplied, and written to the other buffer afterwards.
-template <int BS, int D>
+// Software pipeline over the key blocks of the row.  In iteration j a wave
+//   * writes K(j+2) and V(j+1), fetched from memory during iteration j-1, into the free LDS buffers
+//     and issues the fetches of K(j+3) and V(j+2);
+//   * multiplies S_next = K(j+1) . Q^T on MFMA while the VALU finds the row maximum of S_cur (block j);
+//   * exponentiates S_cur in four chunks, each chunk's probabilities feeding the V(j)^T . P^T MFMAs
+//     while the next chunk is exponentiated.
+// K and V tiles are double-buffered in LDS with K running one block ahead of V; one barrier per key
+// block.  Block indices past the end of the row are clamped: the extra tiles are loaded and
+// multiplied but never used.
+template <int KT, int NO>
+__device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], int u, float c,
+                                          float mc, float& sum0, float& sum1) {
+    const int kt = u / 2, i0 = (u % 2) * 8;
+    const float p0 = exp2_fast(__builtin_fmaf(s[kt][i0 + 0], c, -mc));
+    const float p1 = exp2_fast(__builtin_fmaf(s[kt][i0 + 1], c, -mc));
+    const float p2 = exp2_fast(__builtin_fmaf(s[kt][i0 + 2], c, -mc));
+    const float p3 = exp2_fast(__builtin_fmaf(s[kt][i0 + 3], c, -mc));
+    const float p4 = exp2_fast(__builtin_fmaf(s[kt][i0 + 4], c, -mc));
+    const float p5 = exp2_fast(__builtin_fmaf(s[kt][i0 + 5], c, -mc));
+    const float p6 = exp2_fast(__builtin_fmaf(s[kt][i0 + 6], c, -mc));
+    const float p7 = exp2_fast(__builtin_fmaf(s[kt][i0 + 7], c, -mc));
+    const uint32_t a = pack_bf16(p0, p1), b = pack_bf16(p2, p3), d = pack_bf16(p4, p5), e = pack_bf16(p6, p7);
+    pk[u * 4 + 0] = a; pk[u * 4 + 1] = b; pk[u * 4 + 2] = d; pk[u * 4 + 3] = e;
+    sum0 = dot2_bf16_ones(a, sum0);
+    sum1 = dot2_bf16_ones(b, sum1);
+    sum0 = dot2_bf16_ones(d, sum0);
+    sum1 = dot2_bf16_ones(e, sum1);
+}
+
+template <int BS, int D, bool MASKED>
 __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
     using T = Bf16Tiles<BS, D>;
     constexpr int KT = BS / 32;      // 32-key tiles per block
     constexpr int NO = D / 32;       // 32-column tiles of O
     constexpr int KS = D / 16;       // MFMA k-steps over the head dimension
     constexpr int PU = BS / 16;      // MFMA k-steps over the keys of a block
-    constexpr int BUF = T::K_BYTES + T::V_BYTES;
 
-    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * BUF];
+    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * T::K_BYTES + 2 * T::V_BYTES];
 
     const RowWork w = decode_row_work(p);
     if (!w.valid) return;
@@ -282,42 +310,13 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     bf16x8 qf[KS];
     T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
 
-    typename T::KRegs gk;
-    typename T::VRegs gv;
-
-    f32x16 o_acc[NO];
-#pragma unroll
-    for (int n = 0; n < NO; ++n)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
-    RowState st = {kMaxSeed, kMaxSeed, 0.f};
-    const float c = p.scale_log2e, slack = p.slack;
-
-    sfb_uint2 entry = lut[lut_off];
-    {
-        const size_t base = token_offset(w.b, entry.y * BS, w.h, L, p.heads, D);
-        T::fetch_k(gk, K, base, row_stride, t);
-        T::fetch_v(gv, V, base, row_stride, t);
-        T::stage_k(smem, gk, t);
-        T::stage_v(smem + T::K_BYTES, gv, t);
-    }
-    __syncthreads();
-
-    for (uint32_t j = 0; j < count; ++j) {
-        const uint32_t cur = j & 1;
-        const sfb_uint2 here = entry;
-        const bool more = (j + 1 < count);
-        if (more) {
-            entry = lut[lut_off + j + 1];
-            const size_t base = token_offset(w.b, entry.y * BS, w.h, L, p.heads, D);
-            T::fetch_k(gk, K, base, row_stride, t);
-            T::fetch_v(gv, V, base, row_stride, t);
-        }
-        const uint8_t* k_lds = smem + cur * BUF;
-        const uint8_t* v_lds = k_lds + T::K_BYTES;
-
-        // S^T = K . Q^T
-        f32x16 s[KT];
+    // element offset of key block number j of this item (clamped to the last one)
+    const size_t bh_base = token_offset(w.b, 0, w.h, L, p.heads, D);
+    auto tile_base = [&](uint32_t j) -> size_t {
+        const uint32_t jj = j < count ? j : count - 1;
+        return bh_base + (size_t)(lut[lut_off + jj].y * BS) * row_stride;
+    };
+    auto score_tile = [&](f32x16 (&s)[KT], const uint8_t* k_lds) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -328,31 +327,93 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
             for (int kt = 0; kt < KT; ++kt)
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_lds, kt, ks, qn, half), qf[ks],
                                                                 s[kt], 0, 0, 0);
+    };
 
-        const int limit = valid - (int)(here.y * BS);
-        const bool masked = (mask != nullptr) || (limit < BS);
-        uint64_t keep = ~0ull;
-        if (masked) keep = load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit);
+    // two register sets of fetched tiles: each is written to LDS two iterations after it was requested
+    typename T::KRegs gk0, gk1;
+    typename T::VRegs gv0, gv1;
+    uint8_t* const kb = smem;
+    uint8_t* const vb = smem + 2 * T::K_BYTES;
+
+    f32x16 o_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
+    RowState st = {kMaxSeed, kMaxSeed, 0.f};
+    const float c = p.scale_log2e, slack = p.slack;
+
+    // prologue: K(0), V(0) and K(1) into LDS, S_next = scores of block 0;
+    // set 0 holds K(2), V(1) and set 1 holds K(3), V(2), all in flight
+    f32x16 s_next[KT];
+    T::fetch_k(gk0, K, tile_base(0), row_stride, t);
+    T::fetch_v(gv0, V, tile_base(0), row_stride, t);
+    T::fetch_k(gk1, K, tile_base(1), row_stride, t);
+    T::stage_k(kb, gk0, t);
+    T::stage_v(vb, gv0, t);
+    T::stage_k(kb + T::K_BYTES, gk1, t);
+    T::fetch_k(gk0, K, tile_base(2), row_stride, t);
+    T::fetch_v(gv0, V, tile_base(1), row_stride, t);
+    T::fetch_k(gk1, K, tile_base(3), row_stride, t);
+    T::fetch_v(gv1, V, tile_base(2), row_stride, t);
+    __syncthreads();
+    score_tile(s_next, kb);
+    __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
+
+    auto iteration = [&](uint32_t j, typename T::KRegs& gk, typename T::VRegs& gv) {
+        const uint32_t par = j & 1;
+        uint8_t* const k_write = kb + par * T::K_BYTES;             // K(j+2) replaces K(j)
+        const uint8_t* const k_read = kb + (par ^ 1) * T::K_BYTES;  // K(j+1)
+        uint8_t* const v_write = vb + (par ^ 1) * T::V_BYTES;       // V(j+1) replaces V(j-1)
+        const uint8_t* const v_read = vb + par * T::V_BYTES;        // V(j)
+
+        T::stage_k(k_write, gk, t);
+        T::stage_v(v_write, gv, t);
+        T::fetch_k(gk, K, tile_base(j + 4), row_stride, t);
+        T::fetch_v(gv, V, tile_base(j + 3), row_stride, t);
+
+        f32x16 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) s[kt] = s_next[kt];
+        score_tile(s_next, k_read);
+
+        if (MASKED) {
+            const sfb_uint2 here = lut[lut_off + j];
+            const int limit = valid - (int)(here.y * BS);
+            if ((mask != nullptr) || (limit < BS))
+                apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit), half);
+        }
+        const float mloc = block_row_max<KT>(s);
+        st.m_true = fmaxf(st.m_true, mloc);
+        if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
+            const float m_new = fmaxf(st.m_used, mloc);
+            const float alpha = exp2_fast((st.m_used - m_new) * c);
+            st.m_used = m_new;
+            st.l *= alpha;
+#pragma unroll
+            for (int n = 0; n < NO; ++n) o_acc[n] *= alpha;
+        }
+        const float mc = st.m_used * c;
+        float sum0 = 0.f, sum1 = 0.f;
         uint32_t pk[KT * 8];
-        softmax_block<KT, NO, true>(s, pk, o_acc, st, c, slack, masked, keep, half);
-
-        // O^T += V^T . P^T
+        exp_chunk<KT, NO>(s, pk, 0, c, mc, sum0, sum1);
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
+            if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
             const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
             const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
             for (int mt = 0; mt < NO; ++mt)
-                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(v_lds, mt, u, qn, half), bfrag,
+                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(v_read, mt, u, qn, half), bfrag,
                                                                     o_acc[mt], 0, 0, 0);
         }
-
-        if (more) {
-            uint8_t* nxt = smem + (cur ^ 1) * BUF;
-            T::stage_k(nxt, gk, t);
-            T::stage_v(nxt + T::K_BYTES, gv, t);
-        }
+        st.l += sum0 + sum1;
         __syncthreads();
+    };
+
+    for (uint32_t j = 0; j < count; j += 2) {
+        iteration(j, gk0, gv0);
+        if (j + 1 < count) iteration(j + 1, gk1, gv1);
     }
 
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
@@ -465,11 +526,15 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedPar
 }
 
 template <int BS, int D>
-static int launch_fused(hipStream_t stream, const FusedParams& p, int in_dtype, uint32_t ranks) {
+static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
+    p.ranks = ranks;
     const uint32_t grid = p.groups * 8u * ranks;
-    if (in_dtype == SFB_BF16)
-        fused_attention_bf16_kernel<BS, D><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-    else
+    if (in_dtype == SFB_BF16) {
+        if (p.mask || p.valid_len)
+            fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+        else
+            fused_attention_bf16_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+    } else
         fused_attention_f32_kernel<BS, D><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
     return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
 }
@@ -501,7 +566,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.q = q; p.k = k; p.v = v; p.o = o;
     p.nn_lut = nn_lut; p.mask = mask; p.valid_len = valid_len;
     p.row_order = nullptr; p.items = nullptr; p.counters = nullptr; p.partials = nullptr;
-    p.n_slots = 0; p.n_parts = 0;
+    p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
@@ -545,8 +610,8 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
                                              const void* v, float* o, int in_dtype,
                                              const sfb_uint2* nn_lut, const void* mask,
                                              const int32_t* valid_len, const sfb_work_item* items,
-                                             uint32_t n_items, uint32_t n_slots, uint32_t n_parts,
-                                             void* workspace, size_t workspace_bytes,
+                                             uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                             uint32_t n_parts, void* workspace, size_t workspace_bytes,
                                              uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                              uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                              uint32_t mask_heads, float scale) {
@@ -555,7 +620,7 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
                                 head_dim, state_dim, 1, ctx_blks + blocks, mask_heads, scale);
     if (rc != SFB_OK) return rc;
     if (!items) return SFB_ERR_NULL_POINTER;
-    if (n_items == 0) return SFB_ERR_SHAPE;
+    if (n_items == 0 || n_heavy >= n_items) return SFB_ERR_SHAPE;
     if ((uint64_t)batch_dim * head_dim * n_items > 0x7fffffffull / 64) return SFB_ERR_SHAPE;
     const size_t need = sfb_schedule_workspace_bytes(n_slots, n_parts, batch_dim, head_dim, block_size, state_dim);
     if (n_parts > 0 && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
@@ -564,7 +629,7 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
     fill_common(p, q, k, v, o, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
                 1, ctx_blks + blocks, mask_heads, scale);
     p.items = items;
-    p.n_slots = n_slots; p.n_parts = n_parts;
+    p.n_slots = n_slots; p.n_parts = n_parts; p.heavy = n_heavy;
     const size_t bh = (size_t)batch_dim * head_dim;
     const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
     p.counters = (uint32_t*)workspace;

@@ -73,14 +73,11 @@ struct Bf16Tiles {
             for (int dd = 0; dd < 8; ++dd) {
                 const uint32_t x0 = r.g[ii][0][dd / 2], x1 = r.g[ii][1][dd / 2];
                 const uint32_t x2 = r.g[ii][2][dd / 2], x3 = r.g[ii][3][dd / 2];
+                // byte select over {second, first}: low halves (even column) or high halves (odd column)
+                const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
                 u32x2 out;
-                if (dd & 1) {
-                    out.x = (x0 >> 16) | (x1 & 0xffff0000u);
-                    out.y = (x2 >> 16) | (x3 & 0xffff0000u);
-                } else {
-                    out.x = (x0 & 0xffffu) | (x1 << 16);
-                    out.y = (x2 & 0xffffu) | (x3 << 16);
-                }
+                out.x = __builtin_amdgcn_perm(x1, x0, sel);
+                out.y = __builtin_amdgcn_perm(x3, x2, sel);
                 *(u32x2*)(v_lds + (c * 8 + dd) * V_STRIDE + pos) = out;
             }
         }

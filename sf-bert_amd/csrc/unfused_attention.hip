@@ -200,7 +200,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int LDS_BYTES = kBf16 ? TB::V_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(16))) uint8_t smem[LDS_BYTES];
 
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.groups);
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
     const uint32_t r = p.nb_c - 1 - work.rank;   // long rows of causal layouts first (blocksparse.h:746-748)
@@ -293,7 +293,7 @@ struct SddSoftmaxParams {
 template <int BS, int D, typename TIn, typename TOut>
 __global__ __launch_bounds__(BS * 2, 2) void sdd_softmax_kernel(SddSoftmaxParams p) {
     constexpr int KT = BS / 32;
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.groups);
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
     const uint32_t r = p.nb - 1 - work.rank;

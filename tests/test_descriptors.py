@@ -121,6 +121,9 @@ def test_schedule_covers_every_block_once(max_blocks):
     items = sched["items"]
     counts = lay.sum(axis=1)
     assert sched["n_items"] == len(items)
+    median = items["count"][len(items) // 2]
+    heavy = (items["count"] >= 2 * median) & (items["count"] > median)
+    assert sched["n_heavy"] == min(int(heavy.sum()), len(items) - 1)
     assert (items["count"] <= max(max_blocks, 1)).all()
     assert (np.diff(items["count"].astype(np.int64)) <= 0).all()  # longest first
     split_rows = [r for r in range(64) if counts[r] > max_blocks]
