@@ -39,6 +39,17 @@ def build(verbose=True, jobs=8):
     subprocess.check_call(link + extra)
     if verbose:
         print("built", LIB)
+    # C++ host program that drives the library through the reference-named launchers (run by the GPU tests)
+    host = os.path.join(HERE, "host")
+    exe = os.path.join(host, "attention_host_test")
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-w", "-o", exe,
+                           os.path.join(host, "attention_host_test.cpp"), "-L" + HERE, "-lsfbert_hip",
+                           "-Wl,-rpath,$ORIGIN/.."])
+    # the same headers must also be usable from a translation unit compiled by the plain host compiler
+    subprocess.check_call(["g++", "-std=c++17", "-fsyntax-only", "-I/opt/rocm/include", "-x", "c++",
+                           os.path.join(host, "host_headers_check.cpp")])
+    if verbose:
+        print("built", exe)
     return LIB
 
 

@@ -1,0 +1,144 @@
+// C++ host program in the shape of the reference's *_fusion_test.cu mains (fixed_fusion_test.cu:52-484):
+// build layout -> NT LUT -> NN LUT -> masks on the host, upload, then drive the attention through the
+// reference-named launchers: the unfused trio (bst_sgemm_nt, BlocksparseMaskedSoftmax, bst_sgemm_xn),
+// the two-stage fusion (fusion_attention2) and the full fusion (fusion_attention).  Unlike the
+// reference's timing harnesses it checks results: all-ones Q, K (the reference's inputs,
+// fixed_fusion_test.cu:263-268) give uniform probabilities in closed form, and on random inputs the
+// fused and unfused paths must agree.  Exit code 0 = all checks passed.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "blocksparse.h"
+#include "fusion_blocksparse.h"
+
+#define HIP_OK(call)                                                                      \
+    do {                                                                                  \
+        hipError_t e_ = (call);                                                           \
+        if (e_ != hipSuccess) {                                                           \
+            std::fprintf(stderr, "%s:%d %s\n", __FILE__, __LINE__, hipGetErrorString(e_)); \
+            return 2;                                                                     \
+        }                                                                                 \
+    } while (0)
+
+template <typename T>
+static T* upload(const std::vector<T>& v) {
+    T* d = nullptr;
+    if (hipMalloc((void**)&d, v.size() * sizeof(T)) != hipSuccess) return nullptr;
+    if (hipMemcpy(d, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice) != hipSuccess) return nullptr;
+    return d;
+}
+
+int main() {
+    const uint batch_dim = 2, heads_ = 4, head_state_ = 64, blk_size_ = 32, seq_len = 320;
+    const uint ctx_blks = seq_len / blk_size_;
+    const float scale = 1.0f / std::sqrt((float)head_state_);
+    const size_t tokens = (size_t)batch_dim * seq_len, state = (size_t)heads_ * head_state_;
+
+    // ---- descriptors: the 'fixed' pattern, stride 4, causal, one layout for all heads ----
+    std::vector<uint32_t> layout(ctx_blks * ctx_blks);
+    if (sfb_layout_fixed(layout.data(), 1, ctx_blks, 4, 1) != SFB_OK) return 1;
+    const uint blocks = sfb_count_blocks(layout.data(), ctx_blks);
+    std::vector<uint2> nt_lut(blocks), nn_lut(ctx_blks + blocks);
+    uint nn_max = 0;
+    sfb_build_nt_lut((sfb_uint2*)nt_lut.data(), layout.data(), ctx_blks);
+    sfb_build_nn_lut((sfb_uint2*)nn_lut.data(), (const sfb_uint2*)nt_lut.data(), blocks, ctx_blks, &nn_max);
+    std::vector<uint8_t> keep((size_t)blocks * blk_size_ * blk_size_);
+    sfb_element_mask(keep.data(), (const sfb_uint2*)nt_lut.data(), blocks, blk_size_, 1, 0);  // triangular diagonal blocks
+    std::vector<uint> mask_np((size_t)blocks * blk_size_), mask_rm((size_t)blocks * blk_size_);
+    sfb_pack_mask(mask_np.data(), keep.data(), blocks, blk_size_);
+    sfb_transpose_mask(mask_rm.data(), mask_np.data(), blocks, blk_size_);
+    uint magic = 0, shift = 0;
+    magicu64(CEIL_DIV(head_state_, 64), magic, shift);
+    std::printf("fixed layout: %u blocks, nn_lut_dim %u, nn_max %u, magic %u shift %u\n", blocks, ctx_blks + blocks,
+                nn_max, magic, shift);
+
+    uint2* d_nt = upload(nt_lut);
+    uint2* d_nn = upload(nn_lut);
+    uint* d_mask_np = upload(mask_np);
+    uint* d_mask_rm = upload(mask_rm);
+
+    // ---- inputs ----
+    std::vector<float> ones(tokens * state, 1.0f), q(tokens * state), k(tokens * state), v(tokens * state);
+    srand(7);
+    for (size_t i = 0; i < q.size(); ++i) {
+        q[i] = (rand() % 2001 - 1000) * 1e-3f;
+        k[i] = (rand() % 2001 - 1000) * 1e-3f;
+        v[i] = (rand() % 2001 - 1000) * 1e-3f;
+    }
+    float *d_ones = upload(ones), *d_q = upload(q), *d_k = upload(k), *d_v = upload(v);
+    const size_t sparse = (size_t)batch_dim * heads_ * blocks * blk_size_ * blk_size_;
+    bhalf *d_s = nullptr, *d_p = nullptr;
+    float *d_y = nullptr, *d_o_unfused = nullptr, *d_o_fused = nullptr;
+    HIP_OK(hipMalloc((void**)&d_s, sparse * sizeof(bhalf)));
+    HIP_OK(hipMalloc((void**)&d_p, sparse * sizeof(bhalf)));
+    HIP_OK(hipMalloc((void**)&d_y, sparse * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_o_unfused, tokens * state * sizeof(float)));
+    HIP_OK(hipMalloc((void**)&d_o_fused, tokens * state * sizeof(float)));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    int failures = 0;
+
+    // ---- 1. all-ones Q, K through fusion_attention2: every kept key of a row has probability 1/n ----
+    if (!fusion_attention2<float, float>(stream, d_nt, d_ones, d_ones, nullptr, d_nn, nullptr, nullptr, d_mask_np, nullptr,
+                                         nullptr, d_y, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                                         head_state_, 1, blocks, 1, scale)) {
+        std::fprintf(stderr, "fusion_attention2 failed: %s\n", sfb_status_string(sfb_host::last_status()));
+        return 1;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<float> y(sparse);
+    HIP_OK(hipMemcpy(y.data(), d_y, sparse * sizeof(float), hipMemcpyDeviceToHost));
+    std::vector<uint> kept_in_row((size_t)ctx_blks * blk_size_, 0);
+    for (uint blk = 0; blk < blocks; ++blk)
+        for (uint r = 0; r < blk_size_; ++r)
+            kept_in_row[nt_lut[blk].x * blk_size_ + r] += __builtin_popcount(mask_np[blk * blk_size_ + r]);
+    double worst = 0;
+    for (uint blk = 0; blk < blocks; ++blk)
+        for (uint r = 0; r < blk_size_; ++r)
+            for (uint c = 0; c < blk_size_; ++c) {
+                const float n = (float)kept_in_row[nt_lut[blk].x * blk_size_ + r];
+                const float want = ((mask_np[blk * blk_size_ + r] >> c) & 1u) ? 1.0f / (n + 1e-6f) : 0.0f;
+                worst = std::fmax(worst, std::fabs(y[((size_t)blk * blk_size_ + r) * blk_size_ + c] - want));
+            }
+    std::printf("all-ones closed form: max abs deviation %.3e\n", worst);
+    if (worst > 1e-6) ++failures;
+
+    // ---- 2. random inputs: unfused trio vs full fusion ----
+    bool ok = bst_sgemm_nt(stream, d_nt, d_q, d_k, d_s, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                           head_state_, 1, blocks);
+    ok = ok && BlocksparseMaskedSoftmax<bhalf, bhalf2>(stream, d_nn, d_mask_rm, d_s, d_p, blk_size_, blocks, batch_dim,
+                                                       heads_, ctx_blks, 1, ctx_blks + blocks, nn_max, 1, scale);
+    ok = ok && bst_sgemm_xn(stream, d_nn, d_p, d_v, d_o_unfused, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks,
+                            heads_, head_state_, 1, ctx_blks + blocks, NN_OP, magic, shift, nn_max);
+    ok = ok && fusion_attention<float, float>(stream, d_nt, d_q, d_k, nullptr, d_nn, nullptr, nullptr, d_mask_np,
+                                              nullptr, nullptr, (float*)nullptr, d_v, d_o_fused, blk_size_, blocks,
+                                              batch_dim, ctx_blks, ctx_blks, ctx_blks, heads_, head_state_, 1, blocks,
+                                              1, scale, nn_max);
+    if (!ok) {
+        std::fprintf(stderr, "launcher failed: %s\n", sfb_status_string(sfb_host::last_status()));
+        return 1;
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<float> o_u(tokens * state), o_f(tokens * state);
+    HIP_OK(hipMemcpy(o_u.data(), d_o_unfused, o_u.size() * sizeof(float), hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(o_f.data(), d_o_fused, o_f.size() * sizeof(float), hipMemcpyDeviceToHost));
+    double max_ref = 0, max_diff = 0;
+    for (size_t i = 0; i < o_u.size(); ++i) {
+        max_ref = std::fmax(max_ref, std::fabs(o_f[i]));
+        max_diff = std::fmax(max_diff, std::fabs(o_f[i] - o_u[i]));
+    }
+    std::printf("fused (fp32) vs unfused trio (bf16 S, P): max |diff| / max |O| = %.3e\n", max_diff / max_ref);
+    if (!(max_diff / max_ref < 1e-2)) ++failures;
+
+    // ---- 3. a block size the kernels do not implement is an error, not a silent no-op ----
+    if (bst_sgemm_nt(stream, d_nt, d_q, d_k, d_s, 16, blocks, batch_dim, ctx_blks, ctx_blks, heads_, head_state_, 1,
+                     blocks) || sfb_host::last_status() != SFB_ERR_BLOCK_SIZE)
+        ++failures;
+    std::printf(failures ? "FAILED (%d)\n" : "PASSED\n", failures);
+    return failures ? 1 : 0;
+}

@@ -135,3 +135,16 @@ def test_error_codes_instead_of_silent_no_op():
                                       u(1), u(2), u(1), u(1), C.c_float(0.125)) == 5
     assert sfb.lib.sfb_fused_sdd_softmax(None, None, p(q), p(q), p(q), 0, 0, None, None, u(64), u(1), u(1), u(1),
                                          u(1), u(64), u(1), u(2), u(1), C.c_float(0.125)) == 1
+
+
+def test_cpp_host_program_through_reference_named_launchers():
+    """sf-bert_amd/host/attention_host_test: a C++ main in the shape of the reference's *_fusion_test.cu
+    that calls bst_sgemm_nt / BlocksparseMaskedSoftmax / bst_sgemm_xn / fusion_attention2 / fusion_attention."""
+    import os
+    import subprocess
+    from sfb import ROOT
+    exe = os.path.join(ROOT, "sf-bert_amd", "host", "attention_host_test")
+    assert os.path.exists(exe), "run __graft_entry__.build() first"
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(out.stdout, out.stderr)
+    assert out.returncode == 0 and "PASSED" in out.stdout
