@@ -27,6 +27,12 @@ class SfbError(RuntimeError):
 
 
 def _load():
+    # torch ships its own copy of the HIP runtime; it has to be in the process before this library is
+    # loaded, so that both resolve to the same runtime and torch's streams are valid for our launches
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             "libsfbert_hip.so is not built (%s); run `python __graft_entry__.py` or "

@@ -89,4 +89,9 @@ __device__ __forceinline__ WorkId decode_work(uint32_t wg, uint32_t num_bh, uint
 
 inline uint32_t bh_groups(uint32_t num_bh) { return (num_bh + 7u) / 8u; }
 
+// A launcher reports only its own launch: the thread's last-error state may still hold an error left by
+// an unrelated earlier HIP call of the process, so it is cleared before the launch and read after it.
+inline void clear_stale_error() { (void)hipGetLastError(); }
+inline int launch_status() { return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH; }
+
 }  // namespace sfb

@@ -529,6 +529,7 @@ template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
     const uint32_t grid = p.groups * 8u * ranks;
+    clear_stale_error();
     if (in_dtype == SFB_BF16) {
         if (p.mask || p.valid_len)
             fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
@@ -536,7 +537,7 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
             fused_attention_bf16_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
     } else
         fused_attention_f32_kernel<BS, D><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+    return launch_status();
 }
 
 static int check_common(const void* q, const void* k, const void* v, const float* o, int in_dtype,

@@ -103,7 +103,7 @@ static inline uint32_t grid_for(uint64_t work_items) {
     return (uint32_t)(blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks));
 }
 
-static inline int launched() { return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH; }
+static inline int launched() { return launch_status(); }
 
 }  // namespace sfb
 
@@ -118,6 +118,7 @@ extern "C" int sfb_bias_act(sfb_stream_t stream, void* out, int out_dtype, const
     if (((uintptr_t)out | (uintptr_t)in | (uintptr_t)bias | (uintptr_t)residual) & 15u) return SFB_ERR_ALIGNMENT;
     const uint64_t vecs = rows * (cols / 4);
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
     const dim3 grid(grid_for(vecs));
 #define SFB_BA(T, A) bias_act_kernel<T, A><<<grid, 256, 0, s>>>((T*)out, in, bias, residual, vecs, cols / 4)
     if (out_dtype == SFB_F32) { if (act) SFB_BA(float, 1); else SFB_BA(float, 0); }
@@ -134,6 +135,7 @@ extern "C" int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, floa
     if (rows == 0 || state == 0 || (state & 3u)) return SFB_ERR_SHAPE;
     if (((uintptr_t)out | (uintptr_t)in | (uintptr_t)gain | (uintptr_t)bias) & 15u) return SFB_ERR_ALIGNMENT;
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
     const dim3 grid((rows + 3) / 4);
     if (out_dtype == SFB_F32)
         layernorm_kernel<float><<<grid, 256, 0, s>>>((float*)out, mean, rstd, in, gain, bias, rows, state);
@@ -148,6 +150,7 @@ extern "C" int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, c
     if (dim0 == 0 || inner == 0 || (inner & 3u)) return SFB_ERR_SHAPE;
     if (((uintptr_t)out | (uintptr_t)a | (uintptr_t)m) & 15u) return SFB_ERR_ALIGNMENT;
     const uint64_t vecs = dim0 * (inner / 4);
+    clear_stale_error();
     add_matrix_kernel<<<dim3(grid_for(vecs)), 256, 0, (hipStream_t)stream>>>(out, a, m, vecs, inner / 4);
     return launched();
 }
@@ -158,6 +161,7 @@ extern "C" int sfb_embedding_lookup(sfb_stream_t stream, float* out, const float
     if (!out || !table || !ids) return SFB_ERR_NULL_POINTER;
     if (tokens == 0 || state == 0 || (state & 3u) || vocab == 0 || (pos && seq_len == 0)) return SFB_ERR_SHAPE;
     if (((uintptr_t)out | (uintptr_t)table | (uintptr_t)pos) & 15u) return SFB_ERR_ALIGNMENT;
+    clear_stale_error();
     embedding_kernel<<<dim3(grid_for(tokens * (state / 4))), 256, 0, (hipStream_t)stream>>>(
         out, table, ids, pos, tokens, state / 4, seq_len ? seq_len : 1, vocab);
     return launched();
@@ -167,6 +171,7 @@ extern "C" int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in
     if (!out || !in) return SFB_ERR_NULL_POINTER;
     if (n == 0 || (n & 3u)) return SFB_ERR_SHAPE;
     if (((uintptr_t)out & 7u) || ((uintptr_t)in & 15u)) return SFB_ERR_ALIGNMENT;
+    clear_stale_error();
     bias_act_kernel<__bf16, 0><<<dim3(grid_for(n / 4)), 256, 0, (hipStream_t)stream>>>(
         (__bf16*)out, in, nullptr, nullptr, n / 4, 1);
     return launched();

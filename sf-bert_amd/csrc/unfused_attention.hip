@@ -375,11 +375,12 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
                    lut_heads > 1 ? lut_dim : 0};
     const dim3 grid(blocks, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
 #define SFB_CALL(BSV, TI, TO) sdd_nt_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, out_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, out_dtype, SFB_CALL);
 #undef SFB_CALL
-    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+    return launch_status();
 }
 
 extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, const void* mask, const void* x,
@@ -401,11 +402,12 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     if ((rows + 3) / 4 > 0x7fffffffull) return SFB_ERR_SHAPE;
     const dim3 grid((uint32_t)((rows + 3) / 4));
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
 #define SFB_CALL(BSV, TX, TY) masked_softmax_kernel<BSV, TX, TY><<<grid, dim3(256), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, x_dtype, y_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, x_dtype, y_dtype, SFB_CALL);
 #undef SFB_CALL
-    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+    return launch_status();
 }
 
 extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
@@ -426,11 +428,12 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
                    lut_heads > 1 ? lut_dim : 0, bh_groups(batch_dim * head_dim)};
     const dim3 grid(p.groups * 8u * ctx_blks_c);
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
 #define SFB_CALL(BSV, TP, TV) dsd_nn_kernel<BSV, 64, TP, TV><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, a_dtype, b_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, a_dtype, b_dtype, SFB_CALL);
 #undef SFB_CALL
-    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+    return launch_status();
 }
 
 extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const void* a,
@@ -453,9 +456,10 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
                           bh_groups(batch_dim * head_dim), scale * kLog2e};
     const dim3 grid(p.groups * 8u * ctx_blks);
     hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
 #define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);
 #undef SFB_CALL
-    return hipGetLastError() == hipSuccess ? SFB_OK : SFB_ERR_LAUNCH;
+    return launch_status();
 }
