@@ -168,6 +168,10 @@ __device__ __forceinline__ uint32_t partial_offset(int mt, int ig, uint32_t half
     return (((mt * 4 + ig) * 2 + half) * BS + q_in_block) * 4;
 }
 
+template <int BS, int D>
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, float c,
+                                               uint32_t q_in_block, uint32_t half);
+
 // End of a work item.  Unsplit rows are normalised and stored.  A chunk of a split row writes its
 // partial (unnormalised O, reference maximum, true maximum, sum) and bumps the row's counter; the
 // chunk that finds every other chunk already arrived merges all partials, stores O and resets the
@@ -206,10 +210,19 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     }
     __syncthreads();
     if (!last_flag) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    merge_partials<BS, D>(base, w.nchunks, o_row, c, q_in_block, half);
+    if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
+// Merge of the partial records of a split row (run by the chunk that arrived last).
+template <int BS, int D>
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, float c,
+                                               uint32_t q_in_block, uint32_t half) {
+    constexpr int NO = D / 32;
+    constexpr int PART = BS * D + 4 * BS;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     float m_used = kMaxSeed, m_true = kMaxSeed;
-    for (uint32_t ch = 0; ch < w.nchunks; ++ch) {
+    for (uint32_t ch = 0; ch < nchunks; ++ch) {
         const float* stats = base + (size_t)ch * PART + BS * D + q_in_block * 4;
         m_used = fmaxf(m_used, coherent_load(stats + 0));
         m_true = fmaxf(m_true, coherent_load(stats + 1));
@@ -220,7 +233,7 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
     float sum = 0.f;
-    for (uint32_t ch = 0; ch < w.nchunks; ++ch) {
+    for (uint32_t ch = 0; ch < nchunks; ++ch) {
         const float* part = base + (size_t)ch * PART;
         const float* stats = part + BS * D + q_in_block * 4;
         const float wgt = exp2_fast((coherent_load(stats + 0) - m_used) * c);
@@ -232,7 +245,6 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
         });
     }
     store_output<NO>(o_row, acc, m_used, m_true, sum, c, half);
-    if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int D>
@@ -343,9 +355,10 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     RowState st = {kMaxSeed, kMaxSeed, 0.f};
     const float c = p.scale_log2e, slack = p.slack;
 
-    // prologue: K(0), V(0) and K(1) into LDS, S_next = scores of block 0;
-    // set 0 holds K(2), V(1) and set 1 holds K(3), V(2), all in flight
-    f32x16 s_next[KT];
+    // prologue: K(0), V(0) and K(1) into LDS, scores of block 0 in s_even;
+    // set 0 holds K(2), V(1) and set 1 holds K(3), V(2), all in flight.
+    // Even iterations consume s_even and produce s_odd, odd iterations the reverse (no copies).
+    f32x16 s_even[KT], s_odd[KT];
     T::fetch_k(gk0, K, tile_base(0), row_stride, t);
     T::fetch_v(gv0, V, tile_base(0), row_stride, t);
     T::fetch_k(gk1, K, tile_base(1), row_stride, t);
@@ -357,10 +370,11 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     T::fetch_k(gk1, K, tile_base(3), row_stride, t);
     T::fetch_v(gv1, V, tile_base(2), row_stride, t);
     __syncthreads();
-    score_tile(s_next, kb);
+    score_tile(s_even, kb);
     __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
 
-    auto iteration = [&](uint32_t j, typename T::KRegs& gk, typename T::VRegs& gv) {
+    auto iteration = [&](uint32_t j, typename T::KRegs& gk, typename T::VRegs& gv, f32x16 (&s)[KT],
+                         f32x16 (&s_next)[KT]) {
         const uint32_t par = j & 1;
         uint8_t* const k_write = kb + par * T::K_BYTES;             // K(j+2) replaces K(j)
         const uint8_t* const k_read = kb + (par ^ 1) * T::K_BYTES;  // K(j+1)
@@ -372,9 +386,6 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         T::fetch_k(gk, K, tile_base(j + 4), row_stride, t);
         T::fetch_v(gv, V, tile_base(j + 3), row_stride, t);
 
-        f32x16 s[KT];
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) s[kt] = s_next[kt];
         score_tile(s_next, k_read);
 
         if (MASKED) {
@@ -412,8 +423,8 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     };
 
     for (uint32_t j = 0; j < count; j += 2) {
-        iteration(j, gk0, gv0);
-        if (j + 1 < count) iteration(j + 1, gk1, gv1);
+        iteration(j, gk0, gv0, s_even, s_odd);
+        if (j + 1 < count) iteration(j + 1, gk1, gv1, s_odd, s_even);
     }
 
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
