@@ -15,6 +15,7 @@
 // Arithmetic follows the reference CPU path: scores are raw dot products, the maximum is taken over
 // kept keys with seed -1000000 (ewops.h:70), p = exp((s-max)*scale) (ewops.h:86), the row is divided
 // by sum + 1e-6 (ewops.h:93), and O = P.V (matmul.h:6-20).
+#include <cstdlib>
 #include "tiles.hip.h"
 
 namespace sfb {
@@ -386,8 +387,6 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         T::fetch_k(gk, K, tile_base(j + 4), row_stride, t);
         T::fetch_v(gv, V, tile_base(j + 3), row_stride, t);
 
-        score_tile(s_next, k_read);
-
         if (MASKED) {
             const sfb_uint2 here = lut[lut_off + j];
             const int limit = valid - (int)(here.y * BS);
@@ -411,6 +410,18 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
             if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
+            // a slice of the next block's scores with every chunk keeps the MFMA pipe fed evenly
+#pragma unroll
+            for (int ks = u * (KS / PU); ks < (u + 1) * (KS / PU); ++ks)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    if (ks == 0) {
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, kt, ks, qn, half), qf[ks], zero, 0, 0, 0);
+                    } else {
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, kt, ks, qn, half), qf[ks], s_next[kt], 0, 0, 0);
+                    }
+                }
             const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
             const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
@@ -425,6 +436,165 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     for (uint32_t j = 0; j < count; j += 2) {
         iteration(j, gk0, gv0, s_even, s_odd);
         if (j + 1 < count) iteration(j + 1, gk1, gv1, s_odd, s_even);
+    }
+
+    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
+}
+
+// ------------------------------------------------------------------------------------------------
+// bf16 inputs, tiles copied memory -> LDS without passing through registers
+// ------------------------------------------------------------------------------------------------
+// Same arithmetic as the kernel above with a leaner instruction stream: K and V tiles of a key block are
+// fetched with LDS-direct loads into swizzled row-major buffers (see Bf16DirectTiles), V^T fragments come
+// from transposing LDS reads.  In iteration j a wave
+//   * issues the loads of K(j+2) and V(j+1) into the buffers that iteration j-1 finished reading;
+//   * finds the row maximum of S(j), then, chunk by chunk, exponentiates S(j), feeds V(j)^T . P^T and
+//     computes a slice of S(j+1) = K(j+1) . Q^T;
+//   * waits for its own loads and meets the other waves at the one barrier of the iteration.
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(FusedParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
+    constexpr int TILE = T::TILE_BYTES;
+
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+
+    const RowWork w = decode_row_work(p);
+    if (!w.valid) return;
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t row_bytes = p.heads * D * 2;
+
+    const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
+    const uint32_t lut_off = __builtin_amdgcn_readfirstlane(lut[w.row].x + w.first);
+    const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
+    float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
+
+    if (count == 0) {
+        store_zero_row<D>(o_row, half);
+        return;
+    }
+
+    const __bf16* Q = (const __bf16*)p.q;
+    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)w.h * p.mask_stride * (BS / 8) : nullptr;
+    const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
+
+    // byte address of (b, token 0, h, 0) in K and V; key block column col starts col*BS rows further
+    const size_t bh_bytes = token_offset(w.b, 0, w.h, L, p.heads, D) * 2;
+    const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
+    const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
+    const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+    const uint32_t lds0 = T::lds_address(smem);
+    // LUT entries of key blocks [win, win + 64) of this item, one per lane (clamped to the last one)
+    uint32_t win = 0;
+    sfb_uint2 entries;
+    auto refill = [&](uint32_t first) {
+        win = first;
+        const uint32_t idx = first + lane;
+        entries = lut[lut_off + (idx < count ? idx : count - 1)];
+    };
+    refill(0);
+    auto column_of = [&](uint32_t j) -> uint32_t {
+        const uint32_t jj = j < count ? j : count - 1;
+        return __builtin_amdgcn_readlane(entries.y, jj - win);
+    };
+    auto load_k = [&](uint32_t j, uint32_t buf) {
+        T::load_tile(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+    };
+    auto load_v = [&](uint32_t j, uint32_t buf) {
+        T::load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)column_of(j) * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+    };
+    auto loads_landed = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+
+    bf16x8 qf[KS];
+    T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
+    const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
+
+    f32x16 o_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
+    RowState st = {kMaxSeed, kMaxSeed, 0.f};
+    const float c = p.scale_log2e, slack = p.slack;
+
+    f32x16 s_even[KT], s_odd[KT];
+    loads_landed();
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_even[kt][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            s_even[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(smem, k_lane, kt, ks), qf[ks], s_even[kt], 0, 0, 0);
+    }
+    __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
+
+    auto iteration = [&](uint32_t j, f32x16 (&s)[KT], f32x16 (&s_next)[KT]) {
+        const uint32_t par = j & 1;
+        const uint8_t* const k_read = smem + (par ^ 1) * TILE;       // K(j+1)
+        const uint8_t* const v_read = smem + (2 + par) * TILE;       // V(j)
+        if (j + 2 >= win + 64) refill(j);
+        load_k(j + 2, par);          // replaces K(j)
+        load_v(j + 1, par ^ 1);      // replaces V(j-1)
+
+        if (MASKED) {
+            const sfb_uint2 here = {(uint32_t)__builtin_amdgcn_readlane(entries.x, j - win),
+                                    (uint32_t)__builtin_amdgcn_readlane(entries.y, j - win)};
+            const int limit = valid - (int)(here.y * BS);
+            if ((mask != nullptr) || (limit < BS))
+                apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit), half);
+        }
+        const float mloc = block_row_max<KT>(s);
+        st.m_true = fmaxf(st.m_true, mloc);
+        if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
+            const float m_new = fmaxf(st.m_used, mloc);
+            const float alpha = exp2_fast((st.m_used - m_new) * c);
+            st.m_used = m_new;
+            st.l *= alpha;
+#pragma unroll
+            for (int n = 0; n < NO; ++n) o_acc[n] *= alpha;
+        }
+        const float mc = st.m_used * c;
+        float sum0 = 0.f, sum1 = 0.f;
+        uint32_t pk[KT * 8];
+        exp_chunk<KT, NO>(s, pk, 0, c, mc, sum0, sum1);
+#pragma unroll
+        for (int u = 0; u < PU; ++u) {
+            if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
+#pragma unroll
+            for (int ks = u * (KS / PU); ks < (u + 1) * (KS / PU); ++ks)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    if (ks == 0) {
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, k_lane, kt, ks), qf[ks], zero, 0, 0, 0);
+                    } else {
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, k_lane, kt, ks), qf[ks], s_next[kt], 0, 0, 0);
+                    }
+                }
+            const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
+            const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+#pragma unroll
+            for (int mt = 0; mt < NO; ++mt)
+                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(v_read, v_lane, mt, u), bfrag, o_acc[mt], 0, 0, 0);
+        }
+        st.l += sum0 + sum1;
+        loads_landed();
+    };
+
+    for (uint32_t j = 0; j < count; j += 2) {
+        iteration(j, s_even, s_odd);
+        if (j + 1 < count) iteration(j + 1, s_odd, s_even);
     }
 
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
@@ -536,12 +706,19 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedPar
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
 }
 
+static int g_variant = getenv("SFB_VARIANT") ? atoi(getenv("SFB_VARIANT")) : 1;
+
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
     const uint32_t grid = p.groups * 8u * ranks;
     clear_stale_error();
-    if (in_dtype == SFB_BF16) {
+    if (in_dtype == SFB_BF16 && g_variant == 1) {
+        if (p.mask || p.valid_len)
+            fused_attention_bf16_direct_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+        else
+            fused_attention_bf16_direct_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+    } else if (in_dtype == SFB_BF16) {
         if (p.mask || p.valid_len)
             fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
         else

@@ -99,6 +99,96 @@ struct Bf16Tiles {
 };
 
 // ------------------------------------------------------------------------------------------------
+// bf16 operands, tiles copied from memory straight into LDS (global_load_lds_dwordx4)
+// ------------------------------------------------------------------------------------------------
+// K and V tiles are both kept row-major, [BS keys][D] bf16 = 128-byte rows of eight 16-byte chunks, with
+// no padding: an LDS-direct load writes the 64 lanes' 16 bytes back to back (1 KiB = 8 rows per
+// instruction), so the layout inside a row is chosen through the *global* address each lane fetches.
+// Chunk c of row r is stored at position c ^ swz(r), swz(r) = rotate-right of the 3-bit value (r/2)%8:
+//   * score fragments (ds_read_b128; 16 lanes = 16 consecutive rows, one chunk) hit 16 different
+//     16-byte slots of the 256-byte bank window, because rows 2a and 2a+1 sit in different halves of
+//     the window and swz() is distinct over a = 0..7;
+//   * V^T fragments are read with ds_read_b64_tr_b16, which transposes inside groups of 16 lanes: source
+//     lane s = 4j + q supplies 4 consecutive columns of key row j (j = 0..3) starting at column 4q, and
+//     result lane i receives the 4 consecutive keys of column i.  The lowest bit of r/2 becomes the
+//     highest bit of swz(), which moves key rows j = 2, 3 into the other 64-byte half of the row, so
+//     the 4 rows x 64 bytes that 32 lanes touch are disjoint in the bank window.
+// No registers are spent on staging and no ds_write / v_perm instructions are needed.
+template <int BS, int D>
+struct Bf16DirectTiles {
+    static_assert(D == 64, "128-byte rows");
+    static constexpr int NW = BS / 32;                 // waves per work-group
+    static constexpr int TILE_BYTES = BS * D * 2;
+    static constexpr int GROUPS = BS / 8;              // 8-row groups (one load instruction each)
+
+    typedef uint32_t __attribute__((address_space(3)))* lds_u32_ptr;
+    // LDS byte address of a pointer into a __shared__ array
+    static __device__ __forceinline__ uint32_t lds_address(const void* p) {
+        return (uint32_t)(uintptr_t)(lds_u32_ptr)p;
+    }
+    static __device__ __forceinline__ uint32_t swz(uint32_t row) {
+        const uint32_t x = (row >> 1) & 7u;
+        return ((x & 1u) << 2) | (x >> 1);
+    }
+    // Byte offset, relative to row 0 of an 8-row group, of the 16 bytes this lane fetches; `odd` says
+    // whether the group index is odd (rows 8..15 of a 16-row period).
+    static __device__ __forceinline__ uint32_t lane_source(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
+        const uint32_t rr = lane >> 3, pos = lane & 7u;
+        return rr * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
+    }
+    // This wave's share of the loads of one tile.  g_tile: address of the tile's first row (uniform);
+    // lds_tile: LDS byte address of the tile (uniform); src_even/src_odd from lane_source().
+    static __device__ __forceinline__ void load_tile(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
+                                                     uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
+#pragma unroll
+        for (int i = 0; i < GROUPS / NW; ++i) {
+            const uint32_t n = (NW % 2 == 0) ? (wave + NW * i) : (uint32_t)(NW * i) + wave;
+            uint32_t src;
+            if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
+            else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
+            // the uniform part goes through readfirstlane so that it stays in scalar registers and the
+            // load takes the (scalar base + 32-bit lane offset) form
+            const uint64_t ga = (uint64_t)(g_tile + (size_t)n * 8u * row_bytes);
+            const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
+            const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
+            const uint8_t* g = (const uint8_t*)(((uint64_t)ga_hi << 32) | (uint64_t)ga_lo);
+            __builtin_amdgcn_global_load_lds((const uint32_t*)(g + src), (lds_u32_ptr)(uintptr_t)(lds_tile + n * 1024u),
+                                             16, 0, 0);
+        }
+    }
+    // Per-lane byte offset of the score fragment of k-step 0 in key tile 0; k-step ks is at (base ^ ks*32),
+    // key tile kt 4096 bytes further.
+    static __device__ __forceinline__ uint32_t k_lane_base(uint32_t qn, uint32_t half) {
+        return qn * 128u + ((half ^ swz(qn)) << 4);
+    }
+    static __device__ __forceinline__ bf16x8 k_frag(const uint8_t* k_lds, uint32_t lane_base, int kt, int ks) {
+        return *(const bf16x8*)(k_lds + kt * 4096 + (lane_base ^ (uint32_t)(ks * 32)));
+    }
+    // Per-lane byte offset of the transposing read for (column tile 0, first 4-key group of product step
+    // 0); column tile mt and second group x are at (base ^ (mt*64 + x*32)) + x*1024, step u 2048 bytes on.
+    static __device__ __forceinline__ uint32_t v_lane_base(uint32_t lane) {
+        const uint32_t G = lane >> 4, s = lane & 15u, j = s >> 2, q = s & 3u, h = G >> 1, g2 = G & 1u;
+        const uint32_t lp = (2u * g2 + (q >> 1)) ^ (((j >> 1) << 2) | h);
+        return (h * 4u + j) * 128u + (lp << 4) + (q & 1u) * 8u;
+    }
+    static __device__ __forceinline__ bf16x8 v_frag(const uint8_t* v_lds, uint32_t lane_base, int mt, int u) {
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        typedef s16x4 __attribute__((address_space(3)))* lds_ptr;
+        const uint8_t* a0 = v_lds + u * 2048 + (lane_base ^ (uint32_t)(mt * 64));
+        const uint8_t* a1 = v_lds + u * 2048 + 1024 + (lane_base ^ (uint32_t)(mt * 64 + 32));
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a0);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a1);
+        const u32x4 r = {__builtin_bit_cast(u32x2, lo).x, __builtin_bit_cast(u32x2, lo).y,
+                         __builtin_bit_cast(u32x2, hi).x, __builtin_bit_cast(u32x2, hi).y};
+        return __builtin_bit_cast(bf16x8, r);
+    }
+    static __device__ __forceinline__ void load_q(bf16x8 (&qf)[D / 16], const __bf16* q_row, uint32_t half) {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) qf[ks] = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
 // fp32 operands, v_mfma_f32_32x32x2_f32 (one float per lane per step: k-slot = half)
 // ------------------------------------------------------------------------------------------------
 // K tile in LDS: [BS][D + 4] floats; score k-slot (step, half) is head-dimension index
