@@ -456,6 +456,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
     constexpr int TILE = T::TILE_BYTES;
+    constexpr int SC = PU >= 2 ? PU / 2 : 1;   // chunks that carry a slice of the next block's scores
 
     __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
 
@@ -544,8 +545,11 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(
         const uint8_t* const k_read = smem + (par ^ 1) * TILE;       // K(j+1)
         const uint8_t* const v_read = smem + (2 + par) * TILE;       // V(j)
         if (j + 2 >= win + 64) refill(j);
-        load_k(j + 2, par);          // replaces K(j)
-        load_v(j + 1, par ^ 1);      // replaces V(j-1)
+        // K(j+2) replaces K(j), V(j+1) replaces V(j-1); the loads are issued a few at a time between the
+        // chunks below so that they never queue up in front of the arithmetic
+        const uint8_t* const k_src = k_base + (size_t)column_of(j + 2) * BS * row_bytes;
+        const uint8_t* const v_src = v_base + (size_t)column_of(j + 1) * BS * row_bytes;
+        const uint32_t k_dst = lds0 + par * TILE, v_dst = lds0 + (2 + (par ^ 1)) * TILE;
 
         if (MASKED) {
             const sfb_uint2 here = {(uint32_t)__builtin_amdgcn_readlane(entries.x, j - win),
@@ -572,7 +576,14 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(
         for (int u = 0; u < PU; ++u) {
             if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
 #pragma unroll
-            for (int ks = u * (KS / PU); ks < (u + 1) * (KS / PU); ++ks)
+            for (int i = u * (T::LOADS / PU); i < (u + 1) * (T::LOADS / PU); ++i) {
+                T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
+                T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
+            }
+            // the next block's scores are finished in the first half of the chunks: the maximum at the
+            // top of the next iteration then finds them complete instead of waiting for the MFMA pipe
+#pragma unroll
+            for (int ks = u * (KS / SC); ks < (u + 1) * (KS / SC) && ks < KS; ++ks)
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) {
                     if (ks == 0) {

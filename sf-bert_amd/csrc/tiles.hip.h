@@ -136,25 +136,28 @@ struct Bf16DirectTiles {
         const uint32_t rr = lane >> 3, pos = lane & 7u;
         return rr * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
     }
-    // This wave's share of the loads of one tile.  g_tile: address of the tile's first row (uniform);
-    // lds_tile: LDS byte address of the tile (uniform); src_even/src_odd from lane_source().
+    // Load number i (0 .. LOADS-1) of this wave's share of one tile: 8 rows = 1 KiB.  g_tile: address of
+    // the tile's first row (uniform); lds_tile: LDS byte address of the tile (uniform); src_even /
+    // src_odd from lane_source().
+    static constexpr int LOADS = GROUPS / NW;
+    static __device__ __forceinline__ void load_rows(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
+                                                     uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
+        const uint32_t n = (uint32_t)(NW * i) + wave;   // 8-row group
+        uint32_t src;
+        if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
+        else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
+        // the uniform part goes through readfirstlane so that it stays in scalar registers
+        const uint64_t ga = (uint64_t)(g_tile + (size_t)n * 8u * row_bytes);
+        const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
+        const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
+        const uint8_t* g = (const uint8_t*)(((uint64_t)ga_hi << 32) | (uint64_t)ga_lo);
+        __builtin_amdgcn_global_load_lds((const uint32_t*)(g + src), (lds_u32_ptr)(uintptr_t)(lds_tile + n * 1024u),
+                                         16, 0, 0);
+    }
     static __device__ __forceinline__ void load_tile(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
 #pragma unroll
-        for (int i = 0; i < GROUPS / NW; ++i) {
-            const uint32_t n = (NW % 2 == 0) ? (wave + NW * i) : (uint32_t)(NW * i) + wave;
-            uint32_t src;
-            if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
-            else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
-            // the uniform part goes through readfirstlane so that it stays in scalar registers and the
-            // load takes the (scalar base + 32-bit lane offset) form
-            const uint64_t ga = (uint64_t)(g_tile + (size_t)n * 8u * row_bytes);
-            const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
-            const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
-            const uint8_t* g = (const uint8_t*)(((uint64_t)ga_hi << 32) | (uint64_t)ga_lo);
-            __builtin_amdgcn_global_load_lds((const uint32_t*)(g + src), (lds_u32_ptr)(uintptr_t)(lds_tile + n * 1024u),
-                                             16, 0, 0);
-        }
+        for (int i = 0; i < LOADS; ++i) load_rows(lds_tile, g_tile, i, wave, src_even, src_odd, row_bytes);
     }
     // Per-lane byte offset of the score fragment of k-step 0 in key tile 0; k-step ks is at (base ^ ks*32),
     // key tile kt 4096 bytes further.
