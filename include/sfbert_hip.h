@@ -111,7 +111,7 @@ typedef struct {
     uint32_t chunk;    /* index of this chunk within the row */
     uint32_t slot;     /* index of the row among split rows (arrival counter), 0 if not split */
     uint32_t part;     /* index of the row's first partial-result record, 0 if not split */
-    uint32_t reserved;
+    uint32_t lut_first; /* index of the item's first entry in the NN LUT: nn_lut[row].x + first */
 } sfb_work_item;
 /* items may be NULL to query the counts; otherwise it must hold *n_items entries as returned by a
  * query call.  n_slots = number of split rows, n_parts = total chunks of split rows, n_heavy = number

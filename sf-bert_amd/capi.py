@@ -176,7 +176,7 @@ def transpose_mask(words, blocks, bs):
 
 
 WORK_ITEM_DTYPE = np.dtype([(n, np.uint32) for n in
-                            ("row", "first", "count", "nchunks", "chunk", "slot", "part", "reserved")])
+                            ("row", "first", "count", "nchunks", "chunk", "slot", "part", "lut_first")])
 
 
 def build_schedule(nn_lut, nb, max_blocks=16):

@@ -296,14 +296,14 @@ int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heav
         const uint32_t count = nn_lut[r].y;
         const uint32_t chunks = count > max_blocks ? (count + max_blocks - 1) / max_blocks : 1;
         if (chunks == 1) {
-            all.push_back(sfb_work_item{(uint32_t)r, 0u, count, 1u, 0u, 0u, 0u, 0u});
+            all.push_back(sfb_work_item{(uint32_t)r, 0u, count, 1u, 0u, 0u, 0u, nn_lut[r].x});
             continue;
         }
         const uint32_t base = count / chunks, extra = count % chunks;
         uint32_t first = 0;
         for (uint32_t c = 0; c < chunks; ++c) {
             const uint32_t len = base + (c < extra ? 1u : 0u);
-            all.push_back(sfb_work_item{(uint32_t)r, first, len, chunks, c, slots, parts, 0u});
+            all.push_back(sfb_work_item{(uint32_t)r, first, len, chunks, c, slots, parts, nn_lut[r].x + first});
             first += len;
         }
         ++slots;

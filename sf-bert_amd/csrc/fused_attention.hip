@@ -15,7 +15,6 @@
 // Arithmetic follows the reference CPU path: scores are raw dot products, the maximum is taken over
 // kept keys with seed -1000000 (ewops.h:70), p = exp((s-max)*scale) (ewops.h:86), the row is divided
 // by sum + 1e-6 (ewops.h:93), and O = P.V (matmul.h:6-20).
-#include <cstdlib>
 #include "tiles.hip.h"
 
 namespace sfb {
@@ -49,6 +48,7 @@ struct RowWork {
     uint32_t first, count;          // key blocks [first, first+count) of the row's LUT segment
     uint32_t nchunks, slot, part;   // split rows: number of chunks, counter index, first partial index
     uint32_t chunk;
+    uint32_t lut_first;             // index of the item's first entry in the head's NN LUT
     bool valid;
 };
 
@@ -63,10 +63,13 @@ __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
         const sfb_work_item it = p.items[id.rank];
         w.row = it.row; w.first = it.first; w.count = it.count;
         w.nchunks = it.nchunks; w.slot = it.slot; w.part = it.part; w.chunk = it.chunk;
+        w.lut_first = it.lut_first;
     } else {
         w.row = p.row_order ? p.row_order[id.rank] : (p.nb - 1 - id.rank);
         w.first = 0;
-        w.count = id.valid ? p.nn_lut[(size_t)w.h * p.lut_stride + w.row].y : 0;
+        const sfb_uint2 header = p.nn_lut[(size_t)w.h * p.lut_stride + (id.valid ? w.row : 0u)];
+        w.count = id.valid ? header.y : 0;
+        w.lut_first = header.x;
         w.nchunks = 1; w.slot = 0; w.part = 0; w.chunk = 0;
     }
     return w;
@@ -258,15 +261,9 @@ __device__ __forceinline__ void store_zero_row(float* o_row, uint32_t half) {
 // ------------------------------------------------------------------------------------------------
 // bf16 inputs, fp32 accumulation: v_mfma_f32_32x32x16_bf16
 // ------------------------------------------------------------------------------------------------
-// Software pipeline over the key blocks of the row.  In iteration j a wave
-//   * writes K(j+2) and V(j+1), fetched from memory during iteration j-1, into the free LDS buffers
-//     and issues the fetches of K(j+3) and V(j+2);
-//   * multiplies S_next = K(j+1) . Q^T on MFMA while the VALU finds the row maximum of S_cur (block j);
-//   * exponentiates S_cur in four chunks, each chunk's probabilities feeding the V(j)^T . P^T MFMAs
-//     while the next chunk is exponentiated.
-// K and V tiles are double-buffered in LDS with K running one block ahead of V; one barrier per key
-// block.  Block indices past the end of the row are clamped: the extra tiles are loaded and
-// multiplied but never used.
+// Exponentials of chunk u (16 keys) of a score block: pk[4u .. 4u+3] receive the probabilities rounded to
+// bf16, in the order the P^T operand of product step u wants them; the row sum is taken over the rounded
+// values, i.e. over exactly what the P.V product uses.
 template <int KT, int NO>
 __device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], int u, float c,
                                           float mc, float& sum0, float& sum1) {
@@ -287,172 +284,15 @@ __device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[
     sum1 = dot2_bf16_ones(e, sum1);
 }
 
-template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
-    using T = Bf16Tiles<BS, D>;
-    constexpr int KT = BS / 32;      // 32-key tiles per block
-    constexpr int NO = D / 32;       // 32-column tiles of O
-    constexpr int KS = D / 16;       // MFMA k-steps over the head dimension
-    constexpr int PU = BS / 16;      // MFMA k-steps over the keys of a block
-
-    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * T::K_BYTES + 2 * T::V_BYTES];
-
-    const RowWork w = decode_row_work(p);
-    if (!w.valid) return;
-    const uint32_t L = p.nb * BS;
-    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const uint32_t qn = lane & 31, half = lane >> 5;
-    const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_stride = p.heads * D;
-
-    const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
-    const uint32_t lut_off = lut[w.row].x + w.first, count = w.count;
-    float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
-
-    if (count == 0) {
-        store_zero_row<D>(o_row, half);
-        return;
-    }
-
-    const __bf16* Q = (const __bf16*)p.q;
-    const __bf16* K = (const __bf16*)p.k;
-    const __bf16* V = (const __bf16*)p.v;
-    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)w.h * p.mask_stride * (BS / 8) : nullptr;
-    const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
-
-    bf16x8 qf[KS];
-    T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
-
-    // element offset of key block number j of this item (clamped to the last one)
-    const size_t bh_base = token_offset(w.b, 0, w.h, L, p.heads, D);
-    auto tile_base = [&](uint32_t j) -> size_t {
-        const uint32_t jj = j < count ? j : count - 1;
-        return bh_base + (size_t)(lut[lut_off + jj].y * BS) * row_stride;
-    };
-    auto score_tile = [&](f32x16 (&s)[KT], const uint8_t* k_lds) {
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_lds, kt, ks, qn, half), qf[ks],
-                                                                s[kt], 0, 0, 0);
-    };
-
-    // two register sets of fetched tiles: each is written to LDS two iterations after it was requested
-    typename T::KRegs gk0, gk1;
-    typename T::VRegs gv0, gv1;
-    uint8_t* const kb = smem;
-    uint8_t* const vb = smem + 2 * T::K_BYTES;
-
-    f32x16 o_acc[NO];
-#pragma unroll
-    for (int n = 0; n < NO; ++n)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
-    RowState st = {kMaxSeed, kMaxSeed, 0.f};
-    const float c = p.scale_log2e, slack = p.slack;
-
-    // prologue: K(0), V(0) and K(1) into LDS, scores of block 0 in s_even;
-    // set 0 holds K(2), V(1) and set 1 holds K(3), V(2), all in flight.
-    // Even iterations consume s_even and produce s_odd, odd iterations the reverse (no copies).
-    f32x16 s_even[KT], s_odd[KT];
-    T::fetch_k(gk0, K, tile_base(0), row_stride, t);
-    T::fetch_v(gv0, V, tile_base(0), row_stride, t);
-    T::fetch_k(gk1, K, tile_base(1), row_stride, t);
-    T::stage_k(kb, gk0, t);
-    T::stage_v(vb, gv0, t);
-    T::stage_k(kb + T::K_BYTES, gk1, t);
-    T::fetch_k(gk0, K, tile_base(2), row_stride, t);
-    T::fetch_v(gv0, V, tile_base(1), row_stride, t);
-    T::fetch_k(gk1, K, tile_base(3), row_stride, t);
-    T::fetch_v(gv1, V, tile_base(2), row_stride, t);
-    __syncthreads();
-    score_tile(s_even, kb);
-    __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
-
-    auto iteration = [&](uint32_t j, typename T::KRegs& gk, typename T::VRegs& gv, f32x16 (&s)[KT],
-                         f32x16 (&s_next)[KT]) {
-        const uint32_t par = j & 1;
-        uint8_t* const k_write = kb + par * T::K_BYTES;             // K(j+2) replaces K(j)
-        const uint8_t* const k_read = kb + (par ^ 1) * T::K_BYTES;  // K(j+1)
-        uint8_t* const v_write = vb + (par ^ 1) * T::V_BYTES;       // V(j+1) replaces V(j-1)
-        const uint8_t* const v_read = vb + par * T::V_BYTES;        // V(j)
-
-        T::stage_k(k_write, gk, t);
-        T::stage_v(v_write, gv, t);
-        T::fetch_k(gk, K, tile_base(j + 4), row_stride, t);
-        T::fetch_v(gv, V, tile_base(j + 3), row_stride, t);
-
-        if (MASKED) {
-            const sfb_uint2 here = lut[lut_off + j];
-            const int limit = valid - (int)(here.y * BS);
-            if ((mask != nullptr) || (limit < BS))
-                apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit), half);
-        }
-        const float mloc = block_row_max<KT>(s);
-        st.m_true = fmaxf(st.m_true, mloc);
-        if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
-            const float m_new = fmaxf(st.m_used, mloc);
-            const float alpha = exp2_fast((st.m_used - m_new) * c);
-            st.m_used = m_new;
-            st.l *= alpha;
-#pragma unroll
-            for (int n = 0; n < NO; ++n) o_acc[n] *= alpha;
-        }
-        const float mc = st.m_used * c;
-        float sum0 = 0.f, sum1 = 0.f;
-        uint32_t pk[KT * 8];
-        exp_chunk<KT, NO>(s, pk, 0, c, mc, sum0, sum1);
-#pragma unroll
-        for (int u = 0; u < PU; ++u) {
-            if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
-            // a slice of the next block's scores with every chunk keeps the MFMA pipe fed evenly
-#pragma unroll
-            for (int ks = u * (KS / PU); ks < (u + 1) * (KS / PU); ++ks)
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-                    if (ks == 0) {
-                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, kt, ks, qn, half), qf[ks], zero, 0, 0, 0);
-                    } else {
-                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, kt, ks, qn, half), qf[ks], s_next[kt], 0, 0, 0);
-                    }
-                }
-            const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
-            const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
-#pragma unroll
-            for (int mt = 0; mt < NO; ++mt)
-                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(v_read, mt, u, qn, half), bfrag,
-                                                                    o_acc[mt], 0, 0, 0);
-        }
-        st.l += sum0 + sum1;
-        __syncthreads();
-    };
-
-    for (uint32_t j = 0; j < count; j += 2) {
-        iteration(j, gk0, gv0, s_even, s_odd);
-        if (j + 1 < count) iteration(j + 1, gk1, gv1, s_odd, s_even);
-    }
-
-    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
-}
-
-// ------------------------------------------------------------------------------------------------
-// bf16 inputs, tiles copied memory -> LDS without passing through registers
-// ------------------------------------------------------------------------------------------------
-// Same arithmetic as the kernel above with a leaner instruction stream: K and V tiles of a key block are
-// fetched with LDS-direct loads into swizzled row-major buffers (see Bf16DirectTiles), V^T fragments come
-// from transposing LDS reads.  In iteration j a wave
+// K and V tiles of a key block are fetched with LDS-direct loads into swizzled row-major buffers (see
+// Bf16DirectTiles; no staging registers, no LDS writes by the waves), V^T fragments come from transposing
+// LDS reads.  Software pipeline over the key blocks of the item; in iteration j a wave
 //   * issues the loads of K(j+2) and V(j+1) into the buffers that iteration j-1 finished reading;
 //   * finds the row maximum of S(j), then, chunk by chunk, exponentiates S(j), feeds V(j)^T . P^T and
 //     computes a slice of S(j+1) = K(j+1) . Q^T;
 //   * waits for its own loads and meets the other waves at the one barrier of the iteration.
 template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(FusedParams p) {
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
     constexpr int TILE = T::TILE_BYTES;
@@ -469,7 +309,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_direct_kernel(
     const uint32_t row_bytes = p.heads * D * 2;
 
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
-    const uint32_t lut_off = __builtin_amdgcn_readfirstlane(lut[w.row].x + w.first);
+    const uint32_t lut_off = __builtin_amdgcn_readfirstlane(w.lut_first);
     const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
     float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
 
@@ -634,7 +474,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedPar
     const uint32_t row_stride = p.heads * D;
 
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
-    const uint32_t lut_off = lut[w.row].x + w.first, count = w.count;
+    const uint32_t lut_off = w.lut_first, count = w.count;
     float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
 
     if (count == 0) {
@@ -717,19 +557,12 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedPar
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
 }
 
-static int g_variant = getenv("SFB_VARIANT") ? atoi(getenv("SFB_VARIANT")) : 1;
-
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
     const uint32_t grid = p.groups * 8u * ranks;
     clear_stale_error();
-    if (in_dtype == SFB_BF16 && g_variant == 1) {
-        if (p.mask || p.valid_len)
-            fused_attention_bf16_direct_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-        else
-            fused_attention_bf16_direct_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-    } else if (in_dtype == SFB_BF16) {
+    if (in_dtype == SFB_BF16) {
         if (p.mask || p.valid_len)
             fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
         else
