@@ -177,6 +177,23 @@ def test_c4_scheduled_full_size():
     assert rel_err(got, plain) <= 5e-3  # split rows: probabilities are rounded to bf16 relative to per-chunk maxima
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("scheduled", [False, True])
+def test_rows_longer_than_64_key_blocks(bf16, scheduled):
+    """Dense layout with 80 key blocks per row: a work-group walks more LUT entries than one wave holds
+    (the bf16 kernel keeps 64 entries in registers and fetches the next window on the way)."""
+    bs, nb, B, H, d = 64, 80, 1, 2, 64
+    L = bs * nb
+    luts = sfb.build_luts(PATTERNS["full"](nb))
+    valid = np.array([L - 37], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=131, bf16=bf16)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, valid_len=valid, nthreads=THREADS)
+    got = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, valid_len=valid, max_blocks=1000 if scheduled else None)
+    check(got, want, TOL_BF16 if bf16 else TOL_F32)
+    got = run_fused(Q, K, V, luts, bs, 0.125, bf16=bf16, max_blocks=1000 if scheduled else None)
+    check(got, orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS), TOL_BF16 if bf16 else TOL_F32)
+
+
 def test_scale_and_large_scores():
     # scores far from zero: the running maximum and the 1e-6 term must still follow the oracle
     bs, nb, B, H, d = 64, 4, 1, 2, 64
