@@ -110,7 +110,7 @@ __global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// masked softmax: one wave per query row, lanes = keys (64/BS blocks per step)
+// masked softmax: one wave per query row, 8 consecutive keys per lane (8 or 16 key blocks per wave step)
 // (blocksparse.h:459-722 keeps one CTA per query row; the row-major mask order is the same)
 // ---------------------------------------------------------------------------------------------
 struct SoftmaxParams {
@@ -125,7 +125,9 @@ struct SoftmaxParams {
 
 template <int BS, typename TX, typename TY>
 __global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
-    constexpr int PER = 64 / BS;  // blocks covered by one wave step
+    constexpr int LPB = BS / 8;     // lanes per key block: every lane owns 8 consecutive keys (16 or 32 bytes)
+    constexpr int PER = 64 / LPB;   // key blocks covered by one wave step
+    constexpr int CACHE = 8;        // steps whose scores stay in registers (64 blocks at BS 64)
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint64_t row_id = (uint64_t)blockIdx.x * 4 + wave;        // over batch*heads*nb*BS
     const uint64_t total_rows = (uint64_t)p.batch * p.heads * p.nb * BS;
@@ -136,47 +138,120 @@ __global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
     const uint32_t b = bh / p.heads, h = bh % p.heads;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
     const uint32_t off = lut[r].x, count = lut[r].y;
-    const uint32_t sub = lane / BS, key = lane % BS;
+    const uint32_t sub = lane / LPB, key0 = (lane % LPB) * 8;
     const TX* x = (const TX*)p.x + (size_t)bh * p.blocks * BS * BS;
     TY* y = (TY*)p.y + (size_t)bh * p.blocks * BS * BS;
     const int valid = p.valid_len ? p.valid_len[b] : (int)(p.nb * BS);
     const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
     const float c = p.scale_log2e;
 
-    auto kept = [&](const sfb_uint2 e) -> bool {
-        bool k = (int)(e.y * BS + key) < valid;
+    // keep bits of this lane's 8 keys in key block e
+    auto keep_bits = [&](const sfb_uint2 e) -> uint32_t {
+        const int left = valid - (int)(e.y * BS + key0);
+        uint32_t k = left >= 8 ? 0xffu : (left <= 0 ? 0u : ((1u << left) - 1u));
         if (mask) {
             const size_t w = (size_t)qi * p.blocks + e.x;
             const uint64_t word = (BS == 64) ? ((const uint64_t*)mask)[w] : ((const uint32_t*)mask)[w];
-            k = k && ((word >> key) & 1ull);
+            k &= (uint32_t)(word >> key0);
         }
         return k;
     };
+    auto load8 = [&](const sfb_uint2 e, float (&v)[8]) {
+        const TX* src = x + ((size_t)e.x * BS + qi) * BS + key0;
+        const f32x4 lo = Elem<TX>::load4(src), hi = Elem<TX>::load4(src + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    };
+    auto store8 = [&](const sfb_uint2 e, const float (&v)[8]) {
+        TY* dst = y + ((size_t)e.x * BS + qi) * BS + key0;
+        const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        Elem<TY>::store4(dst, lo);
+        Elem<TY>::store4(dst + 4, hi);
+    };
+    auto wave_max = [](float m) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+        return m;
+    };
+    auto wave_sum = [](float l) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+        return l;
+    };
 
-    // pass 1: row maximum over kept keys (seed as ewops.h:70), then the sum relative to it
+    const uint32_t steps = (count + PER - 1) / PER;
+    if (steps <= CACHE) {
+        // the whole row fits in registers: one read, one write.  Maximum over kept keys (seed as
+        // ewops.h:70), sum relative to it, normalised probabilities with zeros at masked keys (ewops.h:82)
+        float v[CACHE][8];
+        uint32_t keep[CACHE];
+        sfb_uint2 ent[CACHE];
+        float m = kMaxSeed;
+#pragma unroll
+        for (int st = 0; st < CACHE; ++st) {
+            const uint32_t j = st * PER + sub;
+            keep[st] = 0;
+            if (j < count) {
+                ent[st] = lut[off + j];
+                load8(ent[st], v[st]);
+                keep[st] = keep_bits(ent[st]) | 0x100u;   // bit 8: the block exists
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if ((keep[st] >> i) & 1u) m = fmaxf(m, v[st][i]);
+            }
+        }
+        m = wave_max(m);
+        float l = 0.f;
+#pragma unroll
+        for (int st = 0; st < CACHE; ++st)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float e = ((keep[st] >> i) & 1u) ? exp2_fast((v[st][i] - m) * c) : 0.f;
+                v[st][i] = e;
+                l += e;
+            }
+        l = wave_sum(l);
+        const float inv = 1.0f / (l + 1e-6f);
+#pragma unroll
+        for (int st = 0; st < CACHE; ++st)
+            if (keep[st] & 0x100u) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[st][i] *= inv;
+                store8(ent[st], v[st]);
+            }
+        return;
+    }
+    // longer rows: three passes over memory
     float m = kMaxSeed;
     for (uint32_t j = sub; j < count; j += PER) {
         const sfb_uint2 e = lut[off + j];
-        const float v = Elem<TX>::load(x + ((size_t)e.x * BS + qi) * BS + key);
-        if (kept(e)) m = fmaxf(m, v);
-    }
+        float v[8];
+        load8(e, v);
+        const uint32_t k = keep_bits(e);
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+        for (int i = 0; i < 8; ++i)
+            if ((k >> i) & 1u) m = fmaxf(m, v[i]);
+    }
+    m = wave_max(m);
     float l = 0.f;
     for (uint32_t j = sub; j < count; j += PER) {
         const sfb_uint2 e = lut[off + j];
-        const float v = Elem<TX>::load(x + ((size_t)e.x * BS + qi) * BS + key);
-        if (kept(e)) l += exp2_fast((v - m) * c);
-    }
+        float v[8];
+        load8(e, v);
+        const uint32_t k = keep_bits(e);
 #pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+        for (int i = 0; i < 8; ++i)
+            if ((k >> i) & 1u) l += exp2_fast((v[i] - m) * c);
+    }
+    l = wave_sum(l);
     const float inv = 1.0f / (l + 1e-6f);
-    // pass 2: normalised probabilities, zeros at masked keys (ewops.h:82)
     for (uint32_t j = sub; j < count; j += PER) {
         const sfb_uint2 e = lut[off + j];
-        const size_t at = ((size_t)e.x * BS + qi) * BS + key;
-        const float v = Elem<TX>::load(x + at);
-        Elem<TY>::store(y + at, kept(e) ? exp2_fast((v - m) * c) * inv : 0.f);
+        float v[8];
+        load8(e, v);
+        const uint32_t k = keep_bits(e);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = ((k >> i) & 1u) ? exp2_fast((v[i] - m) * c) * inv : 0.f;
+        store8(e, v);
     }
 }
 
@@ -396,6 +471,7 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)x | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
     SoftmaxParams p = {lut, mask, valid_len, x, y, blocks, batch_dim, head_dim, ctx_blks,
                        lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0, scale * kLog2e};
     const uint64_t rows = (uint64_t)batch_dim * head_dim * ctx_blks * block_size;
