@@ -220,6 +220,13 @@ int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, float* mean, fl
 /* tensor_add_matrix (ewops.h:276-282; cuda_kernels.h:526-535): out[b][i] = a[b][i] + m[i]. */
 int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, const float* m, uint32_t dim0,
                    uint64_t inner);
+/* MI355X addition: bias + tensor_add_tensor + layernorm (ewops.h:10-17, 296-301, layernorm.h:13-38) in one
+ * pass over memory: out = LayerNorm((in + bias[col]) + residual), same arithmetic and order as
+ * sfb_bias_act followed by sfb_layernorm.  bias, residual may be NULL; out_bf16 [dev] optional second copy
+ * of the result rounded to bf16 (NULL = none); state % 4 == 0, state <= 2048; out may alias in. */
+int sfb_bias_residual_layernorm(sfb_stream_t stream, float* out, void* out_bf16, const float* in,
+                                const float* bias, const float* residual, const float* gain, const float* beta,
+                                uint32_t rows, uint32_t state);
 /* embedding_lookup (embedding.h:5-12; cuda_kernels.h:210-221), optionally fused with the position add:
  * out[t] = table[ids[t]] (+ pos[t % seq_len]); pos may be NULL. */
 int sfb_embedding_lookup(sfb_stream_t stream, float* out, const float* table, const int32_t* ids,

@@ -58,7 +58,7 @@ EXPORTED = [
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
-    "sfb_bias_act", "sfb_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
+    "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
 ]
 
@@ -376,6 +376,19 @@ def layernorm(x, gain, beta, out_dtype=F32, return_stats=False):
     _check(lib.sfb_layernorm(_stream(), _dev(out), _dtype_code(out), _dev(mean), _dev(rstd), _dev(x),
                              _dev(gain), _dev(beta), C.c_uint32(rows), C.c_uint32(state)), "sfb_layernorm")
     return (out, mean, rstd) if return_stats else out
+
+
+def bias_residual_layernorm(x, bias, residual, gain, beta, with_bf16=False):
+    """LayerNorm((x + bias) + residual) in one pass; returns out fp32 (and a bf16 copy)."""
+    import torch
+    state = x.shape[-1]
+    rows = x.numel() // state
+    out = torch.empty(x.shape, device=x.device, dtype=torch.float32)
+    out16 = torch.empty(x.shape, device=x.device, dtype=torch.bfloat16) if with_bf16 else None
+    _check(lib.sfb_bias_residual_layernorm(_stream(), _dev(out), _dev(out16), _dev(x), _dev(bias), _dev(residual),
+                                           _dev(gain), _dev(beta), C.c_uint32(rows), C.c_uint32(state)),
+           "sfb_bias_residual_layernorm")
+    return (out, out16) if with_bf16 else out
 
 
 def tensor_add_matrix(a, m):

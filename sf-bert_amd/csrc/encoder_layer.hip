@@ -114,20 +114,36 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     const void* ain = attn;
     if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, attn, m * n)); ain = xa; }
     SFB_TRY(sfb_gemm(stream, t, ain, wt->wo, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, t, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_layernorm(stream, x1, SFB_F32, nullptr, nullptr, t, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
+    // bias + residual + LayerNorm 1 in one pass when the row fits in registers; the bf16 path gets its
+    // copy of x1 for the next GEMM from the same kernel
+    const bool fused_ln = n <= 2048;
+    if (fused_ln) {
+        SFB_TRY(sfb_bias_residual_layernorm(stream, x1, bf ? xa : nullptr, t, wt->bo, x, wt->ln1_g, wt->ln1_b,
+                                            (uint32_t)m, (uint32_t)n));
+    } else {
+        SFB_TRY(sfb_bias_act(stream, t, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
+        SFB_TRY(sfb_layernorm(stream, x1, SFB_F32, nullptr, nullptr, t, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
+    }
 
     // FFN: GEMM, bias + sigmoid-GELU, GEMM, bias + residual, LayerNorm 2
     const void* fin = x1;
-    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x1, m * n)); fin = xa; }
+    if (bf) {
+        if (!fused_ln) SFB_TRY(sfb_cast_f32_bf16(stream, xa, x1, m * n));
+        fin = xa;
+    }
     SFB_TRY(sfb_gemm(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
     void* g = bf ? xa : (void*)t;   // activation after GELU, in the compute dtype (in place for fp32)
     SFB_TRY(sfb_bias_act(stream, g, dtype, t, wt->b1, nullptr, 1, m, ffn));
     // the second FFN GEMM reads g and must not write over it: fp32 writes into attn's buffer
     float* t2 = bf ? t : attn;
     SFB_TRY(sfb_gemm(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn));
-    SFB_TRY(sfb_bias_act(stream, t2, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_layernorm(stream, y, SFB_F32, nullptr, nullptr, t2, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
+    if (fused_ln) {
+        SFB_TRY(sfb_bias_residual_layernorm(stream, y, nullptr, t2, wt->b2, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m,
+                                            (uint32_t)n));
+    } else {
+        SFB_TRY(sfb_bias_act(stream, t2, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
+        SFB_TRY(sfb_layernorm(stream, y, SFB_F32, nullptr, nullptr, t2, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
+    }
 #undef SFB_TRY
     return SFB_OK;
 }

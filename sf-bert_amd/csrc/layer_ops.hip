@@ -73,6 +73,55 @@ __global__ __launch_bounds__(256) void layernorm_kernel(TOut* out, float* mean_o
     }
 }
 
+// y = LayerNorm((in + bias) + residual) in one pass over memory: the row stays in registers between
+// the sums and the normalisation (one wave per row, VECS float4 per lane).  Same arithmetic, in the same
+// order, as bias_act_kernel followed by layernorm_kernel.  Optionally also writes y rounded to bf16.
+template <int VECS>
+__global__ __launch_bounds__(256) void bias_residual_layernorm_kernel(float* out, __bf16* out_bf16, const float* in,
+                                                                      const float* bias, const float* residual,
+                                                                      const float* gain, const float* beta,
+                                                                      uint32_t rows, uint32_t state) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const uint32_t vecs = state / 4;
+    const f32x4* x = (const f32x4*)(in + (size_t)row * state);
+    const f32x4* r = residual ? (const f32x4*)(residual + (size_t)row * state) : nullptr;
+    f32x4 v[VECS];
+    float sum = 0.f, sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < VECS; ++k) {
+        const uint32_t i = lane + 64 * k;
+        if (i < vecs) {
+            f32x4 t = x[i];
+            if (bias) t += ((const f32x4*)bias)[i];
+            if (r) t += r[i];
+            v[k] = t;
+            sum += (t.x + t.y) + (t.z + t.w);
+            sq += (t.x * t.x + t.y * t.y) + (t.z * t.z + t.w * t.w);
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        sum += __shfl_xor(sum, d);
+        sq += __shfl_xor(sq, d);
+    }
+    const float mean = sum / (float)state;
+    const float var = sq / (float)state - mean * mean;
+    const float rstd = 1.0f / sqrtf(var + 1e-5f);
+#pragma unroll
+    for (int k = 0; k < VECS; ++k) {
+        const uint32_t i = lane + 64 * k;
+        if (i < vecs) {
+            const f32x4 t = v[k], g = ((const f32x4*)gain)[i], b = ((const f32x4*)beta)[i];
+            const f32x4 y = {((t.x - mean) * rstd) * g.x + b.x, ((t.y - mean) * rstd) * g.y + b.y,
+                             ((t.z - mean) * rstd) * g.z + b.z, ((t.w - mean) * rstd) * g.w + b.w};
+            store_out(out + (size_t)row * state + i * 4, y);
+            if (out_bf16) store_out(out_bf16 + (size_t)row * state + i * 4, y);
+        }
+    }
+}
+
 // out[b][i] = a[b][i] + m[i]  (ewops.h:276-282: position embedding broadcast over the batch)
 __global__ __launch_bounds__(256) void add_matrix_kernel(float* out, const float* a, const float* m,
                                                          uint64_t vecs, uint64_t inner4) {
@@ -141,6 +190,27 @@ extern "C" int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, floa
         layernorm_kernel<float><<<grid, 256, 0, s>>>((float*)out, mean, rstd, in, gain, bias, rows, state);
     else
         layernorm_kernel<__bf16><<<grid, 256, 0, s>>>((__bf16*)out, mean, rstd, in, gain, bias, rows, state);
+    return launched();
+}
+
+extern "C" int sfb_bias_residual_layernorm(sfb_stream_t stream, float* out, void* out_bf16, const float* in,
+                                          const float* bias, const float* residual, const float* gain,
+                                          const float* beta, uint32_t rows, uint32_t state) {
+    if (!out || !in || !gain || !beta) return SFB_ERR_NULL_POINTER;
+    if (rows == 0 || state == 0 || (state & 3u) || state > 64u * 4u * 8u) return SFB_ERR_SHAPE;
+    if (((uintptr_t)out | (uintptr_t)in | (uintptr_t)bias | (uintptr_t)residual | (uintptr_t)gain | (uintptr_t)beta) & 15u)
+        return SFB_ERR_ALIGNMENT;
+    if ((uintptr_t)out_bf16 & 7u) return SFB_ERR_ALIGNMENT;
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+    const dim3 grid((rows + 3) / 4);
+    const uint32_t vecs_per_lane = (state / 4 + 63) / 64;
+#define SFB_BRL(V) bias_residual_layernorm_kernel<V><<<grid, 256, 0, s>>>(out, (__bf16*)out_bf16, in, bias, residual, gain, beta, rows, state)
+    if (vecs_per_lane <= 1) SFB_BRL(1);
+    else if (vecs_per_lane <= 2) SFB_BRL(2);
+    else if (vecs_per_lane <= 4) SFB_BRL(4);
+    else SFB_BRL(8);
+#undef SFB_BRL
     return launched();
 }
 

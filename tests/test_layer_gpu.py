@@ -33,6 +33,29 @@ def test_layer_ops_match_oracle():
     assert rel_err(ln_bf16, want) <= 4e-3
 
 
+@pytest.mark.parametrize("state", [64, 768, 1024, 2048])
+def test_bias_residual_layernorm_one_pass(state):
+    """The fused kernel equals bias -> tensor_add_tensor -> layernorm of the oracle, and bit for bit the
+    two-kernel sequence of the library; its bf16 copy is the fp32 result rounded to nearest even."""
+    rows = 131
+    x = orc.fill_normal((rows, state), 11) * 1.5
+    res = orc.fill_normal((rows, state), 12) + 0.2
+    bias = orc.fill_normal((state,), 13)
+    g = orc.fill_normal((state,), 14) + 1
+    b = orc.fill_normal((state,), 15)
+    want, _, _ = orc.layernorm(orc.bias(x, bias) + res, g, b)
+    got, got16 = sfb.bias_residual_layernorm(T(x), T(bias), T(res), T(g), T(b), with_bf16=True)
+    assert rel_err(got.cpu().numpy(), want) <= 1e-5
+    two = sfb.layernorm(sfb.bias_act(T(x), bias=T(bias), residual=T(res)), T(g), T(b))
+    assert np.array_equal(got.cpu().numpy(), two.cpu().numpy())
+    assert np.array_equal(got16.float().cpu().numpy(), orc.round_bf16(got.cpu().numpy()))
+    plain = sfb.bias_residual_layernorm(T(x), None, None, T(g), T(b))
+    assert rel_err(plain.cpu().numpy(), orc.layernorm(x, g, b)[0]) <= 1e-5
+    with pytest.raises(sfb.SfbError):
+        sfb.bias_residual_layernorm(T(orc.fill_normal((4, 4096), 1)), None, None, T(orc.fill_normal((4096,), 2)),
+                                    T(orc.fill_normal((4096,), 3)))
+
+
 def test_embedding_and_position_add():
     vocab, state, B, L = 1000, 768, 3, 64
     table = orc.fill_normal((vocab, state), 5)
