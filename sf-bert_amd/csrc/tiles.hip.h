@@ -1,4 +1,4 @@
-// LDS tile staging and MFMA fragment access shared by the attention kernels.
+// LDS tiles and MFMA fragment access shared by the attention kernels.
 //
 // A work-group of NT = 2*BS threads (BS/32 waves, each owning 32 query rows) walks key blocks of BS
 // keys.  Lane l of a wave is query column qn = l % 32 and half = l / 32 of the 32x32 MFMA shapes.
@@ -16,90 +16,8 @@
 namespace sfb {
 
 // ------------------------------------------------------------------------------------------------
-// bf16 operands, v_mfma_f32_32x32x16_bf16 (8 bf16 per lane per step: k-slots half*8 .. half*8+7)
-// ------------------------------------------------------------------------------------------------
-// K tile in LDS: [BS keys][D + 8] bf16 row-major; the 16-byte pad makes the 128-bit fragment reads
-//   conflict-free.  Score k-slot (ks, half, j) is head-dimension index (2ks + half)*8 + j.
-// V tile in LDS: transposed, [D][BS + 8] bf16, and inside a row the 4-key groups are stored in the
-//   order the P^T operand holds them: product step u, half hf, slot j is key 16u + 8(j/4) + 4hf + j%4,
-//   i.e. group g = 4u + 2a + hf (a = j/4) lives at byte (2u + hf)*16 + a*8.
-template <int BS, int D>
-struct Bf16Tiles {
-    static constexpr int NT = BS * 2;
-    static constexpr int K_STRIDE = (D + 8) * 2;   // bytes
-    static constexpr int V_STRIDE = (BS + 8) * 2;  // bytes
-    static constexpr int K_BYTES = BS * K_STRIDE;
-    static constexpr int V_BYTES = D * V_STRIDE;
-    static constexpr int K_CHUNKS = D / 16;         // 16-byte chunks of K per thread
-    static constexpr int V_ITEMS = D / 64;          // (4 keys x 8 columns) items of V per thread
-    static_assert(D % 64 == 0, "head state must be a multiple of 64");
-
-    struct KRegs { u32x4 g[K_CHUNKS]; };
-    struct VRegs { u32x4 g[V_ITEMS][4]; };
-
-    // base: element offset of (b, first token of the key block, h, 0); row_stride = heads * D.
-    static __device__ __forceinline__ void fetch_k(KRegs& r, const __bf16* K, size_t base,
-                                                   uint32_t row_stride, uint32_t t) {
-#pragma unroll
-        for (int i = 0; i < K_CHUNKS; ++i) {
-            const uint32_t cid = i * NT + t, row = cid / (D / 8), c = cid % (D / 8);
-            r.g[i] = *(const u32x4*)(K + base + (size_t)(row * row_stride + c * 8));
-        }
-    }
-    static __device__ __forceinline__ void stage_k(uint8_t* k_lds, const KRegs& r, uint32_t t) {
-#pragma unroll
-        for (int i = 0; i < K_CHUNKS; ++i) {
-            const uint32_t cid = i * NT + t, row = cid / (D / 8), c = cid % (D / 8);
-            *(u32x4*)(k_lds + row * K_STRIDE + c * 16) = r.g[i];
-        }
-    }
-    static __device__ __forceinline__ void fetch_v(VRegs& r, const __bf16* V, size_t base,
-                                                   uint32_t row_stride, uint32_t t) {
-#pragma unroll
-        for (int ii = 0; ii < V_ITEMS; ++ii) {
-            const uint32_t id = ii * NT + t, g = id % (BS / 4), c = id / (BS / 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                r.g[ii][e] = *(const u32x4*)(V + base + (size_t)((4 * g + e) * row_stride + c * 8));
-        }
-    }
-    // 4 keys x 8 columns per item -> 8 (column, 4-key group) pairs of 8 bytes.
-    static __device__ __forceinline__ void stage_v(uint8_t* v_lds, const VRegs& r, uint32_t t) {
-#pragma unroll
-        for (int ii = 0; ii < V_ITEMS; ++ii) {
-            const uint32_t id = ii * NT + t, g = id % (BS / 4), c = id / (BS / 4);
-            const uint32_t pos = (2 * (g / 4) + (g & 1)) * 16 + ((g & 3) >> 1) * 8;
-#pragma unroll
-            for (int dd = 0; dd < 8; ++dd) {
-                const uint32_t x0 = r.g[ii][0][dd / 2], x1 = r.g[ii][1][dd / 2];
-                const uint32_t x2 = r.g[ii][2][dd / 2], x3 = r.g[ii][3][dd / 2];
-                // byte select over {second, first}: low halves (even column) or high halves (odd column)
-                const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
-                u32x2 out;
-                out.x = __builtin_amdgcn_perm(x1, x0, sel);
-                out.y = __builtin_amdgcn_perm(x3, x2, sel);
-                *(u32x2*)(v_lds + (c * 8 + dd) * V_STRIDE + pos) = out;
-            }
-        }
-    }
-    static __device__ __forceinline__ bf16x8 k_frag(const uint8_t* k_lds, int kt, int ks, uint32_t qn,
-                                                    uint32_t half) {
-        return *(const bf16x8*)(k_lds + (kt * 32 + qn) * K_STRIDE + (2 * ks + half) * 16);
-    }
-    static __device__ __forceinline__ bf16x8 v_frag(const uint8_t* v_lds, int mt, int u, uint32_t qn,
-                                                    uint32_t half) {
-        return *(const bf16x8*)(v_lds + (mt * 32 + qn) * V_STRIDE + (2 * u + half) * 16);
-    }
-    // Q^T operand of one query row, kept in registers: D/16 steps of 8 bf16.
-    static __device__ __forceinline__ void load_q(bf16x8 (&qf)[D / 16], const __bf16* q_row,
-                                                  uint32_t half) {
-#pragma unroll
-        for (int ks = 0; ks < D / 16; ++ks) qf[ks] = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
-    }
-};
-
-// ------------------------------------------------------------------------------------------------
-// bf16 operands, tiles copied from memory straight into LDS (global_load_lds_dwordx4)
+// bf16 operands, v_mfma_f32_32x32x16_bf16 (8 bf16 per lane per step: k-slots half*8 .. half*8+7);
+// tiles copied from memory straight into LDS (global_load_lds_dwordx4)
 // ------------------------------------------------------------------------------------------------
 // K and V tiles are both kept row-major, [BS keys][D] bf16 = 128-byte rows of eight 16-byte chunks, with
 // no padding: an LDS-direct load writes the 64 lanes' 16 bytes back to back (1 KiB = 8 rows per

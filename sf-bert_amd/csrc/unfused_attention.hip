@@ -270,20 +270,21 @@ template <int BS, int D, typename TP, typename TV>
 __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int KT = BS / 32, NO = D / 32;
     constexpr bool kBf16 = sizeof(TV) == 2;
-    using TB = Bf16Tiles<BS, D>;
+    using TD = Bf16DirectTiles<BS, D>;
     using TF = F32Tiles<BS, D>;
-    constexpr int LDS_BYTES = kBf16 ? TB::V_BYTES : TF::V_FLOATS * 4;
-    __shared__ __attribute__((aligned(16))) uint8_t smem[LDS_BYTES];
+    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
     const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
     const uint32_t r = p.nb_c - 1 - work.rank;   // long rows of causal layouts first (blocksparse.h:746-748)
-    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
     const uint32_t row_stride = p.heads * D;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
-    const uint32_t off = lut[r].x, count = lut[r].y;
+    const uint32_t off = __builtin_amdgcn_readfirstlane(lut[r].x), count = __builtin_amdgcn_readfirstlane(lut[r].y);
     float* o_row = p.c + token_offset(b, r * BS + q_in_block, h, p.nb_c * BS, p.heads, D);
     const TP* P = (const TP*)p.a + (size_t)work.bh * p.blocks * BS * BS;
     const TV* V = (const TV*)p.b;
@@ -294,29 +295,104 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
 
-    for (uint32_t j = 0; j < count; ++j) {
-        const sfb_uint2 e = lut[off + j];
-        const size_t base = token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
-        const TP* p_row = P + ((size_t)e.x * BS + q_in_block) * BS;
-        if constexpr (kBf16) {
-            typename TB::VRegs gv;
-            TB::fetch_v(gv, (const __bf16*)V, base, row_stride, t);
-            TB::stage_v(smem, gv, t);
-            __syncthreads();
+    if constexpr (kBf16 && sizeof(TP) == 2 && BS == 64) {
+        // bf16 P and V: both tiles of a key block go straight into LDS (LDS-direct loads, double-buffered,
+        // swizzled rows, see Bf16DirectTiles); V^T fragments by transposing reads, P^T fragments by two 8-byte
+        // reads per product step.  One barrier per key block, loads of the next block in flight meanwhile.
+        constexpr int PU = BS / 16, TILE = TD::TILE_BYTES;
+        static_assert(BS == 64 || BS == 32, "block size");
+        const uint32_t row_bytes = row_stride * 2;
+        const uint32_t v_even = TD::lane_source(lane, 0, row_bytes), v_odd = TD::lane_source(lane, 1, row_bytes);
+        const uint32_t p_even = TD::lane_source(lane, 0, BS * 2), p_odd = TD::lane_source(lane, 1, BS * 2);
+        const uint32_t lds0 = TD::lds_address(smem), v_lane = TD::v_lane_base(lane);
+        const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
+        const uint8_t* const p_base = (const uint8_t*)P;
+        // P tile rows are BS bf16 = BS*2 bytes: 128-byte rows for BS 64 (the V layout), 64-byte rows for BS 32
+        // (two P rows per 128-byte LDS row; handled by the generic path below)
+        auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
+            TD::load_tile(lds0 + buf * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, v_even, v_odd, row_bytes);
+            TD::load_tile(lds0 + (2 + buf) * TILE, p_base + (size_t)e.x * BS * BS * 2, wave, p_even, p_odd, BS * 2);
+        };
+        auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
+            const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
+            return u;
+        };
+        if (count > 0) fetch(uniform(lut[off]), 0);
+        // P^T operand of step u: keys 16u + 8(j/4) + 4*half + j%4 of query row q_in_block: 8 bytes of chunk 2u
+        // and 8 bytes of chunk 2u + 1 of that row, at byte 8*half
+        const uint32_t p_row = q_in_block * 128u + half * 8u, p_swz = TD::swz(q_in_block) << 4;
+        for (uint32_t j = 0; j < count; ++j) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();   // tiles of block j are in LDS for every wave, and every wave is done with block j-1
+            fetch(uniform(lut[off + (j + 1 < count ? j + 1 : j)]), (j + 1) & 1);
+            const uint8_t* v_read = smem + (j & 1) * TILE;
+            const uint8_t* p_read = smem + (2 + (j & 1)) * TILE + p_row;
 #pragma unroll
-            for (int u = 0; u < BS / 16; ++u) {
-                // slots j: key 16u + 8(j/4) + 4*half + j%4
-                const f32x4 lo = Elem<TP>::load4(p_row + 16 * u + 4 * half);
-                const f32x4 hi = Elem<TP>::load4(p_row + 16 * u + 8 + 4 * half);
+            for (int u = 0; u < PU; ++u) {
+                const u32x2 lo = *(const u32x2*)(p_read + ((uint32_t)(2 * u * 16) ^ p_swz));
+                const u32x2 hi = *(const u32x2*)(p_read + ((uint32_t)((2 * u + 1) * 16) ^ p_swz));
+                const u32x4 pb = {lo.x, lo.y, hi.x, hi.y};
+                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u), bfrag,
+                                                                        o_acc[mt], 0, 0, 0);
+            }
+        }
+    } else if constexpr (kBf16) {
+        // V tiles double-buffered in LDS by LDS-direct loads, V^T fragments by transposing reads (see
+        // Bf16DirectTiles); the P values of the next block are fetched into registers while this one is
+        // multiplied.  One barrier per key block.
+        constexpr int PU = BS / 16;
+        const uint32_t row_bytes = row_stride * 2;
+        const uint32_t src_even = TD::lane_source(lane, 0, row_bytes), src_odd = TD::lane_source(lane, 1, row_bytes);
+        const uint32_t lds0 = TD::lds_address(smem), v_lane = TD::v_lane_base(lane);
+        const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
+        // slots j of product step u: keys 16u + 8(j/4) + 4*half + j%4
+        f32x4 pc[2 * PU], pn[2 * PU];
+        auto fetch_p = [&](f32x4 (&dst)[2 * PU], uint32_t blk) {
+            const TP* p_row = P + ((size_t)blk * BS + q_in_block) * BS;
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                dst[2 * u] = Elem<TP>::load4(p_row + 16 * u + 4 * half);
+                dst[2 * u + 1] = Elem<TP>::load4(p_row + 16 * u + 8 + 4 * half);
+            }
+        };
+        auto fetch_v = [&](uint32_t col, uint32_t buf) {
+            TD::load_tile(lds0 + buf * TD::TILE_BYTES, v_base + (size_t)col * BS * row_bytes, wave, src_even, src_odd,
+                          row_bytes);
+        };
+        if (count > 0) {
+            const sfb_uint2 e0 = lut[off];
+            fetch_v(__builtin_amdgcn_readfirstlane(e0.y), 0);
+            fetch_p(pc, __builtin_amdgcn_readfirstlane(e0.x));
+        }
+        for (uint32_t j = 0; j < count; ++j) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();   // V(j) is in LDS for every wave, and every wave is done with V(j-1)
+            const sfb_uint2 en = lut[off + (j + 1 < count ? j + 1 : j)];
+            fetch_v(__builtin_amdgcn_readfirstlane(en.y), (j + 1) & 1);
+            fetch_p(pn, __builtin_amdgcn_readfirstlane(en.x));
+            const uint8_t* v_read = smem + (j & 1) * TD::TILE_BYTES;
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                const f32x4 lo = pc[2 * u], hi = pc[2 * u + 1];
                 const u32x4 pb = {pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y),
                                   pack_bf16(hi.z, hi.w)};
                 const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
                 for (int mt = 0; mt < NO; ++mt)
-                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TB::v_frag(smem, mt, u, qn, half), bfrag,
+                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u), bfrag,
                                                                         o_acc[mt], 0, 0, 0);
             }
-        } else {
+#pragma unroll
+            for (int x = 0; x < 2 * PU; ++x) pc[x] = pn[x];
+        }
+    } else {
+        for (uint32_t j = 0; j < count; ++j) {
+            const sfb_uint2 e = lut[off + j];
+            const size_t base = token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
+            const TP* p_row = P + ((size_t)e.x * BS + q_in_block) * BS;
             float* v_lds = (float*)smem;
             typename TF::Regs gv;
             TF::fetch(gv, (const float*)V, base, row_stride, t);
@@ -334,8 +410,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
                             o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                                 TF::v_elem(v_lds, kt, ig * 4 + e4, mt, qn, half), pv[e4], o_acc[mt], 0, 0, 0);
                 }
+            __syncthreads();
         }
-        __syncthreads();
     }
     // block-rows without blocks write zeros (blocksparse.h:949-962)
 #pragma unroll
