@@ -64,13 +64,17 @@ struct Bf16DirectTiles {
         uint32_t src;
         if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
         else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
-        // the uniform part goes through readfirstlane so that it stays in scalar registers
+        // scalar 64-bit base + 32-bit lane offset: no vector address arithmetic.  The instruction takes its
+        // LDS destination from M0, which is written here; nothing else in these kernels depends on M0.
         const uint64_t ga = (uint64_t)(g_tile + (size_t)n * 8u * row_bytes);
         const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
         const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
-        const uint8_t* g = (const uint8_t*)(((uint64_t)ga_hi << 32) | (uint64_t)ga_lo);
-        __builtin_amdgcn_global_load_lds((const uint32_t*)(g + src), (lds_u32_ptr)(uintptr_t)(lds_tile + n * 1024u),
-                                         16, 0, 0);
+        const uint64_t base = ((uint64_t)ga_hi << 32) | (uint64_t)ga_lo;
+        const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane(lds_tile + n * 1024u);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dst), "v"(src), "s"(base)
+                     : "memory");
     }
     static __device__ __forceinline__ void load_tile(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
