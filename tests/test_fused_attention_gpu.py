@@ -194,6 +194,44 @@ def test_rows_longer_than_64_key_blocks(bf16, scheduled):
     check(got, orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS), TOL_BF16 if bf16 else TOL_F32)
 
 
+def test_scheduled_launch_in_a_hip_graph():
+    """The scheduled launch (split rows, counters reset by the kernel itself, no memset) captured into a graph:
+    every replay, with eager launches and synchronisations in between, gives the eager result bit for bit."""
+    bs, nb, B, H, d = 64, 32, 2, 4, 64
+    L = bs * nb
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    Q, K, V = qkv(B, L, H, d, seed=77, bf16=True)
+    q, k, v = (dev(x, True) for x in (Q, K, V))
+    nn = sfb.to_device(luts["nn_lut"])
+    sched = sfb.build_schedule(luts["nn_lut"], nb, 8)
+    items = sfb.to_device(sched["items"])
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    launch = lambda out: sfb.fused_attention_scheduled(q, k, v, nn, items, sched, ws, bs, luts["blocks"], 0.125, out=out)
+    eager = torch.empty((B, L, H, d), dtype=torch.float32, device="cuda")
+    launch(eager)
+    torch.cuda.synchronize()
+    captured = torch.zeros_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(captured)   # warm-up on the capture stream
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            launch(captured)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        captured.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager)
+        other = torch.empty_like(eager)
+        launch(other)   # eager launch on the same workspace between replays
+        torch.cuda.synchronize()
+        assert torch.equal(other, eager)
+
+
 def test_scale_and_large_scores():
     # scores far from zero: the running maximum and the 1e-6 term must still follow the oracle
     bs, nb, B, H, d = 64, 4, 1, 2, 64
