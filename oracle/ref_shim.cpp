@@ -4,8 +4,8 @@
 // they lie (the Makefile passes -I$(REFERENCE)) and exports C symbols around the functions the
 // oracle restates, so tests can bit-compare the restatement with the reference's own arithmetic.
 // It is compiled only where the reference checkout exists; the resulting library is git-ignored.
-#include "matmul.h"      // multiheadmatmulNT / multiheadmatmulNN
-#include "ewops.h"       // softmax, bias, gelu, tensor_add_*, transpose_0123to0213
+#include "matmul.h"      // multiheadmatmulNT / multiheadmatmulNN / multiheadmatmulTN
+#include "ewops.h"       // softmax, softmax_grad, bias, gelu, tensor_add_*, transpose_0123to0213
 #include "layernorm.h"   // layernorm
 #include "embedding.h"   // embedding_lookup
 
@@ -19,6 +19,12 @@ void ref_multiheadmatmulNN(float* C, float* A, float* B, int batch, int heads, i
 }
 void ref_softmax(float* C, float* A, float scaler, int seq_len, int batch, int heads) {
     softmax<float, float>(C, A, scaler, seq_len, batch, heads);
+}
+void ref_softmax_grad(float* out, float* dy, float* y, float scaler, int batch, int heads, int seq_len) {
+    softmax_grad<float, float, float>(out, dy, y, scaler, batch, heads, seq_len);
+}
+void ref_multiheadmatmulTN(float* C, float* A, float* B, int batch, int heads, int mA, int nA, int nB) {
+    multiheadmatmulTN<float, float, float>(C, A, B, batch, heads, mA, nA, nB);
 }
 void ref_transpose_0123to0213(float* src, float* dst, int d0, int d1, int d2, int d3) {
     transpose_0123to0213(src, dst, d0, d1, d2, d3);

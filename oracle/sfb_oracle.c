@@ -15,6 +15,12 @@
  *       /root/reference into oracle/_ref (dense-causal special case) and with the fixtures under
  *       tests/golden written by that build; float64 numpy brute force for every other pattern,
  *       closed forms (all-ones inputs), torch SDPA for the full layout.
+ *   orc_masked_softmax_grad, orc_dsd_tn (backward stages) : bit-compared with the reference's own
+ *       softmax_grad / multiheadmatmulTN in oracle/_ref on the dense-causal case (the whole chain dV, dP,
+ *       dS, dK, dQ) and with tests/golden/attention_backward_dense_causal.npz written by that build; torch
+ *       autograd of a float64 dense attention for every pattern, masks and padding included.
+ *   orc_build_tn_lut : the reference only has the commented causal builder (ewops.h:675-701); pinned by a
+ *       brute-force column scan for every pattern and by that builder's count pattern nb, nb-1, ..., 1.
  *   orc_layernorm, orc_gelu, orc_bias, orc_add*, orc_embedding_lookup, orc_transpose_0213 :
  *       bit-compared with the reference functions in oracle/_ref + golden fixtures; float64 numpy.
  *   orc_sgemm : the reference calls OpenBLAS cblas_sgemm (not vendored, no version pinned) --
@@ -240,6 +246,31 @@ void orc_build_rblk_lut(orc_uint2* rblk_lut, const orc_uint2* nn_lut, int nb) {
             count++;
         }
     }
+}
+
+/* TN look-up table of the transposed products (dV = P^T dO, dK = dS^T Q;
+ * transformer_attention_optimize.cu:924-957 passes it as tn_ptr): per key-block column c a header
+ * {offset, count}, offsets starting at nb, then the blocks of that column in ascending row order as
+ * {block id in NT order, row block} -- the column-wise twin of the NN table; the reference's own builder
+ * exists only as the commented causal special case generate_tn_lut (ewops.h:675-701).  Returns the
+ * largest count. */
+uint32_t orc_build_tn_lut(orc_uint2* tn_lut, const orc_uint2* nt_lut, uint32_t blocks, int nb) {
+    uint32_t offset = (uint32_t)nb, tn_max = 0, at = (uint32_t)nb;
+    for (int c = 0; c < nb; c++) {
+        uint32_t count = 0;
+        for (uint32_t blk = 0; blk < blocks; blk++)
+            if ((int)nt_lut[blk].y == c) {   /* NT order is row-major, so rows come out ascending */
+                tn_lut[at].x = blk;
+                tn_lut[at].y = nt_lut[blk].x;
+                at++;
+                count++;
+            }
+        tn_lut[c].x = offset;
+        tn_lut[c].y = count;
+        offset += count;
+        if (count > tn_max) tn_max = count;
+    }
+    return tn_max;
 }
 
 /* blocksparse.h:1016-1043 */
@@ -532,6 +563,60 @@ void orc_dsd_nn(float* O, const float* P, const float* V, const orc_uint2* nn_lu
                                        V[tok(b, (int)col * bs + kk, h, L, H, d) + m];
                         }
                         o[m] = sum;
+                    }
+                }
+            }
+        }
+}
+
+/* ewops.h:101-124 over the sparse storage: per query row sum = sum_k dy*y (float, ascending key; masked
+ * keys hold y = 0 and add nothing), out = (dy - sum) * y * scaler. */
+void orc_masked_softmax_grad(float* dS, const float* dP, const float* P, const orc_uint2* nn_lut, int B,
+                             int H, int nb, int bs, uint32_t blocks, float scale, int lut_heads) {
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < H; h++) {
+            const orc_uint2* lut = nn_lut + (lut_heads > 1 ? (size_t)h * (blocks + nb) : 0);
+            const size_t base = ((size_t)b * H + h) * blocks * bs * bs;
+            for (int r = 0; r < nb; r++) {
+                uint32_t offset = lut[r].x, count = lut[r].y;
+                for (int qi = 0; qi < bs; qi++) {
+                    float sum = 0;
+                    for (uint32_t jj = 0; jj < count; jj++) {
+                        const size_t at = base + ((size_t)lut[offset + jj].x * bs + qi) * bs;
+                        for (int kk = 0; kk < bs; kk++) sum += dP[at + kk] * P[at + kk];
+                    }
+                    for (uint32_t jj = 0; jj < count; jj++) {
+                        const size_t at = base + ((size_t)lut[offset + jj].x * bs + qi) * bs;
+                        for (int kk = 0; kk < bs; kk++) dS[at + kk] = (dP[at + kk] - sum) * P[at + kk] * scale;
+                    }
+                }
+            }
+        }
+}
+
+/* matmul.h:81-99 restricted to the blocks of the TN LUT: C[b, c*bs + kk, h, m] = sum over the column's
+ * blocks (ascending row block) and their query rows qi (ascending) of A_blk[qi][kk] * X[b, row*bs + qi, h, m],
+ * float accumulation in that order. */
+void orc_dsd_tn(float* Cout, const float* A, const float* X, const orc_uint2* tn_lut, int B, int L, int H,
+                int d, int bs, uint32_t blocks, int lut_heads) {
+    int nb = L / bs;
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < H; h++) {
+            const orc_uint2* lut = tn_lut + (lut_heads > 1 ? (size_t)h * (blocks + nb) : 0);
+            const float* a = A + ((size_t)b * H + h) * blocks * bs * bs;
+            for (int c = 0; c < nb; c++) {
+                uint32_t offset = lut[c].x, count = lut[c].y;
+                for (int kk = 0; kk < bs; kk++) {
+                    float* out = Cout + tok(b, c * bs + kk, h, L, H, d);
+                    for (int m = 0; m < d; m++) {
+                        float sum = 0;
+                        for (uint32_t jj = 0; jj < count; jj++) {
+                            uint32_t blk = lut[offset + jj].x, row = lut[offset + jj].y;
+                            for (int qi = 0; qi < bs; qi++)
+                                sum += a[((size_t)blk * bs + qi) * bs + kk] *
+                                       X[tok(b, (int)row * bs + qi, h, L, H, d) + m];
+                        }
+                        out[m] = sum;
                     }
                 }
             }

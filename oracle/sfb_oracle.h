@@ -38,6 +38,7 @@ void     orc_build_nt_lut(orc_uint2* nt_lut, const uint32_t* layout, int nb);
 uint32_t orc_build_nn_lut(orc_uint2* nn_lut, const orc_uint2* nt_lut, uint32_t blocks, int nb,
                           uint32_t nn_max_init);
 void     orc_build_rblk_lut(orc_uint2* rblk_lut, const orc_uint2* nn_lut, int nb);
+uint32_t orc_build_tn_lut(orc_uint2* tn_lut, const orc_uint2* nt_lut, uint32_t blocks, int nb);
 void     orc_magicu64(uint32_t d, uint32_t* magic, uint32_t* shift);
 uint32_t orc_div64(uint32_t value, uint32_t magic, uint32_t shift);
 
@@ -68,6 +69,11 @@ void orc_masked_softmax(float* P, const float* S, const orc_uint2* nn_lut,
                         float scale, int lut_heads, int mask_heads);
 void orc_dsd_nn(float* O, const float* P, const float* V, const orc_uint2* nn_lut, int B, int L,
                 int H, int d, int bs, uint32_t blocks, int lut_heads);
+/* backward stages of the unfused path (transformer_attention_optimize.cu:924-964) */
+void orc_masked_softmax_grad(float* dS, const float* dP, const float* P, const orc_uint2* nn_lut, int B,
+                             int H, int nb, int bs, uint32_t blocks, float scale, int lut_heads);
+void orc_dsd_tn(float* C, const float* A, const float* X, const orc_uint2* tn_lut, int B, int L, int H,
+                int d, int bs, uint32_t blocks, int lut_heads);
 
 /* ---- bf16 storage helpers ---- */
 uint16_t orc_f32_to_bf16_rne(float x);

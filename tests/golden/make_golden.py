@@ -25,6 +25,12 @@ def main():
     np.savez_compressed(os.path.join(HERE, "attention_dense_causal.npz"), Q=Q, K=K, V=V, O=O,
                         shape=np.array([B, L, H, d]), bs=bs, seed=seed, scale=scale)
 
+    from test_oracle_backward import ref_dense_causal_backward
+    dO = orc.fill_normal((B, L, H, d), seed + 4)
+    dQ, dK, dV, _ = ref_dense_causal_backward(Q, K, V, dO, float(scale))
+    np.savez_compressed(os.path.join(HERE, "attention_backward_dense_causal.npz"), dO=dO, dQ=dQ, dK=dK, dV=dV,
+                        shape=np.array([B, L, H, d]), bs=bs, seed=seed, scale=scale)
+
     rows, state = 6, 48
     x = orc.fill_normal((rows, state), 77) * 3 + 0.5
     g = orc.fill_normal((state,), 78)

@@ -29,6 +29,7 @@ ref = C.CDLL(_ref_path) if os.path.exists(_ref_path) else None
 vp = C.c_void_p
 lib.orc_count_blocks.restype = C.c_uint32
 lib.orc_build_nn_lut.restype = C.c_uint32
+lib.orc_build_tn_lut.restype = C.c_uint32
 lib.orc_div64.restype = C.c_uint32
 lib.orc_f32_to_bf16_rne.restype = C.c_uint16
 lib.orc_f32_to_bf16_rne.argtypes = [C.c_float]
@@ -178,6 +179,47 @@ def dsd_nn(P, V, nn_lut, lut_heads=1):
 
 
 # ---------------------------------------------------------------- layer ops
+def build_tn_lut(nt_lut, nb):
+    nt_lut = np.ascontiguousarray(nt_lut, np.uint32)
+    blocks = nt_lut.shape[0]
+    tn = np.zeros((nb + blocks, 2), np.uint32)
+    tn_max = lib.orc_build_tn_lut(_p(tn), _p(nt_lut), blocks, nb)
+    return tn, int(tn_max)
+
+
+def masked_softmax_grad(dP, P, nn_lut, nb, scale, lut_heads=1):
+    B, H, blocks, bs, _ = P.shape
+    dS = np.zeros_like(P)
+    lib.orc_masked_softmax_grad(_p(dS), _p(np.ascontiguousarray(dP, np.float32)), _p(P),
+                                _p(np.ascontiguousarray(nn_lut, np.uint32)), B, H, nb, bs, blocks,
+                                C.c_float(scale), lut_heads)
+    return dS
+
+
+def dsd_tn(A, X, tn_lut, lut_heads=1):
+    B, H, blocks, bs, _ = A.shape
+    _, L, _, d = X.shape
+    out = np.zeros((B, L, H, d), np.float32)
+    lib.orc_dsd_tn(_p(out), _p(A), _p(X), _p(np.ascontiguousarray(tn_lut, np.uint32)), B, L, H, d, bs,
+                   blocks, lut_heads)
+    return out
+
+
+def attention_backward(Q, K, V, dO, luts, bs, scale, mask=None, valid_len=None):
+    """Gradients of the unfused path in the reference's order (transformer_attention_optimize.cu:924-964):
+    dV = P^T dO, dP = dO V^T, dS = softmax_grad(dP, P), dK = dS^T Q, dQ = dS K.  Returns dQ, dK, dV, P."""
+    nb = Q.shape[1] // bs
+    S = sdd_nt(Q, K, luts["nt_lut"], bs)
+    P = masked_softmax(S, luts["nn_lut"], nb, scale, mask=mask, valid_len=valid_len)
+    tn, _ = build_tn_lut(luts["nt_lut"], nb)
+    dV = dsd_tn(P, dO, tn)
+    dP = sdd_nt(dO, V, luts["nt_lut"], bs)
+    dS = masked_softmax_grad(dP, P, luts["nn_lut"], nb, scale)
+    dK = dsd_tn(dS, Q, tn)
+    dQ = dsd_nn(dS, K, luts["nn_lut"])
+    return dQ, dK, dV, P
+
+
 def layernorm(x, g, b):
     rows, state = x.reshape(-1, x.shape[-1]).shape
     out = np.zeros_like(x)
