@@ -81,6 +81,12 @@ int sfb_build_nn_lut(sfb_uint2* nn_lut, const sfb_uint2* nt_lut, uint32_t blocks
                      uint32_t* nn_max);
 /* local_fusion_test.cu:229-237: rblk_lut[blocks] = {block id, row block}. */
 int sfb_build_rblk_lut(sfb_uint2* rblk_lut, const sfb_uint2* nn_lut, int nb);
+/* TN look-up table of the backward products dV = P^T dO and dK = dS^T Q
+ * (transformer_attention_optimize.cu:924, 948 pass it as tn_ptr; the reference's builder survives only as the
+ * commented causal case generate_tn_lut, ewops.h:675-701): tn_lut[nb + blocks], per key-block column a
+ * header {offset, count} with offsets starting at nb, then that column's blocks in ascending row order as
+ * {block id in NT order, row block}.  *tn_max (may be NULL) receives the largest count. */
+int sfb_build_tn_lut(sfb_uint2* tn_lut, const sfb_uint2* nt_lut, uint32_t blocks, int nb, uint32_t* tn_max);
 /* blocksparse.h:1016-1043 */
 void sfb_magicu64(uint32_t d, uint32_t* magic, uint32_t* shift);
 
@@ -182,12 +188,21 @@ int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, const void* ma
                        uint32_t lut_heads, uint32_t lut_dim, uint32_t max_lut, uint32_t mask_heads,
                        float scale);
 
-/* bst_sgemm_xn (blocksparse.h:965-1014), op = SFB_NN_OP: C_rowblk = sum over the row's blocks of
- * A_blk . B_colblk.  a [dev] sparse P of a_dtype; b [dev] V [batch, ctx_b, heads, state] of b_dtype;
- * c [dev] fp32 [batch, ctx_c, heads, state]; block-rows without blocks are zero-filled
- * (blocksparse.h:949-962).  The product runs on bf16 MFMA when b is bf16, on fp32 MFMA otherwise.
- * SFB_TN_OP (the backward product) returns SFB_ERR_ARGUMENT.  magic/shift/max_lut are accepted for
- * signature compatibility. */
+/* BlocksparseMaskedSoftmaxGrad<T,V> (blocksparse.h:1164-1228): dx = (dy - sum_k dy*y) * y * scale over each
+ * sparse row (ewops.h:101-124; masked keys hold y = 0).  dy, y, dx [dev] in the sparse layout, all of
+ * `dtype`; lut = NN LUT; max_lut is accepted for signature compatibility. */
+int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut, const void* dy, const void* y, void* dx,
+                            int dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                            uint32_t head_dim, uint32_t ctx_blks, uint32_t lut_heads, uint32_t lut_dim,
+                            uint32_t max_lut, float scale);
+
+/* bst_sgemm_xn (blocksparse.h:965-1014).  op = SFB_NN_OP: C_rowblk = sum over the row's blocks of
+ * A_blk . B_colblk, lut = NN LUT.  op = SFB_TN_OP (the backward products dV = P^T dO, dK = dS^T Q;
+ * matmul.h:81-99): C_colblk = sum over the column's blocks of A_blk^T . B_rowblk, lut = TN LUT.
+ * a [dev] sparse operand of a_dtype; b [dev] [batch, ctx_b, heads, state] of b_dtype; c [dev] fp32
+ * [batch, ctx_c, heads, state]; block-rows (columns) without blocks are zero-filled
+ * (blocksparse.h:949-962).  The product runs on bf16 MFMA when the operands are bf16, on fp32 MFMA
+ * otherwise.  magic/shift/max_lut are accepted for signature compatibility. */
 int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
                int a_dtype, int b_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim,

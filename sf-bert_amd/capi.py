@@ -53,11 +53,11 @@ EXPORTED = [
     "sfb_status_string", "sfb_device_available",
     "sfb_layout_full", "sfb_layout_local", "sfb_layout_fixed", "sfb_layout_strided_chunks",
     "sfb_layout_strided", "sfb_layout_bigbird", "sfb_bigbird_draw", "sfb_count_blocks",
-    "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_magicu64", "sfb_element_mask",
+    "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled",
-    "sfb_sdd_nt", "sfb_masked_softmax", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
+    "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
 ]
@@ -130,7 +130,8 @@ def layout_bigbird(nb, window, nglobal, both_ends, rand_cols=None):
 
 # ------------------------------------------------------------------------------------ LUTs / masks
 class Luts(dict):
-    """nt_lut [blocks,2], nn_lut [nb+blocks,2], rblk_lut [blocks,2], row_order [nb], nn_max, blocks, nb."""
+    """nt_lut [blocks,2], nn_lut / tn_lut [nb+blocks,2], rblk_lut [blocks,2], row_order [nb], nn_max, tn_max,
+    blocks, nb."""
     __getattr__ = dict.__getitem__
 
 
@@ -148,8 +149,11 @@ def build_luts(layout, nn_max_init=0):
     _check(lib.sfb_build_rblk_lut(_np(rblk), _np(nn), nb), "sfb_build_rblk_lut")
     order = np.zeros(nb, np.uint32)
     _check(lib.sfb_build_row_order(_np(order), _np(nn), nb), "sfb_build_row_order")
-    return Luts(nt_lut=nt, nn_lut=nn, rblk_lut=np.ascontiguousarray(rblk[:blocks]), row_order=order,
-                nn_max=int(nn_max.value), blocks=blocks, nb=nb)
+    tn = np.zeros((nb + blocks, 2), np.uint32)
+    tn_max = C.c_uint32(0)
+    _check(lib.sfb_build_tn_lut(_np(tn), _np(nt), blocks, nb, C.byref(tn_max)), "sfb_build_tn_lut")
+    return Luts(nt_lut=nt, nn_lut=nn, tn_lut=tn, rblk_lut=np.ascontiguousarray(rblk[:blocks]), row_order=order,
+                nn_max=int(nn_max.value), tn_max=int(tn_max.value), blocks=blocks, nb=nb)
 
 
 def element_mask(nt_lut, bs, kind, local_attn_ctx=0):
@@ -305,8 +309,24 @@ def BlocksparseMaskedSoftmax(lut, mask, x, ctx_blks, scale, out_dtype=None, vali
     return y
 
 
+def BlocksparseMaskedSoftmaxGrad(lut, dy, y, ctx_blks, scale, lut_heads=1, max_lut=0, dx=None):
+    """dx = (dy - sum_k dy*y) * y * scale over each sparse row (blocksparse.h:1164); dy, y, dx share a dtype."""
+    import torch
+    B, H, blocks, bs, _ = y.shape
+    if dy.dtype != y.dtype or dy.shape != y.shape:
+        raise SfbError(4, "dy and y differ in dtype or shape")
+    if dx is None:
+        dx = torch.empty_like(y)
+    _check(lib.sfb_masked_softmax_grad(_stream(), _dev(lut), _dev(dy), _dev(y), _dev(dx), _dtype_code(y),
+                                       C.c_uint32(bs), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(H),
+                                       C.c_uint32(ctx_blks), C.c_uint32(lut_heads), C.c_uint32(ctx_blks + blocks),
+                                       C.c_uint32(max_lut), C.c_float(scale)), "sfb_masked_softmax_grad")
+    return dx
+
+
 def bst_sgemm_xn(lut, a, b, ctx_blks_c, op=NN_OP, lut_heads=1, magic=1, shift=0, max_lut=0, c=None):
-    """dsd: O [B, L, H, d] = sum_blk P_blk . V_colblk (blocksparse.h:965)."""
+    """dsd (blocksparse.h:965).  NN_OP: C [B, L, H, d] = sum_blk A_blk . B_colblk over each block-row (lut = NN
+    LUT).  TN_OP: C = sum_blk A_blk^T . B_rowblk over each block-column (lut = TN LUT)."""
     import torch
     B, H, blocks, bs, _ = a.shape
     _, Lb, _, d = b.shape
@@ -338,6 +358,24 @@ def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_
 
 
 fusion_attention1 = fusion_attention2
+
+
+def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None):
+    """Gradients of O = P V, P = masked softmax(scale * Q K^T) from the stored probabilities P, in the order of
+    the reference's backward (transformer_attention_optimize.cu:924-965):
+        dV = P^T dO (TN), dP = dO V^T (NT), dS = softmax grad, dK = dS^T Q (TN), dQ = dS K (NN).
+    q, k, v, d_out [B, L, H, d]; p [B, H, blocks, bs, bs]; luts_dev: dict of device buffers nt_lut, nn_lut,
+    tn_lut.  dP / dS use p's dtype unless work_dtype says otherwise.  Returns (dq, dk, dv) fp32."""
+    nb = q.shape[1] // block_size
+    code = _dtype_code(p) if work_dtype is None else work_dtype
+    dv = bst_sgemm_xn(luts_dev["tn_lut"], p, d_out, nb, op=TN_OP)
+    dp = bst_sgemm_nt(luts_dev["nt_lut"], d_out, v, block_size, blocks, out_dtype=code)
+    if dp.dtype != p.dtype:
+        p = p.to(dp.dtype)
+    ds = BlocksparseMaskedSoftmaxGrad(luts_dev["nn_lut"], dp, p, nb, scale, dx=dp)
+    dk = bst_sgemm_xn(luts_dev["tn_lut"], ds, q, nb, op=TN_OP)
+    dq = bst_sgemm_xn(luts_dev["nn_lut"], ds, k, nb, op=NN_OP)
+    return dq, dk, dv
 
 
 # ------------------------------------------------------------------------------------ layer ops

@@ -203,6 +203,28 @@ int sfb_build_rblk_lut(sfb_uint2* rblk_lut, const sfb_uint2* nn_lut, int nb) {
     return SFB_OK;
 }
 
+int sfb_build_tn_lut(sfb_uint2* tn_lut, const sfb_uint2* nt_lut, uint32_t blocks, int nb, uint32_t* tn_max) {
+    if (!tn_lut || !nt_lut) return SFB_ERR_NULL_POINTER;
+    if (nb <= 0) return SFB_ERR_SHAPE;
+    // bucket the blocks by column; the NT table is a row-major scan, so rows come out ascending
+    std::vector<uint32_t> count((size_t)nb, 0u);
+    for (uint32_t blk = 0; blk < blocks; ++blk) {
+        if (nt_lut[blk].y >= (uint32_t)nb || nt_lut[blk].x >= (uint32_t)nb) return SFB_ERR_ARGUMENT;
+        ++count[nt_lut[blk].y];
+    }
+    uint32_t offset = (uint32_t)nb, longest = 0;
+    std::vector<uint32_t> next((size_t)nb);
+    for (int c = 0; c < nb; ++c) {
+        tn_lut[c] = sfb_uint2{offset, count[c]};
+        next[c] = offset;
+        offset += count[c];
+        if (count[c] > longest) longest = count[c];
+    }
+    for (uint32_t blk = 0; blk < blocks; ++blk) tn_lut[next[nt_lut[blk].y]++] = sfb_uint2{blk, nt_lut[blk].x};
+    if (tn_max) *tn_max = longest;
+    return SFB_OK;
+}
+
 void sfb_magicu64(uint32_t d, uint32_t* magic, uint32_t* shift) {
     if (!magic || !shift || d == 0) return;
     if (d <= 8 && (d & (d - 1)) == 0) {  // 1, 2, 4, 8: plain shifts

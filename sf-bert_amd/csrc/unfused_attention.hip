@@ -256,16 +256,217 @@ __global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// dsd: one work-group per (batch, head, block-row), V staged through LDS, P read in operand layout
+// masked softmax gradient: dx = (dy - sum_k dy*y) * y * scale per query row (ewops.h:101-124), one wave per
+// row, 8 consecutive keys per lane; rows of up to 64 key blocks keep dy and y in registers
+// ---------------------------------------------------------------------------------------------
+struct SoftmaxGradParams {
+    const sfb_uint2* lut;     // NN LUT
+    const void* dy;
+    const void* y;
+    void* dx;
+    uint32_t blocks, batch, heads, nb, lut_stride;
+    float scale;
+};
+
+template <int BS, typename T>
+__global__ __launch_bounds__(256) void masked_softmax_grad_kernel(SoftmaxGradParams p) {
+    constexpr int LPB = BS / 8, PER = 64 / LPB, CACHE = 8;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint64_t row_id = (uint64_t)blockIdx.x * 4 + wave;
+    const uint64_t total_rows = (uint64_t)p.batch * p.heads * p.nb * BS;
+    if (row_id >= total_rows) return;
+    const uint32_t qi = (uint32_t)(row_id % BS);
+    const uint32_t r = (uint32_t)((row_id / BS) % p.nb);
+    const uint32_t bh = (uint32_t)(row_id / ((uint64_t)BS * p.nb));
+    const uint32_t h = bh % p.heads;
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
+    const uint32_t off = lut[r].x, count = lut[r].y;
+    const uint32_t sub = lane / LPB, key0 = (lane % LPB) * 8;
+    const size_t head_base = (size_t)bh * p.blocks * BS * BS;
+    const T* dy = (const T*)p.dy + head_base;
+    const T* y = (const T*)p.y + head_base;
+    T* dx = (T*)p.dx + head_base;
+    auto load8 = [&](const T* base, uint32_t blk, float (&v)[8]) {
+        const T* src = base + ((size_t)blk * BS + qi) * BS + key0;
+        const f32x4 lo = Elem<T>::load4(src), hi = Elem<T>::load4(src + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    };
+    auto store8 = [&](uint32_t blk, const float (&v)[8]) {
+        T* dst = dx + ((size_t)blk * BS + qi) * BS + key0;
+        const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        Elem<T>::store4(dst, lo);
+        Elem<T>::store4(dst + 4, hi);
+    };
+    auto wave_sum = [](float l) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+        return l;
+    };
+    const uint32_t steps = (count + PER - 1) / PER;
+    if (steps <= CACHE) {
+        float g[CACHE][8], v[CACHE][8];
+        uint32_t blk[CACHE];
+        float sum = 0.f;
+#pragma unroll
+        for (int st = 0; st < CACHE; ++st) {
+            const uint32_t j = st * PER + sub;
+            blk[st] = 0xffffffffu;
+            if (j < count) {
+                blk[st] = lut[off + j].x;
+                load8(dy, blk[st], g[st]);
+                load8(y, blk[st], v[st]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sum += g[st][i] * v[st][i];
+            }
+        }
+        sum = wave_sum(sum);
+#pragma unroll
+        for (int st = 0; st < CACHE; ++st)
+            if (blk[st] != 0xffffffffu) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) g[st][i] = (g[st][i] - sum) * v[st][i] * p.scale;
+                store8(blk[st], g[st]);
+            }
+        return;
+    }
+    float sum = 0.f;
+    for (uint32_t j = sub; j < count; j += PER) {
+        const uint32_t b = lut[off + j].x;
+        float g[8], v[8];
+        load8(dy, b, g);
+        load8(y, b, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += g[i] * v[i];
+    }
+    sum = wave_sum(sum);
+    for (uint32_t j = sub; j < count; j += PER) {
+        const uint32_t b = lut[off + j].x;
+        float g[8], v[8];
+        load8(dy, b, g);
+        load8(y, b, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) g[i] = (g[i] - sum) * v[i] * p.scale;
+        store8(b, g);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dsd, transposed sparse operand (TN): C[col block] = sum over the column's blocks of A_blk^T . B_rowblk
+// (matmul.h:81-99; dV = P^T dO and dK = dS^T Q of the backward pass).  One work-group per (batch, head,
+// key-block column); wave w owns keys 32w .. 32w+31 of the column block and all D output columns:
+//   C^T[col][key] += sum_q B[q][col] * A[q][key]      (MFMA: A-operand = B^T tile, B-operand = A tile)
+// Both tiles are stored row-major with the contraction index q as the row, so both operands are read
+// k-major: bf16 tiles through the transposing LDS read, fp32 one element per lane.
 // ---------------------------------------------------------------------------------------------
 struct DsdParams {
-    const sfb_uint2* lut;   // NN LUT
-    const void* a;          // P
-    const void* b;          // V
-    float* c;               // O
+    const sfb_uint2* lut;   // NN LUT (header per block-row) or TN LUT (header per block-column)
+    const void* a;          // sparse operand: P, or dS
+    const void* b;          // dense operand: V, or dO / Q
+    float* c;               // dense result
     uint32_t blocks, batch, heads, nb_b, nb_c, lut_stride, groups;
 };
 
+template <int BS, int D, typename TA, typename TB>
+__global__ __launch_bounds__(BS * 2, 2) void dsd_tn_kernel(DsdParams p) {
+    constexpr int NO = D / 32;
+    constexpr bool kFast = sizeof(TA) == 2 && sizeof(TB) == 2 && BS == 64;
+    using TD = Bf16DirectTiles<BS, D>;
+    constexpr int TILE = TD::TILE_BYTES;
+    constexpr int X_STRIDE = D + 8;   // floats, generic path
+    constexpr int LDS_BYTES = kFast ? 4 * TILE : BS * X_STRIDE * 4;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
+
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t col = work.rank;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t kn = lane & 31, half = lane >> 5;
+    const uint32_t key_in_block = wave * 32 + kn;
+    const uint32_t row_stride = p.heads * D;
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
+    const uint32_t off = __builtin_amdgcn_readfirstlane(lut[col].x), count = __builtin_amdgcn_readfirstlane(lut[col].y);
+    float* c_row = p.c + token_offset(b, col * BS + key_in_block, h, p.nb_c * BS, p.heads, D);
+    const TA* A = (const TA*)p.a + (size_t)work.bh * p.blocks * BS * BS;
+    const TB* X = (const TB*)p.b;
+
+    f32x16 acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[n][i] = 0.f;
+
+    if constexpr (kFast) {
+        // tiles 0, 1: X row blocks [q][D]; tiles 2, 3: sparse blocks [q][key]; LDS-direct loads, double-buffered
+        const uint32_t row_bytes = row_stride * 2;
+        const uint32_t x_even = TD::lane_source(lane, 0, row_bytes), x_odd = TD::lane_source(lane, 1, row_bytes);
+        const uint32_t a_even = TD::lane_source(lane, 0, BS * 2), a_odd = TD::lane_source(lane, 1, BS * 2);
+        const uint32_t lds0 = TD::lds_address(smem);
+        const uint32_t x_lane = TD::v_lane_base(lane);
+        const uint8_t* const x_base = (const uint8_t*)X + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
+        auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
+            TD::load_tile(lds0 + buf * TILE, x_base + (size_t)e.y * BS * row_bytes, wave, x_even, x_odd, row_bytes);
+            TD::load_tile(lds0 + (2 + buf) * TILE, (const uint8_t*)A + (size_t)e.x * BS * BS * 2, wave, a_even, a_odd,
+                          BS * 2);
+        };
+        auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
+            const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
+            return u;
+        };
+        if (count > 0) fetch(uniform(lut[off]), 0);
+        for (uint32_t j = 0; j < count; ++j) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            fetch(uniform(lut[off + (j + 1 < count ? j + 1 : j)]), (j + 1) & 1);
+            const uint8_t* x_read = smem + (j & 1) * TILE;
+            const uint8_t* a_read = smem + (2 + (j & 1)) * TILE;
+#pragma unroll
+            for (int u = 0; u < BS / 16; ++u) {
+                // B-operand: the sparse block [q][key]; this wave's 32 keys are its "column tile" number `wave`
+                const bf16x8 bfrag = TD::v_frag(a_read, x_lane, (int)wave, u);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(x_read, x_lane, mt, u), bfrag, acc[mt], 0, 0, 0);
+            }
+        }
+    } else {
+        // generic path: fp32 MFMA (k = 2 per step, one element per lane and operand); the X row block is staged
+        // in LDS as fp32, the sparse block is read from memory, 32 consecutive keys per half-wave
+        float* x_lds = (float*)smem;
+        for (uint32_t j = 0; j < count; ++j) {
+            const sfb_uint2 e = lut[off + j];
+            const TB* x_blk = X + token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
+            const TA* a_blk = A + (size_t)e.x * BS * BS;
+            for (uint32_t cid = t; cid < BS * (D / 4); cid += BS * 2) {
+                const uint32_t row = cid / (D / 4), cc = cid % (D / 4);
+                *(f32x4*)(x_lds + row * X_STRIDE + cc * 4) = Elem<TB>::load4(x_blk + (size_t)row * row_stride + cc * 4);
+            }
+            __syncthreads();
+#pragma unroll 4
+            for (int s2 = 0; s2 < BS / 2; ++s2) {
+                const uint32_t q = 2 * s2 + half;
+                const float av = Elem<TA>::load(a_blk + (size_t)q * BS + key_in_block);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(x_lds[q * X_STRIDE + mt * 32 + kn], av, acc[mt], 0, 0, 0);
+            }
+            __syncthreads();
+        }
+    }
+    // accumulator element i of column tile mt is column mt*32 + (i/4)*8 + half*4 + i%4 of this lane's key row;
+    // columns without blocks write zeros
+#pragma unroll
+    for (int mt = 0; mt < NO; ++mt)
+#pragma unroll
+        for (int ig = 0; ig < 4; ++ig) {
+            const f32x4 out = {acc[mt][ig * 4 + 0], acc[mt][ig * 4 + 1], acc[mt][ig * 4 + 2], acc[mt][ig * 4 + 3]};
+            *(f32x4*)(c_row + mt * 32 + ig * 8 + half * 4) = out;
+        }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dsd: one work-group per (batch, head, block-row), V staged through LDS, P read in operand layout
+// ---------------------------------------------------------------------------------------------
 template <int BS, int D, typename TP, typename TV>
 __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int KT = BS / 32, NO = D / 32;
@@ -570,7 +771,7 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     (void)magic; (void)shift; (void)max_lut;  // grid decomposition / smem sizing of the reference kernel
     if (!lut || !a || !b || !c) return SFB_ERR_NULL_POINTER;
     if (check_dtype(a_dtype) || check_dtype(b_dtype)) return SFB_ERR_DTYPE;
-    if (op != SFB_NN_OP) return SFB_ERR_ARGUMENT;   // TN_OP is the backward product: not part of this path
+    if (op != SFB_NN_OP && op != SFB_TN_OP) return SFB_ERR_ARGUMENT;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (state_dim != 64) return SFB_ERR_HEAD_STATE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks_b || !ctx_blks_c || !lut_heads) return SFB_ERR_SHAPE;
@@ -581,10 +782,45 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     const dim3 grid(p.groups * 8u * ctx_blks_c);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (op == SFB_TN_OP) {
+#define SFB_CALL(BSV, TA, TB) dsd_tn_kernel<BSV, 64, TA, TB><<<grid, dim3(BSV * 2), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_2(64, a_dtype, b_dtype, SFB_CALL);
+        else SFB_DISPATCH_2(32, a_dtype, b_dtype, SFB_CALL);
+#undef SFB_CALL
+        return launch_status();
+    }
 #define SFB_CALL(BSV, TP, TV) dsd_nn_kernel<BSV, 64, TP, TV><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, a_dtype, b_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, a_dtype, b_dtype, SFB_CALL);
 #undef SFB_CALL
+    return launch_status();
+}
+
+extern "C" int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut, const void* dy, const void* y,
+                                       void* dx, int dtype, uint32_t block_size, uint32_t blocks,
+                                       uint32_t batch_dim, uint32_t head_dim, uint32_t ctx_blks,
+                                       uint32_t lut_heads, uint32_t lut_dim, uint32_t max_lut, float scale) {
+    (void)max_lut;  // sizes the reference's shared memory (blocksparse.h:671-686); not needed here
+    if (!lut || !dy || !y || !dx) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)dy | (uintptr_t)y | (uintptr_t)dx) & 15u) return SFB_ERR_ALIGNMENT;
+    SoftmaxGradParams p = {lut, dy, y, dx, blocks, batch_dim, head_dim, ctx_blks, lut_heads > 1 ? lut_dim : 0, scale};
+    const uint64_t rows = (uint64_t)batch_dim * head_dim * ctx_blks * block_size;
+    if ((rows + 3) / 4 > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const dim3 grid((uint32_t)((rows + 3) / 4));
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+    if (block_size == 64) {
+        if (dtype == SFB_F32) masked_softmax_grad_kernel<64, float><<<grid, dim3(256), 0, s>>>(p);
+        else masked_softmax_grad_kernel<64, __bf16><<<grid, dim3(256), 0, s>>>(p);
+    } else {
+        if (dtype == SFB_F32) masked_softmax_grad_kernel<32, float><<<grid, dim3(256), 0, s>>>(p);
+        else masked_softmax_grad_kernel<32, __bf16><<<grid, dim3(256), 0, s>>>(p);
+    }
     return launch_status();
 }
 

@@ -76,6 +76,8 @@ def test_luts_bit_exact(layout):
         for key in ("nt_lut", "nn_lut", "rblk_lut"):
             assert np.array_equal(got[key], want[key]), key
         assert got["nn_max"] == want["nn_max"] and got["blocks"] == want["blocks"]
+        tn, tn_max = orc.build_tn_lut(want["nt_lut"], layout.shape[0])
+        assert np.array_equal(got["tn_lut"], tn) and got["tn_max"] == tn_max
     counts = layout.sum(axis=1)
     order = got["row_order"]
     assert sorted(order.tolist()) == list(range(layout.shape[0]))

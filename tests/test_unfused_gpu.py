@@ -130,7 +130,7 @@ def test_error_codes_instead_of_silent_no_op():
     assert sfb.lib.sfb_sdd_nt(None, p(lut), p(q), p(q), p(q), 0, 0, u(16), u(1), u(1), u(1), u(1), u(1), u(64),
                               u(1), u(1)) == 2
     assert sfb.lib.sfb_dsd_xn(None, p(lut), p(q), p(q), p(q), 0, 0, u(64), u(1), u(1), u(1), u(1), u(1), u(64),
-                              u(1), u(2), u(sfb.TN_OP), u(1), u(0), u(1)) == 8
+                              u(1), u(2), u(sfb.NT_OP), u(1), u(0), u(1)) == 8
     assert sfb.lib.sfb_masked_softmax(None, p(lut), None, p(q), p(q), 0, 3, None, u(64), u(1), u(1), u(1), u(1),
                                       u(1), u(2), u(1), u(1), C.c_float(0.125)) == 5
     assert sfb.lib.sfb_fused_sdd_softmax(None, None, p(q), p(q), p(q), 0, 0, None, None, u(64), u(1), u(1), u(1),
