@@ -110,7 +110,11 @@ __global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// masked softmax: one wave per query row, 8 consecutive keys per lane (8 or 16 key blocks per wave step)
+// masked softmax and its gradient.  One wave owns 4 consecutive query rows of one block-row; a lane owns 8
+// consecutive keys, so a wave step covers 8 (BS 64) or 16 (BS 32) key blocks of a row.  The wave has 8
+// register slots of one step each: rows of up to 2 steps are processed 4 at a time, rows of up to 4 steps 2
+// at a time, rows of up to 8 steps one by one -- one read and one write of memory each; longer rows take
+// three passes.  The rows of a block-row share their look-up table entries, which are read once per wave.
 // (blocksparse.h:459-722 keeps one CTA per query row; the row-major mask order is the same)
 // ---------------------------------------------------------------------------------------------
 struct SoftmaxParams {
@@ -123,142 +127,358 @@ struct SoftmaxParams {
     float scale_log2e;
 };
 
-template <int BS, typename TX, typename TY>
-__global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
-    constexpr int LPB = BS / 8;     // lanes per key block: every lane owns 8 consecutive keys (16 or 32 bytes)
-    constexpr int PER = 64 / LPB;   // key blocks covered by one wave step
-    constexpr int CACHE = 8;        // steps whose scores stay in registers (64 blocks at BS 64)
-    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const uint64_t row_id = (uint64_t)blockIdx.x * 4 + wave;        // over batch*heads*nb*BS
-    const uint64_t total_rows = (uint64_t)p.batch * p.heads * p.nb * BS;
-    if (row_id >= total_rows) return;
-    const uint32_t qi = (uint32_t)(row_id % BS);
-    const uint32_t r = (uint32_t)((row_id / BS) % p.nb);
-    const uint32_t bh = (uint32_t)(row_id / ((uint64_t)BS * p.nb));
-    const uint32_t b = bh / p.heads, h = bh % p.heads;
-    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
-    const uint32_t off = lut[r].x, count = lut[r].y;
-    const uint32_t sub = lane / LPB, key0 = (lane % LPB) * 8;
-    const TX* x = (const TX*)p.x + (size_t)bh * p.blocks * BS * BS;
-    TY* y = (TY*)p.y + (size_t)bh * p.blocks * BS * BS;
-    const int valid = p.valid_len ? p.valid_len[b] : (int)(p.nb * BS);
-    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
-    const float c = p.scale_log2e;
+constexpr int kSoftmaxSlots = 8;      // register slots (steps) of a wave
+constexpr int kSoftmaxWaveRows = 4;   // query rows per wave
 
-    // keep bits of this lane's 8 keys in key block e
-    auto keep_bits = [&](const sfb_uint2 e) -> uint32_t {
+// The wave's position: rows q0 .. q0+3 of block-row r of (batch, head) bh.
+struct SoftmaxWave {
+    uint32_t q0, r, bh;
+    bool valid;
+};
+template <int BS>
+__device__ __forceinline__ SoftmaxWave softmax_wave(uint32_t batch, uint32_t heads, uint32_t nb) {
+    constexpr uint32_t UNITS = BS / kSoftmaxWaveRows;   // waves per block-row
+    const uint64_t unit = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    SoftmaxWave w;
+    w.valid = unit < (uint64_t)batch * heads * nb * UNITS;
+    w.q0 = (uint32_t)(unit % UNITS) * kSoftmaxWaveRows;
+    w.r = (uint32_t)((unit / UNITS) % nb);
+    w.bh = (uint32_t)(unit / ((uint64_t)UNITS * nb));
+    return w;
+}
+inline uint64_t softmax_grid(uint32_t batch, uint32_t heads, uint32_t nb, uint32_t bs) {
+    const uint64_t waves = (uint64_t)batch * heads * nb * (bs / kSoftmaxWaveRows);
+    return (waves + 3) / 4;
+}
+
+__device__ __forceinline__ float wave_max(float m) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
+    return m;
+}
+__device__ __forceinline__ float wave_sum(float l) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
+    return l;
+}
+
+// 8 consecutive elements of a lane: one 16-byte access for bf16, two for fp32
+template <typename T>
+__device__ __forceinline__ void load8(const T* src, float (&v)[8]) {
+    if constexpr (sizeof(T) == 2) {
+        const u32x4 r = *(const u32x4*)src;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = bf16_bits_to_f32(r[i] & 0xffffu);
+            v[2 * i + 1] = __builtin_bit_cast(float, r[i] & 0xffff0000u);
+        }
+    } else {
+        const f32x4 lo = *(const f32x4*)src, hi = *(const f32x4*)(src + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store8(T* dst, const float (&v)[8]) {
+    if constexpr (sizeof(T) == 2) {
+        const u32x4 r = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+        *(u32x4*)dst = r;
+    } else {
+        const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        *(f32x4*)dst = lo;
+        *(f32x4*)(dst + 4) = hi;
+    }
+}
+
+// The same 8 elements kept in their storage type (4 registers for bf16, 8 for fp32) until they are used
+template <typename T> struct Packed8;
+template <> struct Packed8<float> {
+    f32x4 lo, hi;
+    __device__ __forceinline__ void load(const float* src) { lo = *(const f32x4*)src; hi = *(const f32x4*)(src + 4); }
+    __device__ __forceinline__ float get(int i) const { return i < 4 ? lo[i] : hi[i - 4]; }
+    __device__ __forceinline__ void unpack_after(float&) {}
+};
+template <> struct Packed8<__bf16> {
+    u32x4 r;
+    __device__ __forceinline__ void load(const __bf16* src) { r = *(const u32x4*)src; }
+    __device__ __forceinline__ float get(int i) const {
+        return (i & 1) ? __builtin_bit_cast(float, r[i >> 1] & 0xffff0000u) : bf16_bits_to_f32(r[i >> 1] & 0xffffu);
+    }
+    // Keeps the compiler from unpacking all elements long before `dep` is known (which would cost the registers
+    // that the packed form saves): later get() calls depend on this point.
+    __device__ __forceinline__ void unpack_after(float& dep) {
+        uint32_t a = r[0], b = r[1], c = r[2], d = r[3];
+        asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(dep));
+        r[0] = a; r[1] = b; r[2] = c; r[3] = d;
+    }
+};
+
+template <int BS, typename TX, typename TY>
+struct SoftmaxRows {
+    static constexpr int LPB = BS / 8;     // lanes per key block: every lane owns 8 consecutive keys
+    static constexpr int PER = 64 / LPB;   // key blocks covered by one wave step
+    const sfb_uint2* lut;    // this head's table
+    const uint8_t* mask;     // this head's row-major words, or nullptr
+    const TX* x;             // this (batch, head)'s blocks
+    TY* y;
+    uint32_t off, count, blocks, sub, key0;
+    int valid;
+    float c;
+
+    // keep bits of this lane's 8 keys of query row qi in key block e
+    __device__ __forceinline__ uint32_t keep_bits(const sfb_uint2 e, uint32_t qi) const {
         const int left = valid - (int)(e.y * BS + key0);
         uint32_t k = left >= 8 ? 0xffu : (left <= 0 ? 0u : ((1u << left) - 1u));
         if (mask) {
-            const size_t w = (size_t)qi * p.blocks + e.x;
+            const size_t w = (size_t)qi * blocks + e.x;
             const uint64_t word = (BS == 64) ? ((const uint64_t*)mask)[w] : ((const uint32_t*)mask)[w];
             k &= (uint32_t)(word >> key0);
         }
         return k;
-    };
-    auto load8 = [&](const sfb_uint2 e, float (&v)[8]) {
-        const TX* src = x + ((size_t)e.x * BS + qi) * BS + key0;
-        const f32x4 lo = Elem<TX>::load4(src), hi = Elem<TX>::load4(src + 4);
-        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
-    };
-    auto store8 = [&](const sfb_uint2 e, const float (&v)[8]) {
-        TY* dst = y + ((size_t)e.x * BS + qi) * BS + key0;
-        const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-        Elem<TY>::store4(dst, lo);
-        Elem<TY>::store4(dst + 4, hi);
-    };
-    auto wave_max = [](float m) {
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d));
-        return m;
-    };
-    auto wave_sum = [](float l) {
-#pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
-        return l;
-    };
+    }
+    __device__ __forceinline__ size_t at(const sfb_uint2 e, uint32_t qi) const {
+        return ((size_t)e.x * BS + qi) * BS + key0;
+    }
 
-    const uint32_t steps = (count + PER - 1) / PER;
-    if (steps <= CACHE) {
-        // the whole row fits in registers: one read, one write.  Maximum over kept keys (seed as
-        // ewops.h:70), sum relative to it, normalised probabilities with zeros at masked keys (ewops.h:82)
-        float v[CACHE][8];
-        uint32_t keep[CACHE];
-        sfb_uint2 ent[CACHE];
-        float m = kMaxSeed;
+    // R rows of up to S steps each, all in registers: one read, one write.  Maximum over kept keys (seed as
+    // ewops.h:70), sum relative to it, normalised probabilities with zeros at masked keys (ewops.h:82).
+    // MASKED = false skips the keep bits (no element mask, no key padding).  Masked scores are replaced by
+    // kMaskedScore, whose exponential is an exact zero.
+    template <int R, int S, bool MASKED>
+    __device__ __forceinline__ void in_registers(uint32_t q0) const {
+        static_assert(R * S == kSoftmaxSlots, "slots");
+        float v[R][S][8];
+        sfb_uint2 ent[S];
 #pragma unroll
-        for (int st = 0; st < CACHE; ++st) {
+        for (int st = 0; st < S; ++st) {
             const uint32_t j = st * PER + sub;
-            keep[st] = 0;
-            if (j < count) {
-                ent[st] = lut[off + j];
-                load8(ent[st], v[st]);
-                keep[st] = keep_bits(ent[st]) | 0x100u;   // bit 8: the block exists
+            ent[st].x = 0xffffffffu;
+            if (j < count) ent[st] = lut[off + j];
+        }
 #pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if ((keep[st] >> i) & 1u) m = fmaxf(m, v[st][i]);
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int st = 0; st < S; ++st) {
+                if (ent[st].x != 0xffffffffu) {
+                    load8<TX>(x + at(ent[st], q0 + rr), v[rr][st]);
+                    if (MASKED) {
+                        const uint32_t keep = keep_bits(ent[st], q0 + rr);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) v[rr][st][i] = ((keep >> i) & 1u) ? v[rr][st][i] : kMaskedScore;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[rr][st][i] = kMaskedScore;
+                }
             }
+        float m[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float m0 = kMaxSeed, m1 = kMaxSeed;
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+#pragma unroll
+                for (int i = 0; i < 8; i += 4) {
+                    m0 = fmaxf(fmaxf(m0, v[rr][st][i]), v[rr][st][i + 1]);
+                    m1 = fmaxf(fmaxf(m1, v[rr][st][i + 2]), v[rr][st][i + 3]);
+                }
+            m[rr] = fmaxf(m0, m1);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) m[rr] = wave_max(m[rr]);
+        float l[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            const float mc = m[rr] * c;
+            float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) {
+                    v[rr][st][i] = exp2_fast(__builtin_fmaf(v[rr][st][i], c, -mc));
+                    v[rr][st][i + 1] = exp2_fast(__builtin_fmaf(v[rr][st][i + 1], c, -mc));
+                    l0 += v[rr][st][i];
+                    l1 += v[rr][st][i + 1];
+                }
+            l[rr] = l0 + l1;
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) l[rr] = wave_sum(l[rr]);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            const float inv = 1.0f / (l[rr] + 1e-6f);
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+                if (ent[st].x != 0xffffffffu) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[rr][st][i] *= inv;
+                    store8<TY>(y + at(ent[st], q0 + rr), v[rr][st]);
+                }
+        }
+    }
+    // The same for bf16 scores, which stay packed in registers (half the registers, twice the waves per SIMD);
+    // the exponentials are computed once for the sum and once more for the result.
+    template <int R, int S, bool MASKED>
+    __device__ __forceinline__ void in_registers_packed(uint32_t q0) const {
+        static_assert(R * S == kSoftmaxSlots && sizeof(TX) == 2, "slots");
+        constexpr uint32_t kMaskedPair = 0xff7fff7fu;   // two bf16 of -3.39e38
+        Packed8<TX> v[R][S];
+        sfb_uint2 ent[S];
+#pragma unroll
+        for (int st = 0; st < S; ++st) {
+            const uint32_t j = st * PER + sub;
+            ent[st].x = 0xffffffffu;
+            if (j < count) ent[st] = lut[off + j];
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int st = 0; st < S; ++st) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[rr][st].r[i] = kMaskedPair;
+                if (ent[st].x != 0xffffffffu) {
+                    v[rr][st].load(x + at(ent[st], q0 + rr));
+                    if (MASKED) {
+                        const uint32_t keep = keep_bits(ent[st], q0 + rr);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t lo = 0u - ((keep >> (2 * i)) & 1u), hi = 0u - ((keep >> (2 * i + 1)) & 1u);
+                            const uint32_t sel = (lo & 0xffffu) | (hi & 0xffff0000u);
+                            v[rr][st].r[i] = (v[rr][st].r[i] & sel) | (kMaskedPair & ~sel);
+                        }
+                    }
+                }
+            }
+        float m[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float m0 = kMaxSeed, m1 = kMaxSeed;
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+#pragma unroll
+                for (int i = 0; i < 8; i += 4) {
+                    m0 = fmaxf(fmaxf(m0, v[rr][st].get(i)), v[rr][st].get(i + 1));
+                    m1 = fmaxf(fmaxf(m1, v[rr][st].get(i + 2)), v[rr][st].get(i + 3));
+                }
+            m[rr] = fmaxf(m0, m1);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) m[rr] = wave_max(m[rr]);
+        float l[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float mc = m[rr] * c;
+            float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+            for (int st = 0; st < S; ++st) {
+                v[rr][st].unpack_after(mc);
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) {
+                    l0 += exp2_fast(__builtin_fmaf(v[rr][st].get(i), c, -mc));
+                    l1 += exp2_fast(__builtin_fmaf(v[rr][st].get(i + 1), c, -mc));
+                }
+            }
+            l[rr] = l0 + l1;
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) l[rr] = wave_sum(l[rr]);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            const float mc = m[rr] * c;
+            float inv = 1.0f / (l[rr] + 1e-6f);
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+                if (ent[st].x != 0xffffffffu) {
+                    v[rr][st].unpack_after(inv);
+                    float out[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) out[i] = exp2_fast(__builtin_fmaf(v[rr][st].get(i), c, -mc)) * inv;
+                    store8<TY>(y + at(ent[st], q0 + rr), out);
+                }
+        }
+    }
+    template <int R, int S>
+    __device__ __forceinline__ void in_registers(uint32_t q0, bool masked) const {
+        if constexpr (sizeof(TX) == 2) {
+            if (masked) in_registers_packed<R, S, true>(q0);
+            else in_registers_packed<R, S, false>(q0);
+        } else {
+            if (masked) in_registers<R, S, true>(q0);
+            else in_registers<R, S, false>(q0);
+        }
+    }
+
+    // a row of any length: three passes over memory
+    __device__ __forceinline__ void in_passes(uint32_t qi) const {
+        float m = kMaxSeed;
+        for (uint32_t j = sub; j < count; j += PER) {
+            const sfb_uint2 e = lut[off + j];
+            float v[8];
+            load8<TX>(x + at(e, qi), v);
+            const uint32_t k = keep_bits(e, qi);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((k >> i) & 1u) m = fmaxf(m, v[i]);
         }
         m = wave_max(m);
         float l = 0.f;
+        for (uint32_t j = sub; j < count; j += PER) {
+            const sfb_uint2 e = lut[off + j];
+            float v[8];
+            load8<TX>(x + at(e, qi), v);
+            const uint32_t k = keep_bits(e, qi);
 #pragma unroll
-        for (int st = 0; st < CACHE; ++st)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float e = ((keep[st] >> i) & 1u) ? exp2_fast((v[st][i] - m) * c) : 0.f;
-                v[st][i] = e;
-                l += e;
-            }
+            for (int i = 0; i < 8; ++i)
+                if ((k >> i) & 1u) l += exp2_fast((v[i] - m) * c);
+        }
         l = wave_sum(l);
         const float inv = 1.0f / (l + 1e-6f);
+        for (uint32_t j = sub; j < count; j += PER) {
+            const sfb_uint2 e = lut[off + j];
+            float v[8];
+            load8<TX>(x + at(e, qi), v);
+            const uint32_t k = keep_bits(e, qi);
 #pragma unroll
-        for (int st = 0; st < CACHE; ++st)
-            if (keep[st] & 0x100u) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) v[st][i] *= inv;
-                store8(ent[st], v[st]);
-            }
-        return;
+            for (int i = 0; i < 8; ++i) v[i] = ((k >> i) & 1u) ? exp2_fast((v[i] - m) * c) * inv : 0.f;
+            store8<TY>(y + at(e, qi), v);
+        }
     }
-    // longer rows: three passes over memory
-    float m = kMaxSeed;
-    for (uint32_t j = sub; j < count; j += PER) {
-        const sfb_uint2 e = lut[off + j];
-        float v[8];
-        load8(e, v);
-        const uint32_t k = keep_bits(e);
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if ((k >> i) & 1u) m = fmaxf(m, v[i]);
-    }
-    m = wave_max(m);
-    float l = 0.f;
-    for (uint32_t j = sub; j < count; j += PER) {
-        const sfb_uint2 e = lut[off + j];
-        float v[8];
-        load8(e, v);
-        const uint32_t k = keep_bits(e);
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if ((k >> i) & 1u) l += exp2_fast((v[i] - m) * c);
-    }
-    l = wave_sum(l);
-    const float inv = 1.0f / (l + 1e-6f);
-    for (uint32_t j = sub; j < count; j += PER) {
-        const sfb_uint2 e = lut[off + j];
-        float v[8];
-        load8(e, v);
-        const uint32_t k = keep_bits(e);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = ((k >> i) & 1u) ? exp2_fast((v[i] - m) * c) * inv : 0.f;
-        store8(e, v);
+};
+
+template <int BS, typename TX, typename TY>
+__global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
+    using Rows = SoftmaxRows<BS, TX, TY>;
+    const SoftmaxWave w = softmax_wave<BS>(p.batch, p.heads, p.nb);
+    if (!w.valid) return;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t b = w.bh / p.heads, h = w.bh % p.heads;
+    Rows rows;
+    rows.lut = p.lut + (size_t)h * p.lut_stride;
+    rows.mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    rows.x = (const TX*)p.x + (size_t)w.bh * p.blocks * BS * BS;
+    rows.y = (TY*)p.y + (size_t)w.bh * p.blocks * BS * BS;
+    rows.off = rows.lut[w.r].x;
+    rows.count = rows.lut[w.r].y;
+    rows.blocks = p.blocks;
+    rows.sub = lane / Rows::LPB;
+    rows.key0 = (lane % Rows::LPB) * 8;
+    rows.valid = p.valid_len ? p.valid_len[b] : (int)(p.nb * BS);
+    rows.c = p.scale_log2e;
+    const uint32_t steps = (rows.count + Rows::PER - 1) / Rows::PER;
+    const bool masked = rows.mask != nullptr || rows.valid < (int)(p.nb * BS);
+    if (steps <= 2) {
+        rows.template in_registers<4, 2>(w.q0, masked);
+    } else if (steps <= 4) {
+        rows.template in_registers<2, 4>(w.q0, masked);
+        rows.template in_registers<2, 4>(w.q0 + 2, masked);
+    } else if (steps <= 8) {
+        for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.template in_registers<1, 8>(w.q0 + i, masked);
+    } else {
+        for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.in_passes(w.q0 + i);
     }
 }
 
-// ---------------------------------------------------------------------------------------------
-// masked softmax gradient: dx = (dy - sum_k dy*y) * y * scale per query row (ewops.h:101-124), one wave per
-// row, 8 consecutive keys per lane; rows of up to 64 key blocks keep dy and y in registers
-// ---------------------------------------------------------------------------------------------
+// dx = (dy - sum_k dy*y) * y * scale per query row (ewops.h:101-124); same decomposition, with register
+// slots for dy and for y that hold the storage type
 struct SoftmaxGradParams {
     const sfb_uint2* lut;     // NN LUT
     const void* dy;
@@ -269,84 +489,122 @@ struct SoftmaxGradParams {
 };
 
 template <int BS, typename T>
-__global__ __launch_bounds__(256) void masked_softmax_grad_kernel(SoftmaxGradParams p) {
-    constexpr int LPB = BS / 8, PER = 64 / LPB, CACHE = 8;
-    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const uint64_t row_id = (uint64_t)blockIdx.x * 4 + wave;
-    const uint64_t total_rows = (uint64_t)p.batch * p.heads * p.nb * BS;
-    if (row_id >= total_rows) return;
-    const uint32_t qi = (uint32_t)(row_id % BS);
-    const uint32_t r = (uint32_t)((row_id / BS) % p.nb);
-    const uint32_t bh = (uint32_t)(row_id / ((uint64_t)BS * p.nb));
-    const uint32_t h = bh % p.heads;
-    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
-    const uint32_t off = lut[r].x, count = lut[r].y;
-    const uint32_t sub = lane / LPB, key0 = (lane % LPB) * 8;
-    const size_t head_base = (size_t)bh * p.blocks * BS * BS;
-    const T* dy = (const T*)p.dy + head_base;
-    const T* y = (const T*)p.y + head_base;
-    T* dx = (T*)p.dx + head_base;
-    auto load8 = [&](const T* base, uint32_t blk, float (&v)[8]) {
-        const T* src = base + ((size_t)blk * BS + qi) * BS + key0;
-        const f32x4 lo = Elem<T>::load4(src), hi = Elem<T>::load4(src + 4);
-        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
-    };
-    auto store8 = [&](uint32_t blk, const float (&v)[8]) {
-        T* dst = dx + ((size_t)blk * BS + qi) * BS + key0;
-        const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
-        Elem<T>::store4(dst, lo);
-        Elem<T>::store4(dst + 4, hi);
-    };
-    auto wave_sum = [](float l) {
+struct SoftmaxGradRows {
+    static constexpr int LPB = BS / 8, PER = 64 / LPB;
+    const sfb_uint2* lut;
+    const T* dy;
+    const T* y;
+    T* dx;
+    uint32_t off, count, sub, key0;
+    float scale;
+
+    __device__ __forceinline__ size_t at(uint32_t blk, uint32_t qi) const {
+        return ((size_t)blk * BS + qi) * BS + key0;
+    }
+    // register slots for dy and for y: 8 steps each (32 registers for bf16, 64 for fp32)
+    static constexpr int SLOTS = kSoftmaxSlots;
+    template <int R, int S>
+    __device__ __forceinline__ void in_registers(uint32_t q0) const {
+        static_assert(R * S == SLOTS, "slots");
+        Packed8<T> g[R][S], v[R][S];
+        uint32_t blk[S];
 #pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) l += __shfl_xor(l, d);
-        return l;
-    };
-    const uint32_t steps = (count + PER - 1) / PER;
-    if (steps <= CACHE) {
-        float g[CACHE][8], v[CACHE][8];
-        uint32_t blk[CACHE];
-        float sum = 0.f;
-#pragma unroll
-        for (int st = 0; st < CACHE; ++st) {
+        for (int st = 0; st < S; ++st) {
             const uint32_t j = st * PER + sub;
             blk[st] = 0xffffffffu;
-            if (j < count) {
-                blk[st] = lut[off + j].x;
-                load8(dy, blk[st], g[st]);
-                load8(y, blk[st], v[st]);
+            if (j < count) blk[st] = lut[off + j].x;
+        }
 #pragma unroll
-                for (int i = 0; i < 8; ++i) sum += g[st][i] * v[st][i];
-            }
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+                if (blk[st] != 0xffffffffu) {
+                    g[rr][st].load(dy + at(blk[st], q0 + rr));
+                    v[rr][st].load(y + at(blk[st], q0 + rr));
+                }
+        float sum[R];
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) {
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+                if (blk[st] != 0xffffffffu) {
+#pragma unroll
+                    for (int i = 0; i < 8; i += 2) {
+                        s0 = __builtin_fmaf(g[rr][st].get(i), v[rr][st].get(i), s0);
+                        s1 = __builtin_fmaf(g[rr][st].get(i + 1), v[rr][st].get(i + 1), s1);
+                    }
+                }
+            sum[rr] = s0 + s1;
+        }
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr) sum[rr] = wave_sum(sum[rr]);
+#pragma unroll
+        for (int rr = 0; rr < R; ++rr)
+#pragma unroll
+            for (int st = 0; st < S; ++st)
+                if (blk[st] != 0xffffffffu) {
+                    g[rr][st].unpack_after(sum[rr]);
+                    v[rr][st].unpack_after(sum[rr]);
+                    float out[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) out[i] = (g[rr][st].get(i) - sum[rr]) * v[rr][st].get(i) * scale;
+                    store8<T>(dx + at(blk[st], q0 + rr), out);
+                }
+    }
+    __device__ __forceinline__ void in_passes(uint32_t qi) const {
+        float sum = 0.f;
+        for (uint32_t j = sub; j < count; j += PER) {
+            const uint32_t b = lut[off + j].x;
+            float g[8], v[8];
+            load8<T>(dy + at(b, qi), g);
+            load8<T>(y + at(b, qi), v);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += g[i] * v[i];
         }
         sum = wave_sum(sum);
+        for (uint32_t j = sub; j < count; j += PER) {
+            const uint32_t b = lut[off + j].x;
+            float g[8], v[8];
+            load8<T>(dy + at(b, qi), g);
+            load8<T>(y + at(b, qi), v);
 #pragma unroll
-        for (int st = 0; st < CACHE; ++st)
-            if (blk[st] != 0xffffffffu) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) g[st][i] = (g[st][i] - sum) * v[st][i] * p.scale;
-                store8(blk[st], g[st]);
-            }
-        return;
+            for (int i = 0; i < 8; ++i) g[i] = (g[i] - sum) * v[i] * scale;
+            store8<T>(dx + at(b, qi), g);
+        }
     }
-    float sum = 0.f;
-    for (uint32_t j = sub; j < count; j += PER) {
-        const uint32_t b = lut[off + j].x;
-        float g[8], v[8];
-        load8(dy, b, g);
-        load8(y, b, v);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sum += g[i] * v[i];
-    }
-    sum = wave_sum(sum);
-    for (uint32_t j = sub; j < count; j += PER) {
-        const uint32_t b = lut[off + j].x;
-        float g[8], v[8];
-        load8(dy, b, g);
-        load8(y, b, v);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) g[i] = (g[i] - sum) * v[i] * p.scale;
-        store8(b, g);
+};
+
+template <int BS, typename T>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 2 ? 4 : 2))) void masked_softmax_grad_kernel(
+    SoftmaxGradParams p) {
+    using Rows = SoftmaxGradRows<BS, T>;
+    const SoftmaxWave w = softmax_wave<BS>(p.batch, p.heads, p.nb);
+    if (!w.valid) return;
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t h = w.bh % p.heads;
+    const size_t head_base = (size_t)w.bh * p.blocks * BS * BS;
+    Rows rows;
+    rows.lut = p.lut + (size_t)h * p.lut_stride;
+    rows.dy = (const T*)p.dy + head_base;
+    rows.y = (const T*)p.y + head_base;
+    rows.dx = (T*)p.dx + head_base;
+    rows.off = rows.lut[w.r].x;
+    rows.count = rows.lut[w.r].y;
+    rows.sub = lane / Rows::LPB;
+    rows.key0 = (lane % Rows::LPB) * 8;
+    rows.scale = p.scale;
+    constexpr int SLOTS = Rows::SLOTS;
+    const uint32_t steps = (rows.count + Rows::PER - 1) / Rows::PER;
+    if (steps <= SLOTS / 4) {
+        rows.template in_registers<4, SLOTS / 4>(w.q0);
+    } else if (steps <= SLOTS / 2) {
+        rows.template in_registers<2, SLOTS / 2>(w.q0);
+        rows.template in_registers<2, SLOTS / 2>(w.q0 + 2);
+    } else if (steps <= SLOTS) {
+        for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.template in_registers<1, SLOTS>(w.q0 + i);
+    } else {
+        for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.in_passes(w.q0 + i);
     }
 }
 
@@ -751,9 +1009,9 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     if (((uintptr_t)x | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
     SoftmaxParams p = {lut, mask, valid_len, x, y, blocks, batch_dim, head_dim, ctx_blks,
                        lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0, scale * kLog2e};
-    const uint64_t rows = (uint64_t)batch_dim * head_dim * ctx_blks * block_size;
-    if ((rows + 3) / 4 > 0x7fffffffull) return SFB_ERR_SHAPE;
-    const dim3 grid((uint32_t)((rows + 3) / 4));
+    const uint64_t groups = softmax_grid(batch_dim, head_dim, ctx_blks, block_size);
+    if (groups > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const dim3 grid((uint32_t)groups);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
 #define SFB_CALL(BSV, TX, TY) masked_softmax_kernel<BSV, TX, TY><<<grid, dim3(256), 0, s>>>(p)
@@ -809,9 +1067,9 @@ extern "C" int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (((uintptr_t)dy | (uintptr_t)y | (uintptr_t)dx) & 15u) return SFB_ERR_ALIGNMENT;
     SoftmaxGradParams p = {lut, dy, y, dx, blocks, batch_dim, head_dim, ctx_blks, lut_heads > 1 ? lut_dim : 0, scale};
-    const uint64_t rows = (uint64_t)batch_dim * head_dim * ctx_blks * block_size;
-    if ((rows + 3) / 4 > 0x7fffffffull) return SFB_ERR_SHAPE;
-    const dim3 grid((uint32_t)((rows + 3) / 4));
+    const uint64_t groups = softmax_grid(batch_dim, head_dim, ctx_blks, block_size);
+    if (groups > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const dim3 grid((uint32_t)groups);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (block_size == 64) {

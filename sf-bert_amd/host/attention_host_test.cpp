@@ -4,7 +4,8 @@
 // the two-stage fusion (fusion_attention2) and the full fusion (fusion_attention).  Unlike the
 // reference's timing harnesses it checks results: all-ones Q, K (the reference's inputs,
 // fixed_fusion_test.cu:263-268) give uniform probabilities in closed form, and on random inputs the
-// fused and unfused paths must agree.  Exit code 0 = all checks passed.
+// fused and unfused paths must agree; the backward stages (bst_sgemm_xn with TN_OP, BlocksparseMaskedSoftmaxGrad)
+// are checked through the inner-product identities of a linear and a bilinear map.  Exit code 0 = all passed.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -135,7 +136,60 @@ int main() {
     std::printf("fused (fp32) vs unfused trio (bf16 S, P): max |diff| / max |O| = %.3e\n", max_diff / max_ref);
     if (!(max_diff / max_ref < 1e-2)) ++failures;
 
-    // ---- 3. a block size the kernels do not implement is an error, not a silent no-op ----
+    // ---- 3. backward in the order of transformer_attention_optimize.cu:924-965, on the stored bf16 P ----
+    // O is linear in V and S is bilinear in Q, K, hence <dV, V> = <dO, O> and <dQ, Q> = <dK, K>.
+    {
+        std::vector<uint2> tn_lut(ctx_blks + blocks);
+        uint tn_max = 0;
+        if (sfb_build_tn_lut((sfb_uint2*)tn_lut.data(), (const sfb_uint2*)nt_lut.data(), blocks, ctx_blks, &tn_max) !=
+            SFB_OK)
+            return 1;
+        uint2* d_tn = upload(tn_lut);
+        std::vector<float> d_out(tokens * state);
+        for (size_t i = 0; i < d_out.size(); ++i) d_out[i] = (rand() % 2001 - 1000) * 1e-3f;
+        float* d_do = upload(d_out);
+        float *d_dq = nullptr, *d_dk = nullptr, *d_dv = nullptr;
+        bhalf *d_dp = nullptr, *d_ds = nullptr;
+        HIP_OK(hipMalloc((void**)&d_dq, tokens * state * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&d_dk, tokens * state * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&d_dv, tokens * state * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&d_dp, sparse * sizeof(bhalf)));
+        HIP_OK(hipMalloc((void**)&d_ds, sparse * sizeof(bhalf)));
+        const uint lut_dim = ctx_blks + blocks;
+        ok = bst_sgemm_xn(stream, d_tn, d_p, d_do, d_dv, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                          head_state_, 1, lut_dim, TN_OP, magic, shift, tn_max);
+        ok = ok && bst_sgemm_nt(stream, d_nt, d_do, d_v, d_dp, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                                head_state_, 1, blocks);
+        ok = ok && BlocksparseMaskedSoftmaxGrad<bhalf, bhalf2>(stream, d_nn, d_dp, d_p, d_ds, blk_size_, blocks,
+                                                               batch_dim, heads_, ctx_blks, 1, lut_dim, nn_max, scale);
+        ok = ok && bst_sgemm_xn(stream, d_tn, d_ds, d_q, d_dk, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                                head_state_, 1, lut_dim, TN_OP, magic, shift, tn_max);
+        ok = ok && bst_sgemm_xn(stream, d_nn, d_ds, d_k, d_dq, blk_size_, blocks, batch_dim, ctx_blks, ctx_blks, heads_,
+                                head_state_, 1, lut_dim, NN_OP, magic, shift, nn_max);
+        if (!ok) {
+            std::fprintf(stderr, "backward launcher failed: %s\n", sfb_status_string(sfb_host::last_status()));
+            return 1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<float> dq(tokens * state), dk(tokens * state), dv(tokens * state);
+        HIP_OK(hipMemcpy(dq.data(), d_dq, dq.size() * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(dk.data(), d_dk, dk.size() * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(dv.data(), d_dv, dv.size() * sizeof(float), hipMemcpyDeviceToHost));
+        double dv_v = 0, do_o = 0, dq_q = 0, dk_k = 0, dq_abs = 0;
+        for (size_t i = 0; i < dq.size(); ++i) {
+            dv_v += (double)dv[i] * v[i];
+            do_o += (double)d_out[i] * o_u[i];
+            dq_q += (double)dq[i] * q[i];
+            dk_k += (double)dk[i] * k[i];
+            dq_abs += std::fabs((double)dq[i] * q[i]);
+        }
+        std::printf("backward: <dV,V> = %.6f, <dO,O> = %.6f; <dQ,Q> = %.6f, <dK,K> = %.6f (sum |dQ Q| = %.3f)\n", dv_v,
+                    do_o, dq_q, dk_k, dq_abs);
+        if (!(std::fabs(dv_v - do_o) <= 1e-4 * std::fmax(1.0, std::fabs(do_o)) + 1e-3)) ++failures;
+        if (!(std::fabs(dq_q - dk_k) <= 1e-4 * dq_abs)) ++failures;
+    }
+
+    // ---- 4. a block size the kernels do not implement is an error, not a silent no-op ----
     if (bst_sgemm_nt(stream, d_nt, d_q, d_k, d_s, 16, blocks, batch_dim, ctx_blks, ctx_blks, heads_, head_state_, 1,
                      blocks) || sfb_host::last_status() != SFB_ERR_BLOCK_SIZE)
         ++failures;

@@ -1,4 +1,5 @@
-// The unfused trio with the reference's signatures (blocksparse.h:202, 425, 649-658, 965-972).
+// The unfused trio and its backward stages with the reference's signatures (blocksparse.h:202, 425, 649-658,
+// 965-972, 1164-1173).
 #ifndef SFB_HOST_BLOCKSPARSE_H
 #define SFB_HOST_BLOCKSPARSE_H
 
@@ -23,7 +24,19 @@ bool BlocksparseMaskedSoftmax(CUstream stream, const uint2* lut, const uint* mas
                                            head_dim, ctx_blks, lut_heads, lut_dim, max_lut, mask_heads, scale));
 }
 
-// a: bf16 probabilities (sparse), b: fp32 V, c: fp32 O.  op must be NN_OP (TN_OP is the backward product).
+// dx = (dy - sum_k dy*y) * y * scale over each sparse row (blocksparse.h:1164-1173); T = bhalf or float for dy,
+// y and dx alike; V is accepted and unused.  lut: NN LUT.
+template <typename T, typename V>
+bool BlocksparseMaskedSoftmaxGrad(CUstream stream, const uint2* lut, const T* dy, const T* y, T* dx,
+                                  uint block_size, uint blocks, uint batch_dim, uint head_dim, uint ctx_blks,
+                                  uint lut_heads, uint lut_dim, uint max_lut, float scale) {
+    return sfb_host::ok(sfb_masked_softmax_grad(stream, sfb_host::lut_cast(lut), dy, y, dx,
+                                                sfb_host::dtype_of<T>::value, block_size, blocks, batch_dim,
+                                                head_dim, ctx_blks, lut_heads, lut_dim, max_lut, scale));
+}
+
+// a: bf16 sparse operand, b: fp32 dense operand, c: fp32 result.  op = NN_OP with the NN LUT (O = P V, dQ = dS K)
+// or TN_OP with the TN LUT (dV = P^T dO, dK = dS^T Q).
 inline bool bst_sgemm_xn(CUstream stream, const uint2* lut, const bhalf* a, const float* b, float* c,
                          uint block_size, uint blocks, uint batch_dim, uint ctx_blks_b, uint ctx_blks_c,
                          uint head_dim, uint state_dim, uint lut_heads, uint lut_dim, uint op, uint magic,

@@ -52,6 +52,23 @@ def test_softmax_grad_rows_longer_than_the_register_cache(bs, nb):
     assert rel_err(got.cpu().numpy(), want) <= TOL_F32
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("nb", [12, 24, 48])
+def test_softmax_grad_every_rows_per_wave_variant(nb, bf16):
+    """Row lengths that select each register variant of the kernel (4, 2 or 1 rows of a wave at a time), with
+    causal rows so that one launch mixes them."""
+    bs = 64
+    luts = sfb.build_luts(sfb.layout_full(nb, causal=True))
+    blocks = luts["blocks"]
+    S = orc.fill_normal((1, 2, blocks, bs, bs), 15)
+    P = rounded(orc.masked_softmax(S, luts["nn_lut"], nb, 0.125), bf16)
+    dP = rounded(orc.fill_normal((1, 2, blocks, bs, bs), 16), bf16)
+    want = orc.masked_softmax_grad(dP, P, luts["nn_lut"], nb, 0.125)
+    got = sfb.BlocksparseMaskedSoftmaxGrad(sfb.to_device(luts["nn_lut"]), sparse_dev(dP, bf16), sparse_dev(P, bf16),
+                                           nb, 0.125)
+    assert rel_err(got.float().cpu().numpy(), want) <= (TOL_BF16 if bf16 else TOL_F32)
+
+
 def test_softmax_grad_in_place_and_per_head_luts():
     bs, nb, B, H = 64, 8, 2, 4
     lays = sfb.layout_fixed(H, nb, 4, causal=True)

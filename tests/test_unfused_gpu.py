@@ -121,6 +121,32 @@ def test_empty_block_rows_give_zero_output():
     assert rel_err(O, orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125)) <= TOL_F32
 
 
+@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("nb", [12, 24, 48, 70])
+def test_softmax_every_rows_per_wave_variant(nb, bf16, masked):
+    """Row lengths that select each register variant of the softmax kernel (4, 2 or 1 rows of a wave at a time,
+    and the three-pass form), with causal rows so that one launch mixes them."""
+    bs, B, H = 64, 2, 1
+    luts = sfb.build_luts(sfb.layout_full(nb, causal=True))
+    blocks = luts["blocks"]
+    S = orc.fill_normal((B, H, blocks, bs, bs), 17)
+    if bf16:
+        S = orc.round_bf16(S)
+    mask = valid = None
+    if masked:
+        mask = sfb.pack_mask(sfb.element_mask(luts["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG))
+        valid = np.array([nb * bs, nb * bs - 70], np.int32)
+    want = orc.masked_softmax(S, luts["nn_lut"], nb, 0.125, mask=mask, valid_len=valid)
+    x = torch.from_numpy(S).cuda()
+    got = sfb.BlocksparseMaskedSoftmax(
+        sfb.to_device(luts["nn_lut"]), None if mask is None else sfb.to_device(sfb.transpose_mask(mask, blocks, bs)),
+        x.to(torch.bfloat16) if bf16 else x, nb, 0.125, valid_len=None if valid is None else sfb.to_device(valid))
+    got = got.float().cpu().numpy()
+    assert rel_err(got, want) <= (TOL_BF16 if bf16 else TOL_F32)
+    assert (got[want == 0] == 0).all()
+
+
 def test_error_codes_instead_of_silent_no_op():
     q = torch.zeros((1, 64, 1, 64), device="cuda")
     lut = sfb.to_device(np.zeros((3, 2), np.uint32))
