@@ -112,6 +112,29 @@ def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
     return dict(ms_per_call=ms, fused_speedup=ms / fused_ms, sp_storage="bf16" if bf16 else "f32", **parts)
 
 
+def time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16):
+    """Backward of the unfused path from the stored P (dV, dP, dS, dK, dQ), each stage and the whole chain, with
+    the HBM rate of the two memory-bound stage types on their algorithmic bytes."""
+    B, L, H, d = q.shape
+    nb = L // bs
+    code = sfb.BF16 if bf16 else sfb.F32
+    ld = {name: sfb.to_device(luts[name]) for name in ("nt_lut", "nn_lut", "tn_lut")}
+    p = sfb.fusion_attention2(ld["nn_lut"], q, k, bs, blocks, scale, out_dtype=code)
+    d_out = torch.randn((B, L, H, d), device="cuda").to(q.dtype)
+    dp, ds = torch.empty_like(p), torch.empty_like(p)
+    c = torch.empty((B, L, H, d), device="cuda", dtype=torch.float32)
+    sparse_bytes = p.numel() * p.element_size()
+    dense_bytes = q.numel() * q.element_size()
+    tn = _time(torch, lambda: sfb.bst_sgemm_xn(ld["tn_lut"], p, d_out, nb, op=sfb.TN_OP, c=c), 200, 20)
+    grad = _time(torch, lambda: sfb.BlocksparseMaskedSoftmaxGrad(ld["nn_lut"], dp, p, nb, scale, dx=ds), 200, 20)
+    return {"ms_per_call": _time(torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale), 100, 20),
+            "dsd_tn_ms": tn, "dsd_tn_hbm_GBs": (sparse_bytes + dense_bytes + c.numel() * 4) / tn / 1e6,
+            "sdd_nt_ms": _time(torch, lambda: sfb.bst_sgemm_nt(ld["nt_lut"], d_out, v, bs, blocks, c=dp), 200, 20),
+            "softmax_grad_ms": grad, "softmax_grad_hbm_GBs": 3 * sparse_bytes / grad / 1e6,
+            "dsd_nn_ms": _time(torch, lambda: sfb.bst_sgemm_xn(ld["nn_lut"], ds, k, nb, c=c), 200, 20),
+            "sp_storage": "bf16" if bf16 else "f32"}
+
+
 def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
     """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
     B, L, ffn = 8, 4096, 3072
@@ -247,6 +270,7 @@ def main():
     }
     if not args.skip_extras:
         result["unfused"] = time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
+        result["backward_unfused"] = time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
         if args.workload == "c4":
             result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, args.max_blocks)
     if not args.no_cpu_baseline:

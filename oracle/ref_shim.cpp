@@ -45,4 +45,11 @@ void ref_embedding_lookup(float* C, float* A, int* B, int batch, int seq_len, in
     embedding_lookup(C, A, B, batch, seq_len, heads, size_per_head);
 }
 
+// labels -> one-hot (to_one_hot), then the loss; logits are overwritten by their logarithms as in the reference
+float ref_softmax_cross_entropy(float* D, float* logits, int* labels, int* one_hot_scratch, int batch, int seq_len,
+                                int vocab) {
+    to_one_hot(one_hot_scratch, labels, batch, seq_len, vocab);
+    return softmax_cross_entropy_with_logits(D, logits, one_hot_scratch, batch, seq_len, vocab);
+}
+
 }  // extern "C"

@@ -28,6 +28,11 @@
  *   orc_encoder_layer : composition of the above in the order of transformer.cpp:513-580 with the
  *       post-LN structure the workload definition asks for; checked against a float64 numpy layer.
  *   orc_f32_to_bf16_* : exhaustive check over all bf16 neighbours.
+ *   orc_softmax_cross_entropy : bit-compared with the reference's softmax_cross_entropy_with_logits + to_one_hot
+ *       in oracle/_ref + golden fixture; float64 log-sum-exp.
+ *   orc_sgemm_nt : like orc_sgemm, the reference calls OpenBLAS -- PARITY UNPINNED; float64 numpy.
+ *   orc_encoder_layer_pre_ln, orc_model_forward : compositions of the above in the order of
+ *       transformer_inference_part.cpp:190-256 (dropout omitted); checked against a float64 numpy model.
  */
 #include "sfb_oracle.h"
 
@@ -794,6 +799,135 @@ void orc_encoder_layer(float* y, const float* x, const orc_layer_weights* w,
 
     free(xr); free(wq); free(wk); free(wv); free(wo); free(w1); free(w2);
     free(q); free(k); free(v); free(a); free(t); free(x1); free(f); free(x1r);
+}
+
+/* The reference's own wiring (transformer.cpp:513-580, transformer_inference_part.cpp:209-232), pre-LN,
+ * dropout omitted:  a = LN1(x); x1 = x + (Attn(aWq+bq, aWk+bk, aWv+bv) Wo + bo);
+ *                   y = x1 + (gelu(LN2(x1) W1 + b1) W2 + b2). */
+void orc_encoder_layer_pre_ln(float* y, const float* x, const orc_layer_weights* w,
+                              const orc_uint2* nn_lut, const void* mask_block_major, int mask_word_bytes,
+                              const int32_t* valid_len, int B, int L, int H, int d, int ffn, int bs,
+                              uint32_t blocks, int operands_bf16, int nthreads) {
+    int m = B * L, n = H * d;
+    long mn = (long)m * n, mf = (long)m * ffn;
+    int r = operands_bf16;
+    float* wq = rounded_copy(w->wq, (long)n * n, r);
+    float* wk = rounded_copy(w->wk, (long)n * n, r);
+    float* wv = rounded_copy(w->wv, (long)n * n, r);
+    float* wo = rounded_copy(w->wo, (long)n * n, r);
+    float* w1 = rounded_copy(w->w1, (long)n * ffn, r);
+    float* w2 = rounded_copy(w->w2, (long)n * ffn, r);
+    float* a = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* q = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* k = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* v = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* t = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* x1 = (float*)malloc(sizeof(float) * (size_t)mn);
+    float* f = (float*)malloc(sizeof(float) * (size_t)mf);
+
+    orc_layernorm(a, NULL, NULL, x, w->ln1_g, w->ln1_b, m, n);
+    if (r) orc_round_to_bf16_rne(a, mn);
+    orc_sgemm(q, a, wq, m, n, n, nthreads); orc_bias(q, q, w->bq, n, m);
+    orc_sgemm(k, a, wk, m, n, n, nthreads); orc_bias(k, k, w->bk, n, m);
+    orc_sgemm(v, a, wv, m, n, n, nthreads); orc_bias(v, v, w->bv, n, m);
+    if (r) { orc_round_to_bf16_rne(q, mn); orc_round_to_bf16_rne(k, mn); orc_round_to_bf16_rne(v, mn); }
+    orc_blocksparse_attention(a, q, k, v, nn_lut, mask_block_major, mask_word_bytes, valid_len, B, L,
+                              H, d, bs, 1.0f / sqrtf((float)d), 1, blocks + (uint32_t)(L / bs), 1,
+                              blocks, nthreads);
+    if (r) orc_round_to_bf16_rne(a, mn);
+    orc_sgemm(t, a, wo, m, n, n, nthreads); orc_bias(t, t, w->bo, n, m);
+    orc_add(x1, x, t, mn);
+
+    orc_layernorm(a, NULL, NULL, x1, w->ln2_g, w->ln2_b, m, n);
+    if (r) orc_round_to_bf16_rne(a, mn);
+    orc_sgemm(f, a, w1, m, ffn, n, nthreads); orc_bias(f, f, w->b1, ffn, m);
+    orc_gelu(f, f, mf);
+    if (r) orc_round_to_bf16_rne(f, mf);
+    orc_sgemm(t, f, w2, m, n, ffn, nthreads); orc_bias(t, t, w->b2, n, m);
+    orc_add(y, x1, t, mn);
+
+    free(wq); free(wk); free(wv); free(wo); free(w1); free(w2);
+    free(a); free(q); free(k); free(v); free(t); free(x1); free(f);
+}
+
+/* cblas_sgemm(RowMajor, NoTrans, Trans, m, n, k, 1, A, k, W, k, 0, C, n)
+ * (transformer_inference_part.cpp:236, the tied-embedding logits): C[m][n] = A[m][k] W[n][k]^T, float
+ * accumulation in ascending k. */
+void orc_sgemm_nt(float* C, const float* A, const float* W, int m, int n, int k, int nthreads) {
+    if (nthreads < 1) nthreads = 1;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int i = 0; i < m; i++)
+        for (int j = 0; j < n; j++) {
+            float sum = 0.0f;
+            for (int p = 0; p < k; p++) sum += A[(size_t)i * k + p] * W[(size_t)j * k + p];
+            C[(size_t)i * n + j] = sum;
+        }
+}
+
+/* softmax_cross_entropy_with_logits (ewops.h:233-261) with the one-hot matrix of to_one_hot (ewops.h:352-361)
+ * given by its label column: per row, exp of every logit (double exp of the float, stored as float), their
+ * float sum in ascending column order, D = exp/sum, loss_row = sum_j -(log(D_j) * onehot_j) accumulated in
+ * float in column order, D_label -= 1; the result is the float sum of the row losses in row order divided
+ * by the row count.  d_out (rows x vocab, may be NULL) receives softmax - onehot; row_loss may be NULL. */
+float orc_softmax_cross_entropy(float* d_out, float* row_loss, const float* logits, const int32_t* labels,
+                                long rows, int vocab) {
+    float* e = (float*)malloc(sizeof(float) * (size_t)vocab);
+    float sum_of_loss = 0;
+    for (long i = 0; i < rows; i++) {
+        const float* a = logits + (size_t)i * vocab;
+        float sum_of_row = 0.0f;
+        float loss = 0;
+        for (int j = 0; j < vocab; j++) {
+            e[j] = (float)exp((double)a[j]);
+            sum_of_row += e[j];
+        }
+        for (int j = 0; j < vocab; j++) {
+            float dj = e[j] / sum_of_row;
+            float lg = (float)log((double)dj);
+            int hot = (j == labels[i]) ? 1 : 0;
+            if (d_out) d_out[(size_t)i * vocab + j] = dj - (float)hot;
+            loss += -(lg * (float)hot);
+        }
+        if (row_loss) row_loss[i] = loss;
+        sum_of_loss += loss;
+    }
+    free(e);
+    return sum_of_loss / (float)rows;
+}
+
+/* Forward pass of the whole model in the shape of transformer_inference_part.cpp:190-256 (dropout omitted):
+ * x = tok[ids] + pos; n_layers encoder layers (pre_ln != 0: the reference's wiring; 0: post-LN);
+ * logits = x tok^T (tied embedding); loss = softmax cross-entropy against labels.  logits (tokens x vocab,
+ * may be NULL) and hidden (tokens x state, may be NULL) receive the intermediate results. */
+float orc_model_forward(float* logits, float* hidden, const int32_t* ids, const int32_t* labels,
+                        const float* tok, const float* pos, const orc_layer_weights* layers, int n_layers,
+                        int pre_ln, const orc_uint2* nn_lut, const void* mask_block_major, int mask_word_bytes,
+                        const int32_t* valid_len, int B, int L, int H, int d, int ffn, int bs, uint32_t blocks,
+                        int vocab, int operands_bf16, int nthreads) {
+    long tokens = (long)B * L;
+    int n = H * d;
+    float* x = (float*)malloc(sizeof(float) * (size_t)tokens * n);
+    float* y = (float*)malloc(sizeof(float) * (size_t)tokens * n);
+    orc_embedding_lookup(x, tok, ids, tokens, n);
+    orc_add_matrix(x, x, pos, B, (long)L * n);
+    for (int i = 0; i < n_layers; i++) {
+        if (pre_ln)
+            orc_encoder_layer_pre_ln(y, x, layers + i, nn_lut, mask_block_major, mask_word_bytes, valid_len, B, L, H,
+                                     d, ffn, bs, blocks, operands_bf16, nthreads);
+        else
+            orc_encoder_layer(y, x, layers + i, nn_lut, mask_block_major, mask_word_bytes, valid_len, B, L, H, d,
+                              ffn, bs, blocks, operands_bf16, nthreads);
+        float* swap = x; x = y; y = swap;
+    }
+    if (hidden) memcpy(hidden, x, sizeof(float) * (size_t)tokens * n);
+    float* lg = logits ? logits : (float*)malloc(sizeof(float) * (size_t)tokens * vocab);
+    float* xr = rounded_copy(x, tokens * n, operands_bf16);
+    float* tr = rounded_copy(tok, (long)vocab * n, operands_bf16);
+    orc_sgemm_nt(lg, xr, tr, (int)tokens, vocab, n, nthreads);
+    float loss = orc_softmax_cross_entropy(NULL, NULL, lg, labels, tokens, vocab);
+    if (!logits) free(lg);
+    free(xr); free(tr); free(x); free(y);
+    return loss;
 }
 
 /* ------------------------------------------------------------------------------------------ */

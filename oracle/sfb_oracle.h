@@ -105,6 +105,26 @@ void orc_encoder_layer(float* y, const float* x, const orc_layer_weights* w,
                        const int32_t* valid_len, int B, int L, int H, int d, int ffn, int bs,
                        uint32_t blocks, int operands_bf16, int nthreads);
 
+/* the reference's own pre-LN wiring of the same ops (transformer.cpp:513-580) */
+void orc_encoder_layer_pre_ln(float* y, const float* x, const orc_layer_weights* w,
+                       const orc_uint2* nn_lut, const void* mask_block_major, int mask_word_bytes,
+                       const int32_t* valid_len, int B, int L, int H, int d, int ffn, int bs,
+                       uint32_t blocks, int operands_bf16, int nthreads);
+
+/* C[m][n] = A[m][k] W[n][k]^T (transformer_inference_part.cpp:236) */
+void orc_sgemm_nt(float* C, const float* A, const float* W, int m, int n, int k, int nthreads);
+
+/* ewops.h:233-261 with one-hot labels (ewops.h:352-361); returns the mean loss */
+float orc_softmax_cross_entropy(float* d_out, float* row_loss, const float* logits, const int32_t* labels,
+                                long rows, int vocab);
+
+/* transformer_inference_part.cpp:190-256 without dropout; returns the loss */
+float orc_model_forward(float* logits, float* hidden, const int32_t* ids, const int32_t* labels,
+                        const float* tok, const float* pos, const orc_layer_weights* layers, int n_layers,
+                        int pre_ln, const orc_uint2* nn_lut, const void* mask_block_major, int mask_word_bytes,
+                        const int32_t* valid_len, int B, int L, int H, int d, int ffn, int bs, uint32_t blocks,
+                        int vocab, int operands_bf16, int nthreads);
+
 /* ---- seeded generator shared by tests and bench (splitmix64 + Box-Muller) ---- */
 void orc_fill_normal(float* x, long n, uint64_t seed, float std);
 void orc_fill_uniform_int(int32_t* x, long n, uint64_t seed, int32_t lo, int32_t hi);

@@ -43,6 +43,14 @@ def main():
     orc.ref.ref_bias(P(bi), P(x), P(g), state, rows)
     np.savez_compressed(os.path.join(HERE, "layer_ops.npz"), x=x, g=g, b=b, layernorm=ln, mean=mean,
                         rstd=rstd, gelu=ge, bias=bi)
+    rows, vocab = 12, 50
+    logits = orc.fill_normal((rows, vocab), 81) * 2
+    labels = orc.fill_uniform_int((rows,), 82, 0, vocab - 1)
+    d_out, work, scratch = np.zeros_like(logits), logits.copy(), np.zeros((rows, vocab), np.int32)
+    orc.ref.ref_softmax_cross_entropy.restype = ctypes.c_float
+    loss = orc.ref.ref_softmax_cross_entropy(P(d_out), P(work), P(labels), P(scratch), 3, 4, vocab)
+    np.savez_compressed(os.path.join(HERE, "softmax_cross_entropy.npz"), logits=logits, labels=labels,
+                        loss=np.float32(loss), grad=d_out)
     print("wrote fixtures to", HERE)
 
 

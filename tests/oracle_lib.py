@@ -273,6 +273,57 @@ def encoder_layer(x, weights, nn_lut, B, L, H, d, ffn, bs, blocks, mask=None, va
     return y
 
 
+def encoder_layer_pre_ln(x, weights, nn_lut, B, L, H, d, ffn, bs, blocks, mask=None, valid_len=None,
+                         operands_bf16=False, nthreads=1):
+    keep = [np.ascontiguousarray(v, np.float32) for v in weights.values()]
+    w = LayerWeights(**{k: _p(a) for k, a in zip(weights.keys(), keep)})
+    y = np.zeros_like(x)
+    wb = 0 if mask is None else mask.dtype.itemsize
+    vl = None if valid_len is None else np.ascontiguousarray(valid_len, np.int32)
+    lib.orc_encoder_layer_pre_ln(_p(y), _p(x), C.byref(w), _p(np.ascontiguousarray(nn_lut, np.uint32)),
+                                 _p(mask), wb, _p(vl), B, L, H, d, ffn, bs, blocks, int(operands_bf16), nthreads)
+    return y
+
+
+def sgemm_nt(A, W, nthreads=1):
+    m, k = A.shape
+    n = W.shape[0]
+    out = np.zeros((m, n), np.float32)
+    lib.orc_sgemm_nt(_p(out), _p(A), _p(W), m, n, k, nthreads)
+    return out
+
+
+def softmax_cross_entropy(logits, labels, want_grad=False):
+    """(mean loss, row losses[, softmax - onehot]) of ewops.h:233-261."""
+    rows, vocab = logits.shape
+    row_loss = np.zeros(rows, np.float32)
+    d = np.zeros_like(logits) if want_grad else None
+    lib.orc_softmax_cross_entropy.restype = C.c_float
+    loss = lib.orc_softmax_cross_entropy(_p(d), _p(row_loss), _p(np.ascontiguousarray(logits, np.float32)),
+                                         _p(np.ascontiguousarray(labels, np.int32)), C.c_long(rows), vocab)
+    return (np.float32(loss), row_loss, d) if want_grad else (np.float32(loss), row_loss)
+
+
+def model_forward(ids, labels, tok, pos, layers, nn_lut, B, L, H, d, ffn, bs, blocks, pre_ln=True, mask=None,
+                  valid_len=None, operands_bf16=False, nthreads=1):
+    """(loss, logits [tokens, vocab], hidden [tokens, state]); layers: list of weight dicts."""
+    n, vocab = H * d, tok.shape[0]
+    keep = [[np.ascontiguousarray(v, np.float32) for v in w.values()] for w in layers]
+    arr = (LayerWeights * len(layers))(*[LayerWeights(**{k: _p(a) for k, a in zip(w.keys(), kp)})
+                                         for w, kp in zip(layers, keep)])
+    logits = np.zeros((B * L, vocab), np.float32)
+    hidden = np.zeros((B * L, n), np.float32)
+    wb = 0 if mask is None else mask.dtype.itemsize
+    vl = None if valid_len is None else np.ascontiguousarray(valid_len, np.int32)
+    lib.orc_model_forward.restype = C.c_float
+    loss = lib.orc_model_forward(_p(logits), _p(hidden), _p(np.ascontiguousarray(ids, np.int32)),
+                                 _p(np.ascontiguousarray(labels, np.int32)), _p(np.ascontiguousarray(tok, np.float32)),
+                                 _p(np.ascontiguousarray(pos, np.float32)), arr, len(layers), int(pre_ln),
+                                 _p(np.ascontiguousarray(nn_lut, np.uint32)), _p(mask), wb, _p(vl), B, L, H, d, ffn,
+                                 bs, blocks, vocab, int(operands_bf16), nthreads)
+    return np.float32(loss), logits, hidden
+
+
 def fill_normal(shape, seed, std=1.0):
     x = np.zeros(shape, np.float32)
     lib.orc_fill_normal(_p(x), C.c_long(x.size), C.c_uint64(seed), C.c_float(std))
