@@ -163,6 +163,43 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
     return out
 
 
+def time_model(sfb, torch, luts, bs, H, d, max_blocks):
+    """Forward pass of a whole BERT-base sized model (12 layers, hidden 768, FFN 3072, BigBird attention) with
+    tied-embedding logits and cross-entropy loss over a 30522-token vocabulary at B8 L4096."""
+    B, L, ffn, vocab, n_layers = 8, 4096, 3072, 30522, 12
+    n = H * d
+    torch.manual_seed(2)
+    layers = []
+    for _ in range(n_layers):
+        w = {}
+        for name, shape in (("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)),
+                            ("w2", (ffn, n))):
+            w[name] = torch.randn(shape, device="cuda") * 0.02
+        for name, size in (("bq", n), ("bk", n), ("bv", n), ("bo", n), ("b1", ffn), ("b2", n), ("ln1_b", n),
+                           ("ln2_b", n)):
+            w[name] = torch.zeros(size, device="cuda")
+        w["ln1_g"] = torch.ones(n, device="cuda")
+        w["ln2_g"] = torch.ones(n, device="cuda")
+        layers.append(w)
+    tok = torch.randn((vocab, n), device="cuda") * 0.02
+    pos = torch.randn((L, n), device="cuda") * 0.02
+    ids = torch.randint(0, vocab, (B, L), device="cuda", dtype=torch.int32)
+    labels = torch.randint(0, vocab, (B * L,), device="cuda", dtype=torch.int32)
+    out = {"shape": "B8 L4096, 12 layers hidden 768 heads 12 ffn 3072, BigBird block 64, vocab 30522, post-LN",
+           "gemm_flops": 2.0 * B * L * (n_layers * (4 * n * n + 2 * n * ffn) + n * vocab)}
+    for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
+        model = sfb.Model(tok, pos, layers, luts, bs, H, d, ffn, dtype=code, max_blocks=max_blocks, pre_ln=False)
+        res = {}
+
+        def step():
+            res.update(model.forward(ids, labels))
+        out["ms_per_forward_" + name] = _time(torch, step, 5, 2)
+        out["loss_" + name] = float(res["loss"])
+        del model
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +310,7 @@ def main():
         result["backward_unfused"] = time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
         if args.workload == "c4":
             result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, args.max_blocks)
+            result["model_forward"] = time_model(sfb, torch, luts, bs, H, d, args.max_blocks)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops)
     print(json.dumps(result))

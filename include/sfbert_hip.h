@@ -278,6 +278,58 @@ int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x, con
                               uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
                               uint32_t state_dim, uint32_t ffn, void* workspace, size_t workspace_bytes);
 
+/* The same layer in the reference's own wiring (transformer.cpp:513-580,
+ * transformer_inference_part.cpp:209-232; pre-LN, dropout omitted):
+ * a = LN1(x); x1 = x + Attn(aWq+bq, aWk+bk, aWv+bv) Wo + bo; y = x1 + gelu(LN2(x1) W1 + b1) W2 + b2.
+ * Arguments and workspace as sfb_encoder_layer_forward. */
+int sfb_encoder_layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
+                                     int dtype, const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                                     const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                     uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
+                                     uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                     uint32_t head_dim, uint32_t state_dim, uint32_t ffn, void* workspace,
+                                     size_t workspace_bytes);
+
+/* cblas_sgemm(RowMajor, NoTrans, Trans, m, n, k, 1, A, k, W, k, 0, C, n) (transformer_inference_part.cpp:236, the
+ * tied-embedding logits): C[m][n] = A[m][k] W[n][k]^T, a and w of dtype, c fp32.  Runs on rocBLAS. */
+int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m, uint32_t n,
+                uint32_t k);
+
+/* softmax_cross_entropy_with_logits over to_one_hot labels (ewops.h:233-261, 352-361): row_loss[r] =
+ * log(sum_j exp(logits[r][j])) - logits[r][labels[r]] (computed relative to the row maximum), loss[0] = their
+ * mean, summed in a fixed order.  d_logits (may be NULL, may alias logits) = softmax - onehot, the reference's D.
+ * A label outside [0, vocab) selects no column (row loss 0).  loss [dev] 1 float, row_loss [dev] rows floats,
+ * logits [dev] rows x vocab fp32, labels [dev] rows int32. */
+int sfb_softmax_cross_entropy(sfb_stream_t stream, float* loss, float* row_loss, float* d_logits,
+                              const float* logits, const int32_t* labels, uint64_t rows, uint32_t vocab);
+
+/* Weights of the whole model (transformer_inference_part.cpp:60-148): token embedding [vocab][state] (also the
+ * logits matrix), position embedding [ctx][state], both fp32 [dev]; tok_embed_bf16 [dev] the token embedding
+ * rounded to bf16 (needed when dtype is bf16, else may be NULL); layers: HOST array of n_layers structs of device
+ * pointers. */
+typedef struct {
+    const float* tok_embed;
+    const float* pos_embed;
+    const void* tok_embed_bf16;
+    const sfb_layer_weights* layers;
+    uint32_t n_layers;
+} sfb_model_weights;
+size_t sfb_model_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim, uint32_t state_dim,
+                                 uint32_t ffn, uint32_t vocab, int dtype);
+/* Forward pass of the whole model in the shape of transformer_inference_part.cpp:190-256 (dropout omitted):
+ * x = tok_embed[ids] + pos_embed; n_layers encoder layers (pre_ln != 0: the reference's wiring, 0: post-LN);
+ * logits = x tok_embed^T; loss[0] = mean cross-entropy against labels.  ids, labels [dev] batch*ctx int32
+ * (labels may be NULL: no loss); logits [dev] batch*ctx x vocab fp32 or NULL (kept in the workspace); hidden
+ * [dev] batch*ctx x heads*state fp32 or NULL (copy of the last layer's output); the attention arguments are
+ * those of sfb_encoder_layer_forward; workspace [dev] 256-byte aligned, sfb_model_workspace_bytes() bytes. */
+int sfb_model_forward(sfb_stream_t stream, float* loss, float* logits, float* hidden, const int32_t* ids,
+                      const int32_t* labels, const sfb_model_weights* w, int dtype, int pre_ln,
+                      const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                      const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                      uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes, uint32_t block_size,
+                      uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                      uint32_t ffn, uint32_t vocab, void* workspace, size_t workspace_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,11 +45,16 @@ def build(verbose=True, jobs=8):
     subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-w", "-o", exe,
                            os.path.join(host, "attention_host_test.cpp"), "-L" + HERE, "-lsfbert_hip",
                            "-Wl,-rpath,$ORIGIN/.."])
+    model_exe = os.path.join(host, "transformer_inference")
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-w", "-o", model_exe,
+                           os.path.join(host, "transformer_inference.cpp"), "-L" + HERE, "-lsfbert_hip",
+                           "-Wl,-rpath,$ORIGIN/.."])
     # the same headers must also be usable from a translation unit compiled by the plain host compiler
     subprocess.check_call(["g++", "-std=c++17", "-fsyntax-only", "-I/opt/rocm/include", "-x", "c++",
                            os.path.join(host, "host_headers_check.cpp")])
     if verbose:
         print("built", exe)
+        print("built", model_exe)
     return LIB
 
 

@@ -47,6 +47,7 @@ lib.sfb_count_blocks.restype = C.c_uint32
 lib.sfb_magicu64.restype = None
 lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
+lib.sfb_model_workspace_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -60,6 +61,8 @@ EXPORTED = [
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
+    "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
+    "sfb_model_forward",
 ]
 
 
@@ -467,6 +470,29 @@ def gemm(a, w):
     return c
 
 
+def gemm_nt(a, w):
+    """C[m, n] = a[m, k] @ w[n, k]^T (the tied-embedding logits, transformer_inference_part.cpp:236)."""
+    import torch
+    m, k = a.shape
+    n = w.shape[0]
+    c = torch.empty((m, n), device=a.device, dtype=torch.float32)
+    _check(lib.sfb_gemm_nt(_stream(), _dev(c), _dev(a), _dev(w), _dtype_code(a), C.c_uint32(m), C.c_uint32(n),
+                           C.c_uint32(k)), "sfb_gemm_nt")
+    return c
+
+
+def softmax_cross_entropy(logits, labels, want_grad=False, in_place=False):
+    """(mean loss [1], row losses [rows][, softmax - onehot]) of ewops.h:233-261 over int32 labels."""
+    import torch
+    rows, vocab = logits.shape
+    loss = torch.empty(1, device=logits.device, dtype=torch.float32)
+    row_loss = torch.empty(rows, device=logits.device, dtype=torch.float32)
+    d = (logits if in_place else torch.empty_like(logits)) if want_grad else None
+    _check(lib.sfb_softmax_cross_entropy(_stream(), _dev(loss), _dev(row_loss), _dev(d), _dev(logits), _dev(labels),
+                                         C.c_uint64(rows), C.c_uint32(vocab)), "sfb_softmax_cross_entropy")
+    return (loss, row_loss, d) if want_grad else (loss, row_loss)
+
+
 class LayerWeights(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "bq", "bk", "bv", "bo", "b1", "b2",
                                           "ln1_g", "ln1_b", "ln2_g", "ln2_b")]
@@ -478,10 +504,11 @@ class EncoderLayer:
     weights: dict of fp32 CUDA tensors (wq..w2 [in, out], bq..b2, ln1_g, ln1_b, ln2_g, ln2_b);
     dtype BF16 casts the six matrices to bf16 once."""
 
-    def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16):
+    def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16, pre_ln=False):
         import torch
         self.dtype, self.bs, self.heads, self.d, self.ffn = dtype, block_size, heads, head_state, ffn
         self.luts = luts
+        self.pre_ln = pre_ln   # True: the reference's own wiring (sfb_encoder_layer_forward_pre_ln)
         self.tensors = {}
         for name, t in weights.items():
             t = t.contiguous()
@@ -514,11 +541,83 @@ class EncoderLayer:
             out = torch.empty_like(x)
         ws, aws = self._workspaces(B, L, x.device)
         s = self.sched
-        _check(lib.sfb_encoder_layer_forward(
+        entry = lib.sfb_encoder_layer_forward_pre_ln if self.pre_ln else lib.sfb_encoder_layer_forward
+        _check(entry(
             _stream(), _dev(out), _dev(x), C.byref(self.c_weights), self.dtype, _dev(self.nn_lut), _dev(mask),
             _dev(valid_len), _dev(self.items), C.c_uint32(s["n_items"] if s else 0),
             C.c_uint32(s["n_heavy"] if s else 0), C.c_uint32(s["n_slots"] if s else 0), C.c_uint32(s["n_parts"] if s else 0), _dev(aws),
             C.c_size_t(aws.numel() if aws is not None else 0), C.c_uint32(self.bs), C.c_uint32(self.luts["blocks"]),
             C.c_uint32(B), C.c_uint32(L // self.bs), C.c_uint32(self.heads), C.c_uint32(self.d),
             C.c_uint32(self.ffn), _dev(ws), C.c_size_t(ws.numel())), "sfb_encoder_layer_forward")
+        return out
+
+
+class ModelWeights(C.Structure):
+    _fields_ = [("tok_embed", C.c_void_p), ("pos_embed", C.c_void_p), ("tok_embed_bf16", C.c_void_p),
+                ("layers", C.POINTER(LayerWeights)), ("n_layers", C.c_uint32)]
+
+
+class Model:
+    """Embedding + N encoder layers + tied-embedding logits + cross-entropy loss (sfb_model_forward), in the shape
+    of transformer_inference_part.cpp:190-256.
+
+    tok [vocab, state], pos [ctx, state] fp32 CUDA tensors; layers: list of weight dicts as for EncoderLayer."""
+
+    def __init__(self, tok, pos, layers, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16,
+                 pre_ln=True):
+        self.dtype, self.bs, self.heads, self.d, self.ffn, self.pre_ln = dtype, block_size, heads, head_state, ffn, pre_ln
+        self.luts = luts
+        self.tok, self.pos = tok.contiguous(), pos.contiguous()
+        self.tok16 = cast_bf16(self.tok) if dtype == BF16 else None
+        self.layer_tensors = []
+        for weights in layers:
+            tensors = {}
+            for name, t in weights.items():
+                t = t.contiguous()
+                if dtype == BF16 and name in ("wq", "wk", "wv", "wo", "w1", "w2"):
+                    t = cast_bf16(t)
+                tensors[name] = t
+            self.layer_tensors.append(tensors)
+        self.c_layers = (LayerWeights * max(len(layers), 1))(
+            *[LayerWeights(**{n: t.data_ptr() for n, t in tensors.items()}) for tensors in self.layer_tensors])
+        self.c_weights = ModelWeights(self.tok.data_ptr(), self.pos.data_ptr(),
+                                      self.tok16.data_ptr() if self.tok16 is not None else None, self.c_layers,
+                                      len(layers))
+        self.nn_lut = to_device(luts["nn_lut"])
+        self.sched = build_schedule(luts["nn_lut"], luts["nb"], max_blocks) if max_blocks else None
+        self.items = to_device(self.sched["items"]) if self.sched else None
+        self._ws = {}
+
+    def forward(self, ids, labels=None, mask=None, valid_len=None, want_logits=False, want_hidden=False):
+        """ids [B, L] int32; returns dict(loss [1] if labels given, logits, hidden)."""
+        import torch
+        B, L = ids.shape
+        vocab, n = self.tok.shape
+        key = (B, L)
+        if key not in self._ws:
+            nbytes = int(lib.sfb_model_workspace_bytes(C.c_uint32(B), C.c_uint32(L), C.c_uint32(self.heads),
+                                                       C.c_uint32(self.d), C.c_uint32(self.ffn), C.c_uint32(vocab),
+                                                       self.dtype))
+            aws = None
+            if self.sched:
+                aws = torch.zeros(max(schedule_workspace_bytes(self.sched, B, self.heads, self.bs, self.d), 256),
+                                  dtype=torch.uint8, device=ids.device)
+            self._ws[key] = (torch.empty(nbytes, dtype=torch.uint8, device=ids.device), aws)
+        ws, aws = self._ws[key]
+        out = {}
+        if labels is not None:
+            out["loss"] = torch.empty(1, device=ids.device, dtype=torch.float32)
+        if want_logits:
+            out["logits"] = torch.empty((B * L, vocab), device=ids.device, dtype=torch.float32)
+        if want_hidden:
+            out["hidden"] = torch.empty((B * L, n), device=ids.device, dtype=torch.float32)
+        s = self.sched
+        _check(lib.sfb_model_forward(
+            _stream(), _dev(out.get("loss")), _dev(out.get("logits")), _dev(out.get("hidden")), _dev(ids), _dev(labels),
+            C.byref(self.c_weights), self.dtype, int(self.pre_ln), _dev(self.nn_lut), _dev(mask), _dev(valid_len),
+            _dev(self.items), C.c_uint32(s["n_items"] if s else 0), C.c_uint32(s["n_heavy"] if s else 0),
+            C.c_uint32(s["n_slots"] if s else 0), C.c_uint32(s["n_parts"] if s else 0), _dev(aws),
+            C.c_size_t(aws.numel() if aws is not None else 0), C.c_uint32(self.bs), C.c_uint32(self.luts["blocks"]),
+            C.c_uint32(B), C.c_uint32(L // self.bs), C.c_uint32(self.heads), C.c_uint32(self.d), C.c_uint32(self.ffn),
+            C.c_uint32(vocab), _dev(ws), C.c_size_t(ws.numel())), "sfb_model_forward")
         return out

@@ -49,6 +49,25 @@ extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void
     return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
 }
 
+extern "C" int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
+                           uint32_t n, uint32_t k) {
+    if (!c || !a || !w) return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (!m || !n || !k) return SFB_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    rocblas_handle h = blas_handle();
+    if (!h) return SFB_ERR_LAUNCH;
+    if (rocblas_set_stream(h, (hipStream_t)stream) != rocblas_status_success) return SFB_ERR_LAUNCH;
+    const float alpha = 1.0f, beta = 0.0f;
+    const rocblas_datatype in = dtype == SFB_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
+    // row-major C[m][n] = A[m][k] W[n][k]^T  ==  column-major C^T[n][m] = (W^T[k][n])^T A^T[k][m]
+    const rocblas_status st = rocblas_gemm_ex(h, rocblas_operation_transpose, rocblas_operation_none, (int)n, (int)m,
+                                              (int)k, &alpha, w, in, (int)k, a, in, (int)k, &beta, c,
+                                              rocblas_datatype_f32_r, (int)n, c, rocblas_datatype_f32_r, (int)n,
+                                              rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
 extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim,
                                                     uint32_t state_dim, uint32_t ffn, int dtype) {
     const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
@@ -58,6 +77,110 @@ extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t
     size_t bytes = align256(m * (ffn > n ? ffn : n) * f32) + 3 * align256(m * n * act) + 2 * align256(m * n * f32);
     if (dtype == SFB_BF16) bytes += align256(m * (ffn > n ? ffn : n) * act);
     return bytes;
+}
+
+// Everything a layer needs besides its input, output and weights
+struct LayerArgs {
+    int dtype;
+    const sfb_uint2* nn_lut;
+    const void* mask;
+    const int32_t* valid_len;
+    const sfb_work_item* items;
+    uint32_t n_items, n_heavy, n_slots, n_parts;
+    void* attn_workspace;
+    size_t attn_workspace_bytes;
+    uint32_t block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn;
+    void* workspace;
+    size_t workspace_bytes;
+};
+
+static int attention_call(sfb_stream_t stream, const LayerArgs& g, const void* q, const void* k, const void* v,
+                          float* attn) {
+    const float scale = 1.0f / sqrtf((float)g.state_dim);
+    if (g.items)
+        return sfb_fused_attention_scheduled(stream, q, k, v, attn, g.dtype, g.nn_lut, g.mask, g.valid_len, g.items,
+                                             g.n_items, g.n_heavy, g.n_slots, g.n_parts, g.attn_workspace,
+                                             g.attn_workspace_bytes, g.block_size, g.blocks, g.batch_dim, g.ctx_blks,
+                                             g.head_dim, g.state_dim, 1, scale);
+    return sfb_fused_attention(stream, q, k, v, attn, g.dtype, g.nn_lut, g.mask, g.valid_len, nullptr, g.block_size,
+                               g.blocks, g.batch_dim, g.ctx_blks, g.head_dim, g.state_dim, 1, g.ctx_blks + g.blocks, 1,
+                               scale);
+}
+
+// The reference's own wiring (transformer.cpp:513-580, transformer_inference_part.cpp:209-232), dropout omitted:
+//     a = LN1(x);  x1 = x + (Attn(a Wq + bq, a Wk + bk, a Wv + bv) Wo + bo);  y = x1 + (gelu(LN2(x1) W1 + b1) W2 + b2)
+static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
+                                const LayerArgs& g) {
+    const uint32_t ctx = g.ctx_blks * g.block_size, ffn = g.ffn;
+    const size_t m = (size_t)g.batch_dim * ctx, n = (size_t)g.head_dim * g.state_dim;
+    const int dtype = g.dtype;
+    const bool bf = dtype == SFB_BF16;
+    const size_t act = bf ? 2 : 4, wide = ffn > n ? ffn : n;
+    uint8_t* p = (uint8_t*)g.workspace;
+    float* t = (float*)p;            p += align256(m * wide * sizeof(float));
+    void* q = p;                     p += align256(m * n * act);
+    void* k = p;                     p += align256(m * n * act);
+    void* v = p;                     p += align256(m * n * act);
+    float* attn = (float*)p;         p += align256(m * n * sizeof(float));
+    float* x1 = (float*)p;           p += align256(m * n * sizeof(float));
+    void* xa = bf ? (void*)p : nullptr;
+    int rc;
+#define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
+    // LN1 straight into the compute dtype; the fp32 path borrows the attention output buffer, which is free
+    // until the attention runs
+    void* a = bf ? xa : (void*)attn;
+    SFB_TRY(sfb_layernorm(stream, a, dtype, nullptr, nullptr, x, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, a, wt->wq, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, q, dtype, t, wt->bq, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, a, wt->wk, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, k, dtype, t, wt->bk, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, a, wt->wv, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, v, dtype, t, wt->bv, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(attention_call(stream, g, q, k, v, attn));
+    const void* ain = attn;
+    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, attn, m * n)); ain = xa; }
+    SFB_TRY(sfb_gemm(stream, t, ain, wt->wo, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, x1, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
+    // LN2 into the compute dtype (fp32: the attention output buffer again, consumed by the GEMM above)
+    void* a2 = bf ? xa : (void*)attn;
+    SFB_TRY(sfb_layernorm(stream, a2, dtype, nullptr, nullptr, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
+    SFB_TRY(sfb_gemm(stream, t, a2, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+    void* gl = bf ? xa : (void*)t;
+    SFB_TRY(sfb_bias_act(stream, gl, dtype, t, wt->b1, nullptr, 1, m, ffn));
+    float* t2 = bf ? t : attn;
+    SFB_TRY(sfb_gemm(stream, t2, gl, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn));
+    SFB_TRY(sfb_bias_act(stream, y, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
+#undef SFB_TRY
+    return SFB_OK;
+}
+
+static int check_layer_args(const float* y, const float* x, const sfb_layer_weights* wt, const LayerArgs& g) {
+    if (!y || !x || !wt || !g.nn_lut || !g.workspace) return SFB_ERR_NULL_POINTER;
+    if (g.dtype != SFB_F32 && g.dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    const uint32_t ctx = g.ctx_blks * g.block_size;
+    const size_t m = (size_t)g.batch_dim * ctx, n = (size_t)g.head_dim * g.state_dim;
+    if (!m || !n || !g.ffn || (n & 3u) || (g.ffn & 3u)) return SFB_ERR_SHAPE;
+    if (g.workspace_bytes <
+            sfb_encoder_layer_workspace_bytes(g.batch_dim, ctx, g.head_dim, g.state_dim, g.ffn, g.dtype) ||
+        ((uintptr_t)g.workspace & 255u))
+        return SFB_ERR_WORKSPACE;
+    return SFB_OK;
+}
+
+extern "C" int sfb_encoder_layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x,
+                                                const sfb_layer_weights* wt, int dtype, const sfb_uint2* nn_lut,
+                                                const void* mask, const int32_t* valid_len,
+                                                const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                                                uint32_t n_slots, uint32_t n_parts, void* attn_workspace,
+                                                size_t attn_workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                                uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                                uint32_t state_dim, uint32_t ffn, void* workspace,
+                                                size_t workspace_bytes) {
+    const LayerArgs g = {dtype, nn_lut, mask, valid_len, items, n_items, n_heavy, n_slots, n_parts, attn_workspace,
+                         attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
+                         workspace, workspace_bytes};
+    const int rc = check_layer_args(y, x, wt, g);
+    return rc != SFB_OK ? rc : layer_forward_pre_ln(stream, y, x, wt, g);
 }
 
 extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x,
@@ -144,6 +267,82 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
         SFB_TRY(sfb_bias_act(stream, t2, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
         SFB_TRY(sfb_layernorm(stream, y, SFB_F32, nullptr, nullptr, t2, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
     }
+#undef SFB_TRY
+    return SFB_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Whole-model forward in the shape of transformer_inference_part.cpp:190-256 (dropout omitted):
+// embedding gather + position add, n_layers encoder layers, tied-embedding logits, cross-entropy loss.
+// ------------------------------------------------------------------------------------------------
+extern "C" size_t sfb_model_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim, uint32_t state_dim,
+                                            uint32_t ffn, uint32_t vocab, int dtype) {
+    const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
+    // layer workspace; two activation buffers (fp32); logits (fp32); row losses; bf16 copy of the last hidden state
+    size_t bytes = align256(sfb_encoder_layer_workspace_bytes(batch_dim, ctx, head_dim, state_dim, ffn, dtype)) +
+                   2 * align256(m * n * sizeof(float)) + align256(m * (size_t)vocab * sizeof(float)) +
+                   align256(m * sizeof(float));
+    if (dtype == SFB_BF16) bytes += align256(m * n * 2);
+    return bytes;
+}
+
+extern "C" int sfb_model_forward(sfb_stream_t stream, float* loss, float* logits, float* hidden, const int32_t* ids,
+                                 const int32_t* labels, const sfb_model_weights* w, int dtype, int pre_ln,
+                                 const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                                 const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                 uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
+                                 uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                 uint32_t head_dim, uint32_t state_dim, uint32_t ffn, uint32_t vocab, void* workspace,
+                                 size_t workspace_bytes) {
+    if (!ids || !w || !w->tok_embed || !w->pos_embed || (w->n_layers && !w->layers) || !nn_lut || !workspace)
+        return SFB_ERR_NULL_POINTER;
+    if (labels && !loss) return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (dtype == SFB_BF16 && !w->tok_embed_bf16) return SFB_ERR_NULL_POINTER;
+    const uint32_t ctx = ctx_blks * block_size;
+    const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
+    if (!m || !n || !ffn || !vocab || (n & 3u) || (ffn & 3u)) return SFB_ERR_SHAPE;
+    if (workspace_bytes < sfb_model_workspace_bytes(batch_dim, ctx, head_dim, state_dim, ffn, vocab, dtype) ||
+        ((uintptr_t)workspace & 255u))
+        return SFB_ERR_WORKSPACE;
+    const size_t layer_bytes = align256(sfb_encoder_layer_workspace_bytes(batch_dim, ctx, head_dim, state_dim, ffn, dtype));
+    uint8_t* p = (uint8_t*)workspace;
+    void* layer_ws = p;              p += layer_bytes;
+    float* xa = (float*)p;           p += align256(m * n * sizeof(float));
+    float* xb = (float*)p;           p += align256(m * n * sizeof(float));
+    float* lg = (float*)p;           p += align256(m * (size_t)vocab * sizeof(float));
+    float* row_loss = (float*)p;     p += align256(m * sizeof(float));
+    void* x16 = dtype == SFB_BF16 ? (void*)p : nullptr;
+    if (logits) lg = logits;
+    int rc;
+#define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
+    SFB_TRY(sfb_embedding_lookup(stream, xa, w->tok_embed, ids, w->pos_embed, m, (uint32_t)n, ctx, vocab));
+    for (uint32_t i = 0; i < w->n_layers; ++i) {
+        if (pre_ln)
+            SFB_TRY(sfb_encoder_layer_forward_pre_ln(stream, xb, xa, w->layers + i, dtype, nn_lut, mask, valid_len, items,
+                                                     n_items, n_heavy, n_slots, n_parts, attn_workspace,
+                                                     attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks,
+                                                     head_dim, state_dim, ffn, layer_ws, layer_bytes));
+        else
+            SFB_TRY(sfb_encoder_layer_forward(stream, xb, xa, w->layers + i, dtype, nn_lut, mask, valid_len, items,
+                                              n_items, n_heavy, n_slots, n_parts, attn_workspace, attn_workspace_bytes,
+                                              block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
+                                              layer_ws, layer_bytes));
+        float* swap = xa; xa = xb; xb = swap;
+    }
+    if (hidden && hipMemcpyAsync(hidden, xa, m * n * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)stream) !=
+                      hipSuccess)
+        return SFB_ERR_LAUNCH;
+    // logits = hidden . tok_embed^T (transformer_inference_part.cpp:236)
+    const void* hin = xa;
+    const void* table = w->tok_embed;
+    if (dtype == SFB_BF16) {
+        SFB_TRY(sfb_cast_f32_bf16(stream, x16, xa, m * n));
+        hin = x16;
+        table = w->tok_embed_bf16;
+    }
+    SFB_TRY(sfb_gemm_nt(stream, lg, hin, table, dtype, (uint32_t)m, vocab, (uint32_t)n));
+    if (labels) SFB_TRY(sfb_softmax_cross_entropy(stream, loss, row_loss, nullptr, lg, labels, m, vocab));
 #undef SFB_TRY
     return SFB_OK;
 }

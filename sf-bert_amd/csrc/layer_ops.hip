@@ -147,6 +147,70 @@ __global__ __launch_bounds__(256) void embedding_kernel(float* out, const float*
     }
 }
 
+// Softmax cross-entropy of one row per work-group (ewops.h:233-261 with the one-hot matrix of ewops.h:352-361
+// given by its label): loss = log(sum_j exp(x_j)) - x_label, computed relative to the row maximum;
+// d (optional) = softmax(x) - onehot.  A label outside [0, vocab) selects no column: loss 0, no -1 in d.
+__global__ __launch_bounds__(256) void cross_entropy_kernel(float* row_loss, float* d, const float* logits,
+                                                            const int32_t* labels, uint32_t vocab) {
+    __shared__ float red[4];
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const size_t row = blockIdx.x;
+    const float* x = logits + row * vocab;
+    const int32_t label = labels[row];
+    const bool hot = label >= 0 && (uint32_t)label < vocab;
+    const float x_label = hot ? x[label] : 0.f;   // read before d may overwrite the row in place
+    // one pass over the row: running maximum and the sum of exponentials relative to it, four columns per step
+    float m = -3.0e38f, sum = 0.f;
+    for (uint32_t j0 = t; j0 < vocab; j0 += 1024) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = (j0 + 256 * u < vocab) ? x[j0 + 256 * u] : -3.0e38f;
+        const float m_new = fmaxf(fmaxf(fmaxf(m, v[0]), fmaxf(v[1], v[2])), v[3]);
+        sum *= exp2_fast((m - m_new) * kLog2e);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum += exp2_fast((v[u] - m_new) * kLog2e);
+        m = m_new;
+    }
+    // merge the (maximum, sum) pairs of the 256 threads
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        const float m_o = __shfl_xor(m, s), sum_o = __shfl_xor(sum, s);
+        const float m_new = fmaxf(m, m_o);
+        sum = sum * exp2_fast((m - m_new) * kLog2e) + sum_o * exp2_fast((m_o - m_new) * kLog2e);
+        m = m_new;
+    }
+    __shared__ float red_sum[4];
+    if (lane == 0) { red[wave] = m; red_sum[wave] = sum; }
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    sum = 0.f;
+#pragma unroll
+    for (int w4 = 0; w4 < 4; ++w4) sum += red_sum[w4] * exp2_fast((red[w4] - m) * kLog2e);
+    if (t == 0) row_loss[row] = hot ? (m + logf(sum)) - x_label : 0.f;
+    if (d) {
+        const float inv = 1.0f / sum;
+        float* out = d + row * vocab;
+        for (uint32_t j = t; j < vocab; j += 256) {
+            const float pj = exp2_fast((x[j] - m) * kLog2e) * inv;
+            out[j] = (hot && j == (uint32_t)label) ? pj - 1.0f : pj;
+        }
+    }
+}
+
+// out[0] = (sum of in[0..n)) / n by one work-group, in a fixed order: every launch gives the same bits
+__global__ __launch_bounds__(1024) void mean_kernel(float* out, const float* in, uint64_t n) {
+    __shared__ float red[1024];
+    float sum = 0.f;
+    for (uint64_t i = threadIdx.x; i < n; i += 1024) sum += in[i];
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (uint32_t s = 512; s >= 1; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0] / (float)n;
+}
+
 static inline uint32_t grid_for(uint64_t work_items) {
     const uint64_t blocks = (work_items + 255) / 256;
     return (uint32_t)(blocks < 1 ? 1 : (blocks > 16384 ? 16384 : blocks));
@@ -244,5 +308,17 @@ extern "C" int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in
     clear_stale_error();
     bias_act_kernel<__bf16, 0><<<dim3(grid_for(n / 4)), 256, 0, (hipStream_t)stream>>>(
         (__bf16*)out, in, nullptr, nullptr, n / 4, 1);
+    return launched();
+}
+
+extern "C" int sfb_softmax_cross_entropy(sfb_stream_t stream, float* loss, float* row_loss, float* d_logits,
+                                         const float* logits, const int32_t* labels, uint64_t rows,
+                                         uint32_t vocab) {
+    if (!loss || !row_loss || !logits || !labels) return SFB_ERR_NULL_POINTER;
+    if (rows == 0 || rows > 0x7fffffffull || vocab == 0) return SFB_ERR_SHAPE;
+    clear_stale_error();
+    cross_entropy_kernel<<<dim3((uint32_t)rows), 256, 0, (hipStream_t)stream>>>(row_loss, d_logits, logits, labels,
+                                                                                vocab);
+    mean_kernel<<<dim3(1), 1024, 0, (hipStream_t)stream>>>(loss, row_loss, rows);
     return launched();
 }

@@ -34,4 +34,13 @@ inline bool embedding_lookup(float* C, const float* A, const int* B, int batch_s
                                              (uint32_t)(head_num * size_per_head), (uint32_t)seq_len, (uint32_t)vocab));
 }
 
+// The loss of ewops.h:233-261 over integer labels (the reference expands them with to_one_hot, ewops.h:352-361,
+// and returns the mean on the host).  loss: 1 float, row_loss: batch*seq floats, D: softmax - onehot or NULL; all
+// device pointers.
+inline bool softmax_cross_entropy_with_logits(float* loss, float* row_loss, float* D, const float* A, const int* labels,
+                                              int batch_size, int seq_len, int vocab_size, CUstream stream = nullptr) {
+    return sfb_host::ok(sfb_softmax_cross_entropy(stream, loss, row_loss, D, A, labels,
+                                                  (uint64_t)batch_size * seq_len, (uint32_t)vocab_size));
+}
+
 #endif

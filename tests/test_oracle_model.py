@@ -59,7 +59,7 @@ def test_sgemm_nt_is_a_textbook_product():
     assert np.array_equal(orc.sgemm_nt(A, W), orc.sgemm_nt(A, W, nthreads=3))
 
 
-def make_model(n_layers, n, ffn, vocab, L, seed):
+def make_model(n_layers, n, ffn, vocab, L, seed, tok_std=0.5):
     layers = []
     for i in range(n_layers):
         s = seed + 100 * i
@@ -74,7 +74,7 @@ def make_model(n_layers, n, ffn, vocab, L, seed):
         w["ln2_g"] = orc.fill_normal((n,), s + 22, 0.1) + 1
         w["ln2_b"] = orc.fill_normal((n,), s + 23, 0.1)
         layers.append(w)
-    tok = orc.fill_normal((vocab, n), seed + 50, 0.5)
+    tok = orc.fill_normal((vocab, n), seed + 50, tok_std)
     pos = orc.fill_normal((L, n), seed + 51, 0.5)
     return layers, tok, pos
 
