@@ -163,6 +163,17 @@ int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
+/* The same launch with the output element type chosen by the caller: o [dev] [batch, ctx, heads, state] of
+ * out_dtype (SFB_F32 or SFB_BF16).  bf16 output is the fp32 result rounded once to nearest even; it feeds a bf16
+ * GEMM (the layer's output projection) without a separate conversion pass. */
+int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const void* k, const void* v,
+                                  void* o, int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                  const int32_t* valid_len, const sfb_work_item* items,
+                                  uint32_t n_items, uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts,
+                                  void* workspace, size_t workspace_bytes, uint32_t block_size,
+                                  uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                  uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
+                                  float scale);
 
 /* ---- the unfused trio (kept as the no_fusion comparison) ------------------------------------ */
 
@@ -255,6 +266,14 @@ int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in, uint64_t 
  * a and w of dtype (fp32, or bf16 with fp32 accumulation), c fp32.  Runs on rocBLAS. */
 int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m, uint32_t n,
              uint32_t k);
+
+/* The same product followed by bias (ewops.h:10-17), as the reference issues them back to back
+ * (transformer.cpp:516-527), in one kernel: C[m][n] = A[m][k] W[k][n] + bias[n], c of out_dtype (fp32 or bf16,
+ * rounded once from the fp32 sum).  Runs on hipBLASLt with the bias in the GEMM epilogue; returns SFB_ERR_LAUNCH
+ * if that library has no kernel for the shape and out_dtype is bf16 (fp32 output falls back to sfb_gemm +
+ * sfb_bias_act in place).  n % 4 == 0. */
+int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w, const float* bias,
+                  int dtype, uint32_t m, uint32_t n, uint32_t k);
 
 /* Weights of one encoder layer, [in][out] row-major (transformer.cpp:98-136): matrices in the compute
  * dtype (fp32 or bf16), biases and LayerNorm parameters fp32.  All [dev]. */

@@ -34,7 +34,7 @@ def build(verbose=True, jobs=8):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))
         if verbose and text.strip():
             print(text)
-    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-L/opt/rocm/lib", "-lrocblas"]
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-L/opt/rocm/lib", "-lrocblas", "-lhipblaslt"]
     extra = [l for l in os.environ.get("SFB_EXTRA_LIBS", "").split() if l]
     subprocess.check_call(link + extra)
     if verbose:

@@ -57,10 +57,10 @@ EXPORTED = [
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
-    "sfb_fused_attention", "sfb_fused_attention_scheduled",
+    "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
-    "sfb_gemm", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
+    "sfb_gemm", "sfb_gemm_bias", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
     "sfb_model_forward",
 ]
@@ -255,13 +255,26 @@ def fused_attention(q, k, v, nn_lut, block_size, blocks, scale, mask=None, valid
 
 
 def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_size, blocks, scale,
-                              mask=None, valid_len=None, mask_heads=1, out=None):
+                              mask=None, valid_len=None, mask_heads=1, out=None, out_dtype=F32):
     """fused_attention over sfb_build_schedule's work items; `items` and `workspace` are device buffers
-    (workspace: zero-filled uint8 tensor of schedule_workspace_bytes(), or None if nothing is split)."""
+    (workspace: zero-filled uint8 tensor of schedule_workspace_bytes(), or None if nothing is split).
+    out_dtype BF16 (or a bf16 `out`) takes the sfb_fused_attention_scheduled_to entry point."""
     import torch
     B, L, H, d = q.shape
     if out is None:
-        out = torch.empty((B, L, H, d), dtype=torch.float32, device=q.device)
+        out = torch.empty((B, L, H, d), dtype=_torch_dtype(out_dtype), device=q.device)
+    if out.dtype == torch.bfloat16:
+        for t in (q, k, v, out):
+            if not t.is_contiguous():
+                raise SfbError(4, "non-contiguous tensor")
+        ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+        _check(lib.sfb_fused_attention_scheduled_to(
+            _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dtype_code(q), BF16, _dev(nn_lut), _dev(mask),
+            _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]),
+            C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes),
+            C.c_uint32(block_size), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H),
+            C.c_uint32(d), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled_to")
+        return out
     nb = L // block_size
     for t in (q, k, v, out):
         if not t.is_contiguous():
@@ -467,6 +480,18 @@ def gemm(a, w):
     c = torch.empty((m, n), device=a.device, dtype=torch.float32)
     _check(lib.sfb_gemm(_stream(), _dev(c), _dev(a), _dev(w), _dtype_code(a), C.c_uint32(m), C.c_uint32(n),
                         C.c_uint32(k)), "sfb_gemm")
+    return c
+
+
+def gemm_bias(a, w, bias, out_dtype=None):
+    """C[m, n] = a[m, k] @ w[k, n] + bias[n] in one kernel; C in a's dtype unless out_dtype says otherwise."""
+    import torch
+    m, k = a.shape
+    n = w.shape[1]
+    code = _dtype_code(a) if out_dtype is None else out_dtype
+    c = torch.empty((m, n), device=a.device, dtype=_torch_dtype(code))
+    _check(lib.sfb_gemm_bias(_stream(), _dev(c), code, _dev(a), _dev(w), _dev(bias), _dtype_code(a), C.c_uint32(m),
+                             C.c_uint32(n), C.c_uint32(k)), "sfb_gemm_bias")
     return c
 
 

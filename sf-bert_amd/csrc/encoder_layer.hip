@@ -8,9 +8,12 @@
 // C, n), transformer.cpp:516); the GEMM is issued column-major as C^T = W^T A^T, the same trick as the
 // reference's cuBLAS calls (transformer_attention_optimize.cu:693-716).
 #include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
 #include <rocblas/rocblas.h>
 
+#include <map>
 #include <mutex>
+#include <tuple>
 
 #include "../../include/sfbert_hip.h"
 
@@ -27,6 +30,56 @@ rocblas_handle blas_handle() {
 }
 
 inline size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// GEMM with the bias add and the output conversion in its epilogue (hipBLASLt).  One plan per problem shape,
+// made on first use and kept; no workspace is requested, so nothing is allocated on the device.
+struct LtPlan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    bool usable = false;
+};
+hipblasLtHandle_t g_lt = nullptr;
+std::map<std::tuple<uint32_t, uint32_t, uint32_t, int, int>, LtPlan> g_plans;
+
+// row-major C[m][n] = A[m][k] W[k][n] + bias[n]  ==  column-major D[n][m] = W'[n][k] A'[k][m] + bias (per row of D)
+LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype) {
+    const auto key = std::make_tuple(m, n, k, dtype, out_dtype);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) return it->second;
+    LtPlan& p = g_plans[key];
+    if (!g_lt && hipblasLtCreate(&g_lt) != HIPBLAS_STATUS_SUCCESS) { g_lt = nullptr; return p; }
+    const hipDataType in = dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
+    const hipDataType out = out_dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
+    const hipblasOperation_t none = HIPBLAS_OP_N;
+    const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    const hipDataType bias_type = HIP_R_32F;
+    bool ok = hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.w, in, n, k, n) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.a, in, k, m, k) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out, n, m, n) == HIPBLAS_STATUS_SUCCESS;
+    if (!ok) return p;
+    // the heuristic needs a bias pointer to be present in the descriptor; the real one is set per call
+    const void* placeholder = &p;
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &placeholder, sizeof(placeholder));
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
+    const uint64_t no_workspace = 0;
+    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &no_workspace, sizeof(no_workspace));
+    hipblasLtMatmulHeuristicResult_t result;
+    int found = 0;
+    if (hipblasLtMatmulAlgoGetHeuristic(g_lt, p.desc, p.w, p.a, p.c, p.c, pref, 1, &result, &found) == HIPBLAS_STATUS_SUCCESS &&
+        found > 0 && result.workspaceSize == 0) {
+        p.algo = result.algo;
+        p.usable = true;
+    }
+    hipblasLtMatmulPreferenceDestroy(pref);
+    return p;
+}
 
 }  // namespace
 
@@ -47,6 +100,32 @@ extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void
                                               rocblas_datatype_f32_r, (int)n, c, rocblas_datatype_f32_r, (int)n,
                                               rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
     return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
+}
+
+extern "C" int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
+                             const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k) {
+    if (!c || !a || !w || !bias) return SFB_ERR_NULL_POINTER;
+    if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
+    if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        LtPlan& p = lt_plan(m, n, k, dtype, out_dtype);
+        if (p.usable) {
+            const float alpha = 1.0f, beta = 0.0f;
+            const void* bias_ptr = bias;
+            if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) ==
+                    HIPBLAS_STATUS_SUCCESS &&
+                hipblasLtMatmul(g_lt, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo, nullptr, 0,
+                                (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS)
+                return SFB_OK;
+            p.usable = false;   // do not try this plan again
+        }
+    }
+    // no fused kernel for this shape: plain GEMM, then the bias pass.  The fp32 product needs room: in place for
+    // fp32 output, otherwise there is none here
+    if (out_dtype != SFB_F32) return SFB_ERR_LAUNCH;
+    const int rc = sfb_gemm(stream, (float*)c, a, w, dtype, m, n, k);
+    return rc != SFB_OK ? rc : sfb_bias_act(stream, c, SFB_F32, (const float*)c, bias, nullptr, 0, m, n);
 }
 
 extern "C" int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
@@ -94,6 +173,39 @@ struct LayerArgs {
     size_t workspace_bytes;
 };
 
+// out = a W + bias in the compute dtype: one GEMM with the bias in its epilogue, or, where that is not available,
+// GEMM into the fp32 scratch t followed by the bias pass
+static int project(sfb_stream_t stream, void* out, int out_dtype, float* t, const void* a, const void* w,
+                   const float* bias, int dtype, size_t m, uint32_t n, uint32_t k) {
+    if (sfb_gemm_bias(stream, out, out_dtype, a, w, bias, dtype, (uint32_t)m, n, k) == SFB_OK) return SFB_OK;
+    const int rc = sfb_gemm(stream, t, a, w, dtype, (uint32_t)m, n, k);
+    return rc != SFB_OK ? rc : sfb_bias_act(stream, out, out_dtype, t, bias, nullptr, 0, m, n);
+}
+
+// Attention output as the operand of the output projection: *ain points at it.  A scheduled bf16 launch writes
+// bf16 straight into lp; otherwise the fp32 result in attn is used (fp32 path) or cast into lp (bf16 path).
+static int attention_call(sfb_stream_t stream, const LayerArgs& g, const void* q, const void* k, const void* v,
+                          float* attn);
+static int attention_operand(sfb_stream_t stream, const LayerArgs& g, const void* q, const void* k, const void* v,
+                             float* attn, void* lp, size_t elements, const void** ain) {
+    const float scale = 1.0f / sqrtf((float)g.state_dim);
+    if (g.dtype == SFB_BF16 && g.items) {
+        *ain = lp;
+        return sfb_fused_attention_scheduled_to(stream, q, k, v, lp, g.dtype, SFB_BF16, g.nn_lut, g.mask, g.valid_len,
+                                                g.items, g.n_items, g.n_heavy, g.n_slots, g.n_parts, g.attn_workspace,
+                                                g.attn_workspace_bytes, g.block_size, g.blocks, g.batch_dim, g.ctx_blks,
+                                                g.head_dim, g.state_dim, 1, scale);
+    }
+    int rc = attention_call(stream, g, q, k, v, attn);
+    if (rc != SFB_OK) return rc;
+    *ain = attn;
+    if (g.dtype == SFB_BF16) {
+        rc = sfb_cast_f32_bf16(stream, lp, attn, elements);
+        *ain = lp;
+    }
+    return rc;
+}
+
 static int attention_call(sfb_stream_t stream, const LayerArgs& g, const void* q, const void* k, const void* v,
                           float* attn) {
     const float scale = 1.0f / sqrtf((float)g.state_dim);
@@ -130,17 +242,13 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     // until the attention runs
     void* a = bf ? xa : (void*)attn;
     SFB_TRY(sfb_layernorm(stream, a, dtype, nullptr, nullptr, x, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, a, wt->wq, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, q, dtype, t, wt->bq, nullptr, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, a, wt->wk, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, k, dtype, t, wt->bk, nullptr, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, a, wt->wv, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, v, dtype, t, wt->bv, nullptr, 0, m, (uint32_t)n));
-    SFB_TRY(attention_call(stream, g, q, k, v, attn));
-    const void* ain = attn;
-    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, attn, m * n)); ain = xa; }
-    SFB_TRY(sfb_gemm(stream, t, ain, wt->wo, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, x1, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
+    SFB_TRY(project(stream, q, dtype, t, a, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, k, dtype, t, a, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, v, dtype, t, a, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n));
+    const void* ain = nullptr;
+    SFB_TRY(attention_operand(stream, g, q, k, v, attn, xa, m * n, &ain));
+    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(sfb_bias_act(stream, x1, SFB_F32, t, nullptr, x, 0, m, (uint32_t)n));
     // LN2 into the compute dtype (fp32: the attention output buffer again, consumed by the GEMM above)
     void* a2 = bf ? xa : (void*)attn;
     SFB_TRY(sfb_layernorm(stream, a2, dtype, nullptr, nullptr, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
@@ -216,35 +324,27 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     // Q, K, V projections (+ bias), stored in the compute dtype for the attention kernel
     const void* xin = x;
     if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x, m * n)); xin = xa; }
-    SFB_TRY(sfb_gemm(stream, t, xin, wt->wq, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, q, dtype, t, wt->bq, nullptr, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, xin, wt->wk, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, k, dtype, t, wt->bk, nullptr, 0, m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, xin, wt->wv, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(sfb_bias_act(stream, v, dtype, t, wt->bv, nullptr, 0, m, (uint32_t)n));
+    SFB_TRY(project(stream, q, dtype, t, xin, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, k, dtype, t, xin, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n));
 
     // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
-    if (items)
-        SFB_TRY(sfb_fused_attention_scheduled(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, items, n_items,
-                                              n_heavy, n_slots, n_parts, attn_workspace, attn_workspace_bytes, block_size,
-                                              blocks, batch_dim, ctx_blks, head_dim, state_dim, 1, scale));
-    else
-        SFB_TRY(sfb_fused_attention(stream, q, k, v, attn, dtype, nn_lut, mask, valid_len, nullptr, block_size,
-                                    blocks, batch_dim, ctx_blks, head_dim, state_dim, 1, ctx_blks + blocks, 1,
-                                    scale));
+    const LayerArgs args = {dtype, nn_lut, mask, valid_len, items, n_items, n_heavy, n_slots, n_parts, attn_workspace,
+                         attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
+                         workspace, workspace_bytes};
+    const void* ain = nullptr;
+    SFB_TRY(attention_operand(stream, args, q, k, v, attn, xa, m * n, &ain));
 
-    // output projection + bias + residual, LayerNorm 1
-    const void* ain = attn;
-    if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, attn, m * n)); ain = xa; }
-    SFB_TRY(sfb_gemm(stream, t, ain, wt->wo, dtype, (uint32_t)m, (uint32_t)n, (uint32_t)n));
-    // bias + residual + LayerNorm 1 in one pass when the row fits in registers; the bf16 path gets its
-    // copy of x1 for the next GEMM from the same kernel
+    // output projection + bias, residual, LayerNorm 1
+    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n));
+    // residual + LayerNorm 1 in one pass when the row fits in registers; the bf16 path gets its copy of x1
+    // for the next GEMM from the same kernel
     const bool fused_ln = n <= 2048;
     if (fused_ln) {
-        SFB_TRY(sfb_bias_residual_layernorm(stream, x1, bf ? xa : nullptr, t, wt->bo, x, wt->ln1_g, wt->ln1_b,
+        SFB_TRY(sfb_bias_residual_layernorm(stream, x1, bf ? xa : nullptr, t, nullptr, x, wt->ln1_g, wt->ln1_b,
                                             (uint32_t)m, (uint32_t)n));
     } else {
-        SFB_TRY(sfb_bias_act(stream, t, SFB_F32, t, wt->bo, x, 0, m, (uint32_t)n));
+        SFB_TRY(sfb_bias_act(stream, t, SFB_F32, t, nullptr, x, 0, m, (uint32_t)n));
         SFB_TRY(sfb_layernorm(stream, x1, SFB_F32, nullptr, nullptr, t, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
     }
 

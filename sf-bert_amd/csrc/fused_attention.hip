@@ -23,7 +23,7 @@ struct FusedParams {
     const void* q;
     const void* k;
     const void* v;
-    float* o;
+    float* o;                       // fp32, or bf16 (o_bf16 != 0) behind the same pointer
     const sfb_uint2* nn_lut;
     const void* mask;               // block-major keep words, or nullptr
     const int32_t* valid_len;       // per batch, or nullptr
@@ -32,6 +32,7 @@ struct FusedParams {
     uint32_t* counters;             // [batch*heads][n_slots] arrival counters of split rows
     float* partials;                // [batch*heads][n_parts][BS*D + 4*BS]
     uint32_t n_slots, n_parts;
+    uint32_t o_bf16;                // output element type: 0 fp32, 1 bf16 (rounded once from the fp32 result)
     uint32_t batch, heads, nb, blocks;
     uint32_t lut_stride;            // entries between heads' LUTs (0 = shared)
     uint32_t mask_stride;           // words between heads' masks (0 = shared)
@@ -142,15 +143,26 @@ __device__ __forceinline__ void for_each_out_vec(F&& f) {
 
 // Normalise and store: the sum relative to the true maximum is total / f with
 // f = 2^((m_true - m_used) c), hence O = acc / (total + 1e-6 f)  (ewops.h:93 divides by sum + 1e-6).
+// Address of the output row of one query: o_row points at element 0 of the row in either element type.
+__device__ __forceinline__ float* output_row(const FusedParams& p, size_t element_offset) {
+    return (float*)((uint8_t*)p.o + element_offset * (p.o_bf16 ? 2u : 4u));
+}
+
 template <int NO>
-__device__ __forceinline__ void store_output(float* o_row, f32x16 (&o)[NO], float m_used, float m_true,
-                                             float total, float c, uint32_t half) {
+__device__ __forceinline__ void store_output(float* o_row, uint32_t as_bf16, f32x16 (&o)[NO], float m_used,
+                                             float m_true, float total, float c, uint32_t half) {
     const float f = exp2_fast((m_true - m_used) * c);
     const float inv = 1.0f / (total + 1e-6f * f);
     for_each_out_vec<NO>([&](int mt, int ig) {
         const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
                            o[mt][ig * 4 + 3] * inv};
-        *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
+        const uint32_t col = mt * 32 + ig * 8 + half * 4;
+        if (as_bf16) {
+            const u32x2 packed = {pack_bf16(out.x, out.y), pack_bf16(out.z, out.w)};
+            *(u32x2*)((uint8_t*)o_row + col * 2) = packed;
+        } else {
+            *(f32x4*)(o_row + col) = out;
+        }
     });
 }
 
@@ -173,8 +185,8 @@ __device__ __forceinline__ uint32_t partial_offset(int mt, int ig, uint32_t half
 }
 
 template <int BS, int D>
-__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, float c,
-                                               uint32_t q_in_block, uint32_t half);
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
+                                               uint32_t as_bf16, float c, uint32_t q_in_block, uint32_t half);
 
 // End of a work item.  Unsplit rows are normalised and stored.  A chunk of a split row writes its
 // partial (unnormalised O, reference maximum, true maximum, sum) and bumps the row's counter; the
@@ -188,7 +200,7 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     constexpr int PART = BS * D + 4 * BS;   // floats per partial
     const float total = st.l + __shfl_xor(st.l, 32);
     if (w.nchunks <= 1) {
-        store_output<NO>(o_row, o, st.m_used, st.m_true, total, c, half);
+        store_output<NO>(o_row, p.o_bf16, o, st.m_used, st.m_true, total, c, half);
         return;
     }
     float* base = p.partials + ((size_t)w.bh * p.n_parts + w.part) * PART;
@@ -214,14 +226,14 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     }
     __syncthreads();
     if (!last_flag) return;
-    merge_partials<BS, D>(base, w.nchunks, o_row, c, q_in_block, half);
+    merge_partials<BS, D>(base, w.nchunks, o_row, p.o_bf16, c, q_in_block, half);
     if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Merge of the partial records of a split row (run by the chunk that arrived last).
 template <int BS, int D>
-__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, float c,
-                                               uint32_t q_in_block, uint32_t half) {
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
+                                               uint32_t as_bf16, float c, uint32_t q_in_block, uint32_t half) {
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -248,14 +260,16 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchun
             for (int e = 0; e < 4; ++e) acc[mt][ig * 4 + e] += coherent_load(src + e) * wgt;
         });
     }
-    store_output<NO>(o_row, acc, m_used, m_true, sum, c, half);
+    store_output<NO>(o_row, as_bf16, acc, m_used, m_true, sum, c, half);
 }
 
 template <int D>
-__device__ __forceinline__ void store_zero_row(float* o_row, uint32_t half) {
+__device__ __forceinline__ void store_zero_row(float* o_row, uint32_t as_bf16, uint32_t half) {
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int x = 0; x < D / 8; ++x) *(f32x4*)(o_row + half * (D / 2) + x * 4) = zero;
+    // this lane's half of the row: D/2 elements = D/8 (fp32) or D/16 (bf16) 16-byte stores
+    uint8_t* dst = (uint8_t*)o_row + half * (D / 2) * (as_bf16 ? 2 : 4);
+    const int n = as_bf16 ? D / 16 : D / 8;
+    for (int x = 0; x < n; ++x) *(f32x4*)(dst + x * 16) = zero;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -311,10 +325,10 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
     const uint32_t lut_off = __builtin_amdgcn_readfirstlane(w.lut_first);
     const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
-    float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
 
     if (count == 0) {
-        store_zero_row<D>(o_row, half);
+        store_zero_row<D>(o_row, p.o_bf16, half);
         return;
     }
 
@@ -475,10 +489,10 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedPar
 
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
     const uint32_t lut_off = w.lut_first, count = w.count;
-    float* o_row = p.o + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D);
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
 
     if (count == 0) {
-        store_zero_row<D>(o_row, half);
+        store_zero_row<D>(o_row, p.o_bf16, half);
         return;
     }
 
@@ -572,7 +586,7 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
     return launch_status();
 }
 
-static int check_common(const void* q, const void* k, const void* v, const float* o, int in_dtype,
+static int check_common(const void* q, const void* k, const void* v, const void* o, int in_dtype,
                         const sfb_uint2* nn_lut, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                         uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
                         uint32_t lut_dim, uint32_t mask_heads, float scale) {
@@ -591,12 +605,12 @@ static int check_common(const void* q, const void* k, const void* v, const float
     return SFB_OK;
 }
 
-static void fill_common(FusedParams& p, const void* q, const void* k, const void* v, float* o,
+static void fill_common(FusedParams& p, const void* q, const void* k, const void* v, void* o, int out_dtype,
                         const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                         uint32_t head_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
                         float scale) {
-    p.q = q; p.k = k; p.v = v; p.o = o;
+    p.q = q; p.k = k; p.v = v; p.o = (float*)o; p.o_bf16 = out_dtype == SFB_BF16 ? 1u : 0u;
     p.nn_lut = nn_lut; p.mask = mask; p.valid_len = valid_len;
     p.row_order = nullptr; p.items = nullptr; p.counters = nullptr; p.partials = nullptr;
     p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
@@ -622,7 +636,7 @@ extern "C" int sfb_fused_attention(sfb_stream_t stream, const void* q, const voi
                                 head_dim, state_dim, lut_heads, lut_dim, mask_heads, scale);
     if (rc != SFB_OK) return rc;
     FusedParams p;
-    fill_common(p, q, k, v, o, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
+    fill_common(p, q, k, v, o, SFB_F32, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
                 lut_heads, lut_dim, mask_heads, scale);
     p.row_order = row_order;
     hipStream_t s = (hipStream_t)stream;
@@ -639,8 +653,8 @@ extern "C" size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_part
     return counters + bh * n_parts * part;
 }
 
-extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k,
-                                             const void* v, float* o, int in_dtype,
+static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k,
+                                             const void* v, void* o, int in_dtype, int out_dtype,
                                              const sfb_uint2* nn_lut, const void* mask,
                                              const int32_t* valid_len, const sfb_work_item* items,
                                              uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
@@ -652,6 +666,7 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
     const int rc = check_common(q, k, v, o, in_dtype, nn_lut, block_size, blocks, batch_dim, ctx_blks,
                                 head_dim, state_dim, 1, ctx_blks + blocks, mask_heads, scale);
     if (rc != SFB_OK) return rc;
+    if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (!items) return SFB_ERR_NULL_POINTER;
     if (n_items == 0 || n_heavy >= n_items) return SFB_ERR_SHAPE;
     if ((uint64_t)batch_dim * head_dim * n_items > 0x7fffffffull / 64) return SFB_ERR_SHAPE;
@@ -659,7 +674,7 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
     if (n_parts > 0 && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
         return SFB_ERR_WORKSPACE;
     FusedParams p;
-    fill_common(p, q, k, v, o, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
+    fill_common(p, q, k, v, o, out_dtype, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
                 1, ctx_blks + blocks, mask_heads, scale);
     p.items = items;
     p.n_slots = n_slots; p.n_parts = n_parts; p.heavy = n_heavy;
@@ -670,4 +685,32 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
     hipStream_t s = (hipStream_t)stream;
     if (block_size == 64) return launch_fused<64, 64>(s, p, in_dtype, n_items);
     return launch_fused<32, 64>(s, p, in_dtype, n_items);
+}
+
+extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k,
+                                             const void* v, float* o, int in_dtype,
+                                             const sfb_uint2* nn_lut, const void* mask,
+                                             const int32_t* valid_len, const sfb_work_item* items,
+                                             uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                             uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                             uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                             uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                             uint32_t mask_heads, float scale) {
+    return fused_attention_scheduled(stream, q, k, v, o, in_dtype, SFB_F32, nn_lut, mask, valid_len, items, n_items,
+                                     n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
+}
+
+extern "C" int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const void* k,
+                                                const void* v, void* o, int in_dtype, int out_dtype,
+                                                const sfb_uint2* nn_lut, const void* mask,
+                                                const int32_t* valid_len, const sfb_work_item* items,
+                                                uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                                uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                                uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                                uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                                uint32_t mask_heads, float scale) {
+    return fused_attention_scheduled(stream, q, k, v, o, in_dtype, out_dtype, nn_lut, mask, valid_len, items, n_items,
+                                     n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
 }

@@ -194,6 +194,29 @@ def test_rows_longer_than_64_key_blocks(bf16, scheduled):
     check(got, orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS), TOL_BF16 if bf16 else TOL_F32)
 
 
+@pytest.mark.parametrize("bf16_in", [False, True])
+@pytest.mark.parametrize("bs,max_blocks", [(64, 4), (32, 100)])
+def test_bf16_output_is_the_fp32_output_rounded_once(bs, max_blocks, bf16_in):
+    """sfb_fused_attention_scheduled_to with bf16 output (split rows merged and rows kept whole, zero rows too)."""
+    nb, B, H, d = 16, 2, 3, 64
+    lay = PATTERNS["bigbird"](nb).copy()
+    lay[5] = 0
+    luts = sfb.build_luts(lay)
+    Q, K, V = qkv(B, nb * bs, H, d, seed=77, bf16=bf16_in)
+    q, k, v = (dev(x, bf16_in) for x in (Q, K, V))
+    sched = sfb.build_schedule(luts["nn_lut"], nb, max_blocks)
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    args = (q, k, v, sfb.to_device(luts["nn_lut"]), sfb.to_device(sched["items"]), sched, ws, bs, luts["blocks"], 0.125)
+    o32 = sfb.fused_attention_scheduled(*args)
+    o16 = torch.full((B, nb * bs, H, d), 7.0, device="cuda", dtype=torch.bfloat16)
+    sfb.fused_attention_scheduled(*args, out=o16)
+    torch.cuda.synchronize()
+    assert torch.equal(o16, o32.to(torch.bfloat16))
+    assert (o16[:, 5 * bs:6 * bs] == 0).all()
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125)
+    assert rel_err(o16.float().cpu().numpy(), want) <= TOL_BF16
+
+
 def test_scheduled_launch_in_a_hip_graph():
     """The scheduled launch (split rows, counters reset by the kernel itself, no memset) captured into a graph:
     every replay, with eager launches and synchronisations in between, gives the eager result bit for bit."""

@@ -85,6 +85,30 @@ def test_gemm_matches_oracle(bf16):
     assert rel_err(got, want64) <= 1e-5
 
 
+@pytest.mark.parametrize("bf16,out_bf16", [(False, False), (True, True), (True, False)])
+def test_gemm_bias_one_kernel(bf16, out_bf16):
+    """GEMM with bias (and rounding to bf16) in the epilogue equals sgemm -> bias (-> one rounding) of the oracle."""
+    m, k, n = 520, 768, 768
+    A = orc.fill_normal((m, k), 19)
+    W = orc.fill_normal((k, n), 20, 0.02)
+    b = orc.fill_normal((n,), 21)
+    if bf16:
+        A, W = orc.round_bf16(A), orc.round_bf16(W)
+    want = orc.bias(orc.sgemm(A, W, nthreads=16), b)
+    a, w = T(A), T(W)
+    if bf16:
+        a, w = a.to(torch.bfloat16), w.to(torch.bfloat16)
+    got = sfb.gemm_bias(a, w, T(b), out_dtype=sfb.BF16 if out_bf16 else sfb.F32)
+    assert got.dtype == (torch.bfloat16 if out_bf16 else torch.float32)
+    got = got.float().cpu().numpy()
+    if out_bf16:
+        # one rounding of the fp32 result: at most one bf16 step away from the rounded oracle value
+        assert np.abs(got - orc.round_bf16(want)).max() <= 2.0 ** -8 * np.abs(want).max()
+        assert np.array_equal(got, orc.round_bf16(got))
+    else:
+        assert rel_err(got, want) <= 1e-5
+
+
 def layer_weights(n, ffn, seed):
     shapes = [("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)), ("w2", (ffn, n)),
               ("bq", (n,)), ("bk", (n,)), ("bv", (n,)), ("bo", (n,)), ("b1", (ffn,)), ("b2", (n,)),
