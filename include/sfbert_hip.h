@@ -96,7 +96,7 @@ void sfb_magicu64(uint32_t d, uint32_t* magic, uint32_t* shift);
 int sfb_element_mask(uint8_t* keep, const sfb_uint2* nt_lut, uint32_t blocks, int bs, int kind,
                      int local_attn_ctx);
 /* no_fusion_test.cu:145-157: block-major words[blk*bs + row], bit j = keep key column j.
- * Word type follows blocksparse.h:684-720: uint32 for bs 32, uint64 for bs 64. */
+ * Word type follows blocksparse.h:684-720: uint8 / uint16 / uint32 / uint64 for bs 8 / 16 / 32 / 64. */
 int sfb_pack_mask(void* words, const uint8_t* keep, uint32_t blocks, int bs);
 /* no_fusion_test.cu:159-163: row-major words[row*blocks + blk] for the unfused softmax. */
 int sfb_transpose_mask(void* row_major, const void* block_major, uint32_t blocks, int bs);
@@ -188,8 +188,9 @@ int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const v
                uint32_t lut_heads, uint32_t lut_dim);
 
 /* BlocksparseMaskedSoftmax<T,V> (blocksparse.h:649-722): y = softmax over each sparse row of x.
- * lut = NN LUT, lut_dim = ctx_blks + blocks; mask [dev] ROW-major words[row*blocks + blk] (uint32 for
- * bs 32, uint64 for bs 64) or NULL; valid_len [dev] int32[batch] or NULL (MI355X addition); scale is
+ * block_size 8, 16, 32 or 64 (blocksparse.h:684-720; the matrix products take 32 and 64 only).
+ * lut = NN LUT, lut_dim = ctx_blks + blocks; mask [dev] ROW-major words[row*blocks + blk] (uint8 / uint16 /
+ * uint32 / uint64 for bs 8 / 16 / 32 / 64) or NULL; valid_len [dev] int32[batch] or NULL (MI355X addition); scale is
  * the raw 1/sqrt(d) -- log2(e) is folded inside, as blocksparse.h:669 does.  max_lut is accepted for
  * signature compatibility.  Numerics follow the CPU softmax (ewops.h:64-98), not the reference GPU
  * kernel's approximations. */
@@ -201,7 +202,7 @@ int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, const void* ma
 
 /* BlocksparseMaskedSoftmaxGrad<T,V> (blocksparse.h:1164-1228): dx = (dy - sum_k dy*y) * y * scale over each
  * sparse row (ewops.h:101-124; masked keys hold y = 0).  dy, y, dx [dev] in the sparse layout, all of
- * `dtype`; lut = NN LUT; max_lut is accepted for signature compatibility. */
+ * `dtype`; block_size 8, 16, 32 or 64; lut = NN LUT; max_lut is accepted for signature compatibility. */
 int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut, const void* dy, const void* y, void* dx,
                             int dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                             uint32_t head_dim, uint32_t ctx_blks, uint32_t lut_heads, uint32_t lut_dim,

@@ -347,7 +347,9 @@ void orc_pack_mask(void* words, const uint8_t* keep, uint32_t blocks, int bs, in
             w |= k << j;
         }
         if (word_bytes == 8) ((uint64_t*)words)[i] = w;
-        else ((uint32_t*)words)[i] = (uint32_t)w;
+        else if (word_bytes == 4) ((uint32_t*)words)[i] = (uint32_t)w;
+        else if (word_bytes == 2) ((uint16_t*)words)[i] = (uint16_t)w;   /* block 16: blocksparse.h:705 */
+        else ((uint8_t*)words)[i] = (uint8_t)w;                          /* block 8: blocksparse.h:714 */
     }
 }
 
@@ -357,8 +359,8 @@ void orc_transpose_mask(void* row_major, const void* block_major, uint32_t block
     for (uint32_t i = 0; i < blocks; i++) {
         for (int j = 0; j < bs; j++) {
             size_t src = (size_t)i * bs + j, dst = (size_t)j * blocks + i;
-            if (word_bytes == 8) ((uint64_t*)row_major)[dst] = ((const uint64_t*)block_major)[src];
-            else ((uint32_t*)row_major)[dst] = ((const uint32_t*)block_major)[src];
+            memcpy((char*)row_major + dst * (size_t)word_bytes, (const char*)block_major + src * (size_t)word_bytes,
+                   (size_t)word_bytes);
         }
     }
 }
@@ -366,7 +368,9 @@ void orc_transpose_mask(void* row_major, const void* block_major, uint32_t block
 static inline int mask_bit(const void* words, int word_bytes, size_t word_index, int bit) {
     if (!words) return 1;
     if (word_bytes == 8) return (int)((((const uint64_t*)words)[word_index] >> bit) & 1ull);
-    return (int)((((const uint32_t*)words)[word_index] >> bit) & 1u);
+    if (word_bytes == 4) return (int)((((const uint32_t*)words)[word_index] >> bit) & 1u);
+    if (word_bytes == 2) return (int)((((const uint16_t*)words)[word_index] >> bit) & 1u);
+    return (int)((((const uint8_t*)words)[word_index] >> bit) & 1u);
 }
 
 /* ------------------------------------------------------------------------------------------ */

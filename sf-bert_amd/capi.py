@@ -170,7 +170,7 @@ def element_mask(nt_lut, bs, kind, local_attn_ctx=0):
 
 def pack_mask(keep):
     blocks, bs, _ = keep.shape
-    words = np.zeros(blocks * bs, np.uint64 if bs == 64 else np.uint32)
+    words = np.zeros(blocks * bs, {8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}.get(bs, np.uint32))
     _check(lib.sfb_pack_mask(_np(words), _np(np.ascontiguousarray(keep, np.uint8)), blocks, bs),
            "sfb_pack_mask")
     return words

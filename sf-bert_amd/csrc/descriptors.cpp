@@ -40,7 +40,8 @@ struct SplitMix64 {
     }
 };
 
-inline int word_bytes_for(int bs) { return bs == 64 ? 8 : bs == 32 ? 4 : 0; }
+// one mask word per (block, row): uchar / ushort / uint / uint64 for block 8 / 16 / 32 / 64 (blocksparse.h:684-720)
+inline int word_bytes_for(int bs) { return bs == 64 ? 8 : bs == 32 ? 4 : bs == 16 ? 2 : bs == 8 ? 1 : 0; }
 
 }  // namespace
 
@@ -281,7 +282,9 @@ int sfb_pack_mask(void* words, const uint8_t* keep, uint32_t blocks, int bs) {
         const uint8_t* src = keep + row * bs;
         for (int j = 0; j < bs; ++j) w |= (uint64_t)(src[j] != 0) << j;
         if (wb == 8) static_cast<uint64_t*>(words)[row] = w;
-        else static_cast<uint32_t*>(words)[row] = (uint32_t)w;
+        else if (wb == 4) static_cast<uint32_t*>(words)[row] = (uint32_t)w;
+        else if (wb == 2) static_cast<uint16_t*>(words)[row] = (uint16_t)w;
+        else static_cast<uint8_t*>(words)[row] = (uint8_t)w;
     }
     return SFB_OK;
 }

@@ -230,7 +230,11 @@ struct SoftmaxRows {
         uint32_t k = left >= 8 ? 0xffu : (left <= 0 ? 0u : ((1u << left) - 1u));
         if (mask) {
             const size_t w = (size_t)qi * blocks + e.x;
-            const uint64_t word = (BS == 64) ? ((const uint64_t*)mask)[w] : ((const uint32_t*)mask)[w];
+            uint64_t word;
+            if (BS == 64) word = ((const uint64_t*)mask)[w];
+            else if (BS == 32) word = ((const uint32_t*)mask)[w];
+            else if (BS == 16) word = ((const uint16_t*)mask)[w];
+            else word = mask[w];
             k &= (uint32_t)(word >> key0);
         }
         return k;
@@ -1001,7 +1005,7 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     (void)max_lut;  // sizes the reference's shared memory (blocksparse.h:671-686); not needed here
     if (!lut || !x || !y) return SFB_ERR_NULL_POINTER;
     if (check_dtype(x_dtype) || check_dtype(y_dtype)) return SFB_ERR_DTYPE;
-    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (block_size != 8 && block_size != 16 && block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads || !mask_heads) return SFB_ERR_SHAPE;
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
@@ -1016,7 +1020,9 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     clear_stale_error();
 #define SFB_CALL(BSV, TX, TY) masked_softmax_kernel<BSV, TX, TY><<<grid, dim3(256), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, x_dtype, y_dtype, SFB_CALL);
-    else SFB_DISPATCH_2(32, x_dtype, y_dtype, SFB_CALL);
+    else if (block_size == 32) SFB_DISPATCH_2(32, x_dtype, y_dtype, SFB_CALL);
+    else if (block_size == 16) SFB_DISPATCH_2(16, x_dtype, y_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(8, x_dtype, y_dtype, SFB_CALL);
 #undef SFB_CALL
     return launch_status();
 }
@@ -1061,7 +1067,7 @@ extern "C" int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut
     (void)max_lut;  // sizes the reference's shared memory (blocksparse.h:671-686); not needed here
     if (!lut || !dy || !y || !dx) return SFB_ERR_NULL_POINTER;
     if (check_dtype(dtype)) return SFB_ERR_DTYPE;
-    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (block_size != 8 && block_size != 16 && block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads) return SFB_ERR_SHAPE;
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
@@ -1072,13 +1078,16 @@ extern "C" int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut
     const dim3 grid((uint32_t)groups);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
-    if (block_size == 64) {
-        if (dtype == SFB_F32) masked_softmax_grad_kernel<64, float><<<grid, dim3(256), 0, s>>>(p);
-        else masked_softmax_grad_kernel<64, __bf16><<<grid, dim3(256), 0, s>>>(p);
-    } else {
-        if (dtype == SFB_F32) masked_softmax_grad_kernel<32, float><<<grid, dim3(256), 0, s>>>(p);
-        else masked_softmax_grad_kernel<32, __bf16><<<grid, dim3(256), 0, s>>>(p);
-    }
+#define SFB_CALL(BSV)                                                                            \
+    do {                                                                                         \
+        if (dtype == SFB_F32) masked_softmax_grad_kernel<BSV, float><<<grid, dim3(256), 0, s>>>(p); \
+        else masked_softmax_grad_kernel<BSV, __bf16><<<grid, dim3(256), 0, s>>>(p);               \
+    } while (0)
+    if (block_size == 64) SFB_CALL(64);
+    else if (block_size == 32) SFB_CALL(32);
+    else if (block_size == 16) SFB_CALL(16);
+    else SFB_CALL(8);
+#undef SFB_CALL
     return launch_status();
 }
 

@@ -115,8 +115,8 @@ def element_mask(nt_lut, bs, kind, local_attn_ctx=0):
 
 def pack_mask(keep):
     blocks, bs, _ = keep.shape
-    wb = 8 if bs == 64 else 4
-    words = np.zeros(blocks * bs, np.uint64 if wb == 8 else np.uint32)
+    wb = max(bs // 8, 1)
+    words = np.zeros(blocks * bs, {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[wb])
     lib.orc_pack_mask(_p(words), _p(np.ascontiguousarray(keep)), blocks, bs, wb)
     return words
 

@@ -39,6 +39,33 @@ def test_softmax_grad(pattern, bs, bf16):
     assert (got[P == 0] == 0).all()   # masked keys carry no gradient
 
 
+@pytest.mark.parametrize("bs", [8, 16])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_softmax_and_its_gradient_at_small_block_sizes(bs, bf16):
+    """Block sizes 8 and 16 exist for the softmax stages only (blocksparse.h:703-720, 1199-1224): uint8 / uint16
+    mask words, 64 / 32 key blocks per wave step; nb 80 gives rows of one and of several steps."""
+    nb, B, H = 80, 2, 2
+    luts = sfb.build_luts(sfb.layout_full(nb, causal=True))
+    blocks = luts["blocks"]
+    S = rounded(orc.fill_normal((B, H, blocks, bs, bs), 40), bf16)
+    mask = sfb.pack_mask(sfb.element_mask(luts["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG))
+    assert mask.dtype.itemsize == bs // 8
+    valid = np.array([nb * bs, nb * bs - bs - 3], np.int32)
+    want = orc.masked_softmax(S, luts["nn_lut"], nb, 0.125, mask=mask, valid_len=valid)
+    nn = sfb.to_device(luts["nn_lut"])
+    P = sfb.BlocksparseMaskedSoftmax(nn, sfb.to_device(sfb.transpose_mask(mask, blocks, bs)), sparse_dev(S, bf16), nb,
+                                     0.125, valid_len=sfb.to_device(valid))
+    tol = TOL_BF16 if bf16 else TOL_F32
+    got = P.float().cpu().numpy()
+    assert rel_err(got, want) <= tol and (got[want == 0] == 0).all()
+    plain = sfb.BlocksparseMaskedSoftmax(nn, None, sparse_dev(S, bf16), nb, 0.125).float().cpu().numpy()
+    assert rel_err(plain, orc.masked_softmax(S, luts["nn_lut"], nb, 0.125)) <= tol
+    Pw = rounded(want, bf16)
+    dP = rounded(orc.fill_normal((B, H, blocks, bs, bs), 41), bf16)
+    dS = sfb.BlocksparseMaskedSoftmaxGrad(nn, sparse_dev(dP, bf16), sparse_dev(Pw, bf16), nb, 0.125)
+    assert rel_err(dS.float().cpu().numpy(), orc.masked_softmax_grad(dP, Pw, luts["nn_lut"], nb, 0.125)) <= tol
+
+
 @pytest.mark.parametrize("bs,nb", [(64, 70), (32, 132)])
 def test_softmax_grad_rows_longer_than_the_register_cache(bs, nb):
     luts = sfb.build_luts(sfb.layout_full(nb, causal=False))

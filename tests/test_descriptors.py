@@ -85,14 +85,14 @@ def test_luts_bit_exact(layout):
                for a, b in zip(order[:-1], order[1:]))
 
 
-@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("bs", [8, 16, 32, 64])
 @pytest.mark.parametrize("kind", [0, 1, 2, 3])
 def test_masks_bit_exact(bs, kind):
     luts = orc.build_luts(orc.layout_local(6, 2))
     keep = sfb.element_mask(luts["nt_lut"], bs, kind, local_attn_ctx=bs + 5)
     assert np.array_equal(keep, orc.element_mask(luts["nt_lut"], bs, kind, local_attn_ctx=bs + 5))
     words = sfb.pack_mask(keep)
-    assert words.dtype == (np.uint64 if bs == 64 else np.uint32)
+    assert words.dtype.itemsize == bs // 8
     assert np.array_equal(words, orc.pack_mask(keep))
     blocks = keep.shape[0]
     assert np.array_equal(sfb.transpose_mask(words, blocks, bs), orc.transpose_mask(words, blocks, bs))
@@ -109,7 +109,7 @@ def test_error_codes():
     lay = np.zeros((4, 4), np.uint32)
     assert sfb.lib.sfb_layout_full(None, 4, 1) == 1
     assert sfb.lib.sfb_layout_full(lay.ctypes.data_as(C.c_void_p), 0, 1) == 4
-    assert sfb.lib.sfb_pack_mask(lay.ctypes.data_as(C.c_void_p), lay.ctypes.data_as(C.c_void_p), 1, 16) == 2
+    assert sfb.lib.sfb_pack_mask(lay.ctypes.data_as(C.c_void_p), lay.ctypes.data_as(C.c_void_p), 1, 24) == 2
     with pytest.raises(sfb.capi.SfbError):
         sfb.layout_local(4, -1)
 
