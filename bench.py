@@ -109,6 +109,19 @@ def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
     parts = {"sdd_ms": _time(torch, lambda: sfb.bst_sgemm_nt(nt, q, k, bs, blocks, c=S), 200, 20),
              "softmax_ms": _time(torch, lambda: sfb.BlocksparseMaskedSoftmax(nn, None, S, nb, scale, y=P), 200, 20),
              "dsd_ms": _time(torch, lambda: sfb.bst_sgemm_xn(nn, P, v, nb, c=O), 200, 20)}
+    # sdd + softmax in one kernel (P still goes through HBM): one work-group per block-row against the
+    # reference's own decomposition, one work-group per block with flag / spin exchange
+    order = sfb.to_device(luts["row_order"])
+    parts["sdd_softmax_row_owner_ms"] = _time(
+        torch, lambda: sfb.fusion_attention2(nn, q, k, bs, blocks, scale, y=P, row_order=order), 200, 20)
+    nbytes = int(sfb.lib.sfb_split_softmax_scratch_bytes(bs, blocks, B, H, nb))
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    status = []
+
+    def split():
+        status[:] = [sfb.fusion_attention2_split(nt, nn, q, k, bs, blocks, scale, y=P, scratch=scratch)[1]]
+    parts["sdd_softmax_per_block_with_flags_ms"] = _time(torch, split, 100, 10)
+    parts["sdd_softmax_per_block_status"] = int(status[0])
     return dict(ms_per_call=ms, fused_speedup=ms / fused_ms, sp_storage="bf16" if bf16 else "f32", **parts)
 
 

@@ -224,12 +224,32 @@ int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const v
 /* fusion_attention1 / fusion_attention2 (fusion_blocksparse.h:400-455, 1212-1268): sdd + masked
  * softmax in one kernel, y = P in the sparse layout (fp32 or bf16).  One work-group owns a whole
  * block-row, so the reference's rblk_flag / rblk_flag1 / Max / Sum scratch and its spin-waits are not
- * needed.  mask is BLOCK-major here (fusion_blocksparse.h:690). */
+ * needed.  mask is BLOCK-major here (fusion_blocksparse.h:690).  row_order [dev] uint32[ctx_blks] (from
+ * sfb_build_row_order: block-rows by falling block count) or NULL: the order in which block-rows are handed to
+ * work-groups; with it the longest rows start first instead of forming the tail of the launch. */
 int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const void* a, const void* b,
                           void* y, int in_dtype, int y_dtype, const void* mask,
-                          const int32_t* valid_len, uint32_t block_size, uint32_t blocks,
-                          uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
-                          uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale);
+                          const int32_t* valid_len, const uint32_t* row_order, uint32_t block_size,
+                          uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                          uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
+                          float scale);
+
+/* Comparison variant of sfb_fused_sdd_softmax with the reference's own decomposition (fusion_nt_softmax2 /
+ * fusion_attention2, fusion_blocksparse.h:458-833, 1212-1268): one work-group per block; the blocks of a
+ * block-row exchange row maxima and row sums through global scratch and wait for each other on two flags per
+ * block-row.  Same results as sfb_fused_sdd_softmax.  nt_lut, nn_lut [dev]; mask BLOCK-major; scratch [dev]
+ * 256-byte aligned, sfb_split_softmax_scratch_bytes() bytes (Max, Sum, the flags, one status word; cleared by
+ * the call).  The waits are bounded by spin_limit polls: a work-group whose wait runs out leaves its block
+ * unwritten and sets the status word (the last 256 bytes of scratch, uint32: 0 = every block written), because
+ * the scheme cannot finish unless all work-groups of a block-row get to run at the same time. */
+size_t sfb_split_softmax_scratch_bytes(uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t head_dim,
+                                       uint32_t ctx_blks);
+int sfb_fused_sdd_softmax_split(sfb_stream_t stream, const sfb_uint2* nt_lut, const sfb_uint2* nn_lut,
+                                const void* a, const void* b, void* y, int in_dtype, int y_dtype, const void* mask,
+                                const int32_t* valid_len, void* scratch, size_t scratch_bytes, uint32_t spin_limit,
+                                uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads, uint32_t mask_heads,
+                                float scale);
 
 /* ---- encoder-layer ops (one pass over HBM each) ------------------------------------------------ */
 

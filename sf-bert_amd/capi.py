@@ -48,6 +48,7 @@ lib.sfb_magicu64.restype = None
 lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
 lib.sfb_model_workspace_bytes.restype = C.c_size_t
+lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -59,6 +60,7 @@ EXPORTED = [
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
+    "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_gemm_bias", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
@@ -357,8 +359,9 @@ def bst_sgemm_xn(lut, a, b, ctx_blks_c, op=NN_OP, lut_heads=1, magic=1, shift=0,
 
 
 def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_len=None, out_dtype=None,
-                      lut_heads=1, mask_heads=1, y=None):
-    """sdd + masked softmax in one kernel -> P (fusion_blocksparse.h:1212); mask is BLOCK-major."""
+                      lut_heads=1, mask_heads=1, y=None, row_order=None):
+    """sdd + masked softmax in one kernel -> P (fusion_blocksparse.h:1212); mask is BLOCK-major; row_order:
+    device buffer of build_luts()["row_order"] (longest block-rows first) or None."""
     import torch
     B, L, H, d = a.shape
     if y is None:
@@ -366,7 +369,7 @@ def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_
                         dtype=_torch_dtype(F32 if out_dtype is None else out_dtype))
     nb = L // block_size
     _check(lib.sfb_fused_sdd_softmax(_stream(), _dev(nn_lut), _dev(a), _dev(b), _dev(y), _dtype_code(a),
-                                     _dtype_code(y), _dev(mask), _dev(valid_len), C.c_uint32(block_size),
+                                     _dtype_code(y), _dev(mask), _dev(valid_len), _dev(row_order), C.c_uint32(block_size),
                                      C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H),
                                      C.c_uint32(d), C.c_uint32(lut_heads), C.c_uint32(nb + blocks),
                                      C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_sdd_softmax")
@@ -374,6 +377,30 @@ def fusion_attention2(nn_lut, a, b, block_size, blocks, scale, mask=None, valid_
 
 
 fusion_attention1 = fusion_attention2
+
+
+def fusion_attention2_split(nt_lut, nn_lut, a, b, block_size, blocks, scale, mask=None, valid_len=None,
+                            out_dtype=None, lut_heads=1, mask_heads=1, y=None, scratch=None, spin_limit=1 << 16):
+    """sdd + masked softmax -> P by one work-group per block with flag / spin exchange between the blocks of a
+    block-row (the reference's fusion_nt_softmax2 decomposition; comparison variant).  Returns (P, status) where
+    status is a device uint32 tensor: 0 = every block written."""
+    import torch
+    B, L, H, d = a.shape
+    nb = L // block_size
+    if y is None:
+        y = torch.empty((B, H, blocks, block_size, block_size), device=a.device,
+                        dtype=_torch_dtype(F32 if out_dtype is None else out_dtype))
+    nbytes = int(lib.sfb_split_softmax_scratch_bytes(C.c_uint32(block_size), C.c_uint32(blocks), C.c_uint32(B),
+                                                     C.c_uint32(H), C.c_uint32(nb)))
+    if scratch is None:
+        scratch = torch.empty(nbytes, dtype=torch.uint8, device=a.device)
+    _check(lib.sfb_fused_sdd_softmax_split(_stream(), _dev(nt_lut), _dev(nn_lut), _dev(a), _dev(b), _dev(y),
+                                           _dtype_code(a), _dtype_code(y), _dev(mask), _dev(valid_len), _dev(scratch),
+                                           C.c_size_t(scratch.numel()), C.c_uint32(spin_limit), C.c_uint32(block_size),
+                                           C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H),
+                                           C.c_uint32(d), C.c_uint32(lut_heads), C.c_uint32(mask_heads),
+                                           C.c_float(scale)), "sfb_fused_sdd_softmax_split")
+    return y, scratch[nbytes - 256:nbytes - 252].view(torch.int32)
 
 
 def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None):

@@ -7,9 +7,16 @@
 // (sfb_fused_sdd_softmax), done by one work-group per block-row without any inter-group exchange.
 //
 // Arithmetic follows the CPU path of the reference (matmul.h:53-78, ewops.h:64-98, matmul.h:6-20).
+#include <type_traits>
+
 #include "tiles.hip.h"
 
 namespace sfb {
+
+// relaxed device-scope load: reads what another work-group of the same launch published
+__device__ __forceinline__ float coherent_load_f32(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <typename T> struct Elem;
 template <> struct Elem<float> {
@@ -70,6 +77,54 @@ __device__ __forceinline__ void score_tile_direct(f32x16 (&s)[BS / 32], const TI
             }
         }
     }
+}
+
+// The same product with the operands fetched ahead of their use: a lane's share of one K tile (KTile) and of its
+// query row (QRow) in MFMA operand layout, so that the next tile can be in flight while this one is multiplied.
+template <int BS, int D, typename TIn>
+struct KTile {
+    static constexpr int KT = BS / 32, STEPS = sizeof(TIn) == 2 ? D / 16 : D / 8;
+    typedef typename std::conditional<sizeof(TIn) == 2, bf16x8, f32x4>::type Vec;
+    Vec v[KT][STEPS];
+    __device__ __forceinline__ void load(const TIn* k_blk, uint32_t row_stride, uint32_t qn, uint32_t half) {
+        constexpr int W = sizeof(TIn) == 2 ? 8 : 4;   // elements per vector
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int st = 0; st < STEPS; ++st)
+                v[kt][st] = *(const Vec*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + (2 * st + half) * W);
+    }
+};
+template <int D, typename TIn>
+struct QRow {
+    static constexpr int STEPS = sizeof(TIn) == 2 ? D / 16 : D / 8;
+    typedef typename std::conditional<sizeof(TIn) == 2, bf16x8, f32x4>::type Vec;
+    Vec v[STEPS];
+    __device__ __forceinline__ void load(const TIn* q_row, uint32_t half) {
+        constexpr int W = sizeof(TIn) == 2 ? 8 : 4;
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) v[st] = *(const Vec*)(q_row + (2 * st + half) * W);
+    }
+};
+template <int BS, int D, typename TIn>
+__device__ __forceinline__ void score_tile(f32x16 (&s)[BS / 32], const KTile<BS, D, TIn>& k, const QRow<D, TIn>& q) {
+    constexpr int KT = BS / 32;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+    for (int st = 0; st < QRow<D, TIn>::STEPS; ++st)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            if constexpr (sizeof(TIn) == 2) {
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k.v[kt][st], q.v[st], s[kt], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(k.v[kt][st][e], q.v[st][e], s[kt], 0, 0, 0);
+            }
+        }
 }
 
 // Store this lane's part of a BS x BS block (row = its query): groups of 4 consecutive keys.
@@ -900,19 +955,28 @@ struct SddSoftmaxParams {
     void* y;
     const void* mask;        // block-major words
     const int32_t* valid_len;
+    const uint32_t* row_order;   // rank -> block-row, or nullptr
     uint32_t blocks, batch, heads, nb, lut_stride, mask_stride, groups;
     float scale_log2e;
 };
 
+// Waves of a work-group: BS/32 query halves x kSddSoftmaxKeyGroups key groups.  Key group g takes the row's blocks
+// g, g + 2, ...; the groups meet once, through LDS, to agree on the row maximum and sum.  A long block-row thus
+// has two independent streams of tile loads in flight per query half instead of one (four measured the same on
+// rows of 64 blocks and slower on rows of 11, where the larger work-group leaves fewer of them per CU).
+constexpr int kSddSoftmaxKeyGroups = 2;
+
 template <int BS, int D, typename TIn, typename TOut>
-__global__ __launch_bounds__(BS * 2, 2) void sdd_softmax_kernel(SddSoftmaxParams p) {
-    constexpr int KT = BS / 32;
+__global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_kernel(SddSoftmaxParams p) {
+    constexpr int KT = BS / 32, QW = BS / 32, KG = kSddSoftmaxKeyGroups;
+    __shared__ float stats[KG][BS][2];
     const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
-    const uint32_t r = p.nb - 1 - work.rank;
+    const uint32_t r = p.row_order ? p.row_order[work.rank] : p.nb - 1 - work.rank;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
-    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t group = wave / QW;
+    const uint32_t q_in_block = (wave % QW) * 32 + qn;
     const uint32_t L = p.nb * BS, row_stride = p.heads * D;
     const sfb_uint2* lut = p.nn_lut + (size_t)h * p.lut_stride;
     const uint32_t off = lut[r].x, count = lut[r].y;
@@ -923,21 +987,45 @@ __global__ __launch_bounds__(BS * 2, 2) void sdd_softmax_kernel(SddSoftmaxParams
     const float c = p.scale_log2e;
     TOut* Y = (TOut*)p.y + (size_t)work.bh * p.blocks * BS * BS;
 
+    QRow<D, TIn> q_ops;
+    q_ops.load(q_row, half);
     float m = kMaxSeed, l = 0.f;   // exact running maximum and the sum relative to it (this lane's keys)
     for (int pass = 0; pass < 2; ++pass) {
         float inv = 0.f;
         if (pass == 1) {
-            const float total = l + __shfl_xor(l, 32);
+            // this group's statistics (both lanes of a query hold the same maximum; their sums add up), then
+            // the row's: maximum over the groups, sums rescaled to it
+            const float mine = l + __shfl_xor(l, 32);
+            if (half == 0) {
+                stats[group][q_in_block][0] = m;
+                stats[group][q_in_block][1] = mine;
+            }
+            __syncthreads();
+            float m_row = kMaxSeed;
+#pragma unroll
+            for (int g = 0; g < KG; ++g) m_row = fmaxf(m_row, stats[g][q_in_block][0]);
+            float total = 0.f;
+#pragma unroll
+            for (int g = 0; g < KG; ++g)
+                total += stats[g][q_in_block][1] * exp2_fast((stats[g][q_in_block][0] - m_row) * c);
+            m = m_row;
             inv = 1.0f / (total + 1e-6f);
         }
-        for (uint32_t j = 0; j < count; ++j) {
-            const sfb_uint2 e = lut[off + j];
+        // the K tile of this group's next block is fetched while the current one is multiplied
+        KTile<BS, D, TIn> k_cur, k_next;
+        sfb_uint2 e = group < count ? lut[off + group] : sfb_uint2{0u, 0u};
+        if (group < count) k_cur.load(K + token_offset(b, e.y * BS, h, L, p.heads, D), row_stride, qn, half);
+        for (uint32_t j = group; j < count; j += KG) {
+            const sfb_uint2 e_next = lut[off + (j + KG < count ? j + KG : j)];
+            k_next.load(K + token_offset(b, e_next.y * BS, h, L, p.heads, D), row_stride, qn, half);
             f32x16 s[KT];
-            score_tile_direct<BS, D, TIn>(s, q_row, K + token_offset(b, e.y * BS, h, L, p.heads, D), row_stride,
-                                          qn, half);
+            score_tile<BS, D, TIn>(s, k_cur, q_ops);
             const int limit = valid - (int)(e.y * BS);
             const bool masked = (mask != nullptr) || (limit < BS);
             if (masked) apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)e.x * BS + q_in_block, limit), half);
+            const uint32_t blk = e.x;
+            e = e_next;
+            k_cur = k_next;
             if (pass == 0) {
                 const float m_new = fmaxf(m, block_row_max<KT>(s));
                 l *= exp2_fast((m - m_new) * c);
@@ -953,10 +1041,128 @@ __global__ __launch_bounds__(BS * 2, 2) void sdd_softmax_kernel(SddSoftmaxParams
                 for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) s[kt][i] = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc)) * inv;
-                store_block_row<BS, TOut>(Y + ((size_t)e.x * BS + q_in_block) * BS, s, half);
+                store_block_row<BS, TOut>(Y + ((size_t)blk * BS + q_in_block) * BS, s, half);
             }
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// sdd + softmax -> P with ONE WORK-GROUP PER BLOCK, the decomposition of the reference's fusion_nt_softmax2
+// (fusion_blocksparse.h:458-833): every work-group computes its block's scores, publishes the row maxima of
+// the block, counts itself in on the block-row's flag and spins until all blocks of the row have done so;
+// takes the row maximum over the published values, publishes its partial row sums, spins on a second flag, and
+// normalises.  Kept as the comparison for sdd_softmax_kernel above, which needs none of this because one
+// work-group owns the whole block-row.  The spins are bounded: a work-group that runs out of its budget sets
+// *status and leaves without writing its block (the scheme only makes progress while every work-group of a
+// block-row is resident or can become resident, which a launch cannot guarantee).
+// ---------------------------------------------------------------------------------------------
+struct SplitSoftmaxParams {
+    const sfb_uint2* nt_lut;
+    const sfb_uint2* nn_lut;
+    const void* a;
+    const void* b;
+    void* y;
+    const void* mask;         // block-major words
+    const int32_t* valid_len;
+    float* row_max;           // [batch][heads][blocks][BS]
+    float* row_sum;           // [batch][heads][blocks][BS]
+    uint32_t* flags;          // [batch][heads][nb][2], zero at launch
+    uint32_t* status;         // set to 1 by a work-group whose spin budget ran out
+    uint32_t blocks, heads, nb, nt_stride, nn_stride, mask_stride, spin_limit;
+    float scale_log2e;
+};
+
+// Thread 0 waits until *flag reaches `want`; every thread learns whether it did.
+__device__ __forceinline__ bool wait_for_row(uint32_t* flag, uint32_t want, uint32_t spin_limit, uint32_t t) {
+    __shared__ uint32_t arrived;
+    if (t == 0) {
+        uint32_t seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (uint32_t spin = 0; seen < want && spin < spin_limit; ++spin) {
+            __builtin_amdgcn_s_sleep(4);
+            seen = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        arrived = seen >= want ? 1u : 0u;
+    }
+    __syncthreads();
+    const bool ok = arrived != 0;
+    __syncthreads();   // `arrived` is reused by the second wait
+    return ok;
+}
+
+template <int BS, int D, typename TIn, typename TOut>
+__global__ __launch_bounds__(BS * 2) void sdd_softmax_split_kernel(SplitSoftmaxParams p) {
+    constexpr int KT = BS / 32;
+    const uint32_t blk = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t bh = b * p.heads + h;
+    const sfb_uint2 e = p.nt_lut[(size_t)h * p.nt_stride + blk];   // {row block, col block}
+    const sfb_uint2* nn = p.nn_lut + (size_t)h * p.nn_stride;
+    const uint32_t off = nn[e.x].x, count = nn[e.x].y;
+    const uint32_t L = p.nb * BS, row_stride = p.heads * D;
+    const float c = p.scale_log2e;
+
+    f32x16 s[KT];
+    const TIn* q_row = (const TIn*)p.a + token_offset(b, e.x * BS + q_in_block, h, L, p.heads, D);
+    score_tile_direct<BS, D, TIn>(s, q_row, (const TIn*)p.b + token_offset(b, e.y * BS, h, L, p.heads, D), row_stride,
+                                  qn, half);
+    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+    const int limit = valid - (int)(e.y * BS);
+    if (mask != nullptr || limit < BS)
+        apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)blk * BS + q_in_block, limit), half);
+
+    // phase 1: the block's row maxima (seeded as ewops.h:70), then the block-row's first flag
+    const size_t head_rows = (size_t)bh * p.blocks * BS;
+    const float m_blk = fmaxf(kMaxSeed, block_row_max<KT>(s));
+    if (half == 0) __hip_atomic_store(p.row_max + head_rows + (size_t)blk * BS + q_in_block, m_blk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    __syncthreads();
+    uint32_t* flags = p.flags + ((size_t)bh * p.nb + e.x) * 2;
+    if (t == 0) __hip_atomic_fetch_add(flags, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!wait_for_row(flags, count, p.spin_limit, t)) {
+        if (t == 0) __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    float m = kMaxSeed;
+    for (uint32_t j = 0; j < count; ++j)
+        m = fmaxf(m, coherent_load_f32(p.row_max + head_rows + (size_t)nn[off + j].x * BS + q_in_block));
+
+    // phase 2: partial row sums relative to the row maximum, second flag
+    const float mc = m * c;
+    float l = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[kt][i] = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc));
+            l += s[kt][i];
+        }
+    l += __shfl_xor(l, 32);
+    if (half == 0) __hip_atomic_store(p.row_sum + head_rows + (size_t)blk * BS + q_in_block, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    __syncthreads();
+    if (t == 0) __hip_atomic_fetch_add(flags + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!wait_for_row(flags + 1, count, p.spin_limit, t)) {
+        if (t == 0) __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+    }
+    float total = 0.f;
+    for (uint32_t j = 0; j < count; ++j)
+        total += coherent_load_f32(p.row_sum + head_rows + (size_t)nn[off + j].x * BS + q_in_block);
+    const float inv = 1.0f / (total + 1e-6f);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] *= inv;
+    TOut* Y = (TOut*)p.y + (size_t)bh * p.blocks * BS * BS;
+    store_block_row<BS, TOut>(Y + ((size_t)blk * BS + q_in_block) * BS, s, half);
+}
+
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) words[i] = 0u;
 }
 
 static int check_dtype(int d) { return (d == SFB_F32 || d == SFB_BF16) ? SFB_OK : SFB_ERR_DTYPE; }
@@ -1093,8 +1299,8 @@ extern "C" int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut
 
 extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lut, const void* a,
                                      const void* b, void* y, int in_dtype, int y_dtype, const void* mask,
-                                     const int32_t* valid_len, uint32_t block_size, uint32_t blocks,
-                                     uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                     const int32_t* valid_len, const uint32_t* row_order, uint32_t block_size,
+                                     uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
                                      uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim,
                                      uint32_t mask_heads, float scale) {
     if (!nn_lut || !a || !b || !y) return SFB_ERR_NULL_POINTER;
@@ -1106,13 +1312,61 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
-    SddSoftmaxParams p = {nn_lut, a, b, y, mask, valid_len, blocks, batch_dim, head_dim, ctx_blks,
+    SddSoftmaxParams p = {nn_lut, a, b, y, mask, valid_len, row_order, blocks, batch_dim, head_dim, ctx_blks,
                           lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0,
                           bh_groups(batch_dim * head_dim), scale * kLog2e};
     const dim3 grid(p.groups * 8u * ctx_blks);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
-#define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
+#define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+    if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);
+#undef SFB_CALL
+    return launch_status();
+}
+
+extern "C" size_t sfb_split_softmax_scratch_bytes(uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                                  uint32_t head_dim, uint32_t ctx_blks) {
+    const size_t bh = (size_t)batch_dim * head_dim;
+    const size_t stats = (bh * blocks * block_size * sizeof(float) + 255) / 256 * 256;
+    const size_t flags = (bh * ctx_blks * 2 * sizeof(uint32_t) + 255) / 256 * 256;
+    return 2 * stats + flags + 256;
+}
+
+extern "C" int sfb_fused_sdd_softmax_split(sfb_stream_t stream, const sfb_uint2* nt_lut, const sfb_uint2* nn_lut,
+                                           const void* a, const void* b, void* y, int in_dtype, int y_dtype,
+                                           const void* mask, const int32_t* valid_len, void* scratch,
+                                           size_t scratch_bytes, uint32_t spin_limit, uint32_t block_size,
+                                           uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                           uint32_t state_dim, uint32_t lut_heads, uint32_t mask_heads, float scale) {
+    if (!nt_lut || !nn_lut || !a || !b || !y || !scratch) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(in_dtype) || check_dtype(y_dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads || !mask_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && lut_heads != head_dim) return SFB_ERR_SHAPE;
+    if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
+    if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
+    if (scratch_bytes < sfb_split_softmax_scratch_bytes(block_size, blocks, batch_dim, head_dim, ctx_blks) ||
+        ((uintptr_t)scratch & 255u))
+        return SFB_ERR_WORKSPACE;
+    const size_t bh = (size_t)batch_dim * head_dim;
+    const size_t stats = (bh * blocks * block_size * sizeof(float) + 255) / 256 * 256;
+    const size_t flags = (bh * ctx_blks * 2 * sizeof(uint32_t) + 255) / 256 * 256;
+    uint8_t* base = (uint8_t*)scratch;
+    SplitSoftmaxParams p = {nt_lut, nn_lut, a, b, y, mask, valid_len, (float*)base, (float*)(base + stats),
+                            (uint32_t*)(base + 2 * stats), (uint32_t*)(base + 2 * stats + flags), blocks, head_dim,
+                            ctx_blks, lut_heads > 1 ? blocks : 0, lut_heads > 1 ? ctx_blks + blocks : 0,
+                            mask_heads > 1 ? blocks * block_size : 0, spin_limit, scale * kLog2e};
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+    // the flags and the status word start at zero on every launch (the reference's callers clear rblk_flag,
+    // rblk_flag1 with cudaMemset before each launch, fixed_fusion_test.cu:348-351)
+    zero_words_kernel<<<dim3((uint32_t)((flags + 256) / 4 / 256 + 1)), dim3(256), 0, s>>>(p.flags, (uint32_t)((flags + 256) / 4));
+    const dim3 grid(blocks, batch_dim, head_dim);
+#define SFB_CALL(BSV, TI, TO) sdd_softmax_split_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);
 #undef SFB_CALL

@@ -19,7 +19,7 @@ inline bool fused_sdd_softmax(CUstream stream, const uint2* nn_lut, const float*
                               uint state_dim, uint lut_heads, uint lut_dim, uint mask_heads, float scale) {
     // the reference passes the NT LUT length as lut_dim and derives the NN stride itself (:434)
     return ok(sfb_fused_sdd_softmax(stream, lut_cast(nn_lut), a, b, Y, SFB_F32, dtype_of<T>::value, Mask, nullptr,
-                                    block_size, blocks, batch_dim, ctx_blks_a, head_dim, state_dim, lut_heads,
+                                    /*row_order*/ nullptr, block_size, blocks, batch_dim, ctx_blks_a, head_dim, state_dim, lut_heads,
                                     lut_dim + ctx_blks_a, mask_heads, scale));
 }
 }  // namespace sfb_host

@@ -90,6 +90,45 @@ def test_fusion_attention2_probabilities(bs, bf16):
     assert np.abs(rows[0] - 1).max() < 2e-2
 
 
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("pattern", ["causal", "bigbird", "strided"])
+def test_split_variant_with_flags_matches_the_row_owner_kernel(pattern, bs, bf16):
+    """One work-group per block with flag / spin exchange (the reference's fusion_nt_softmax2 decomposition):
+    same probabilities as the oracle and as fusion_attention2, status word zero."""
+    nb, B, H = 16, 2, 3
+    luts, mask, Q, K, V, valid = setup(pattern, bs, nb, B, H, 50 + bs, bf16)
+    S = orc.sdd_nt(Q, K, luts["nt_lut"], bs)
+    P_want = orc.masked_softmax(S, luts["nn_lut"], nb, 0.125, mask=mask, valid_len=valid)
+    q, k = dev(Q, bf16), dev(K, bf16)
+    nt, nn = sfb.to_device(luts["nt_lut"]), sfb.to_device(luts["nn_lut"])
+    m, vl = (None if mask is None else sfb.to_device(mask)), sfb.to_device(valid)
+    for _ in range(2):   # the second call finds used scratch: the call clears what it needs
+        P, status = sfb.fusion_attention2_split(nt, nn, q, k, bs, luts["blocks"], 0.125, mask=m, valid_len=vl)
+        torch.cuda.synchronize()
+        assert int(status) == 0
+        got = P.cpu().numpy()
+        assert rel_err(got, P_want) <= (TOL_BF16 if bf16 else TOL_F32)
+        assert (got[P_want == 0] == 0).all()
+    row_owner = sfb.fusion_attention2(nn, q, k, bs, luts["blocks"], 0.125, mask=m, valid_len=vl)
+    assert rel_err(got, row_owner.cpu().numpy()) <= 1e-5
+    ordered = sfb.fusion_attention2(nn, q, k, bs, luts["blocks"], 0.125, mask=m, valid_len=vl,
+                                    row_order=sfb.to_device(luts["row_order"]))
+    assert torch.equal(ordered, row_owner)   # the order of the work does not change a bit of the result
+
+
+def test_split_variant_gives_up_instead_of_waiting_forever():
+    """With no polls allowed, a block whose block-row partners have not all arrived leaves without writing and
+    reports it; every work-group still exits."""
+    bs, nb, B, H = 64, 8, 1, 2
+    luts, mask, Q, K, V, valid = setup("causal", bs, nb, B, H, 60, False, masked=False)
+    q, k = dev(Q), dev(K)
+    P, status = sfb.fusion_attention2_split(sfb.to_device(luts["nt_lut"]), sfb.to_device(luts["nn_lut"]), q, k, bs,
+                                            luts["blocks"], 0.125, spin_limit=0)
+    torch.cuda.synchronize()
+    assert int(status) == 1
+
+
 def test_c2_shape_unfused_chain_fp32():
     B, H, L, d, bs = 2, 12, 1024, 64, 32
     luts = sfb.build_luts(PATTERNS["fixed"](L // bs))
@@ -159,7 +198,7 @@ def test_error_codes_instead_of_silent_no_op():
                               u(1), u(2), u(sfb.NT_OP), u(1), u(0), u(1)) == 8
     assert sfb.lib.sfb_masked_softmax(None, p(lut), None, p(q), p(q), 0, 3, None, u(64), u(1), u(1), u(1), u(1),
                                       u(1), u(2), u(1), u(1), C.c_float(0.125)) == 5
-    assert sfb.lib.sfb_fused_sdd_softmax(None, None, p(q), p(q), p(q), 0, 0, None, None, u(64), u(1), u(1), u(1),
+    assert sfb.lib.sfb_fused_sdd_softmax(None, None, p(q), p(q), p(q), 0, 0, None, None, None, u(64), u(1), u(1), u(1),
                                          u(1), u(64), u(1), u(2), u(1), C.c_float(0.125)) == 1
 
 
