@@ -134,6 +134,10 @@ size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t
  * Device entry points
  * ============================================================================================== */
 
+/* state_dim (the head size d) in every attention entry point below: 64 with fp32 or bf16 tensors; 32, 96 and
+ * 128 with fp32 Q / K / V (the dense operand of a product) -- the reference's K64 = false paths,
+ * openai_blocksparse.h:221-222.  Anything else returns SFB_ERR_HEAD_STATE. */
+
 /* Fully fused attention: O = softmax_rows(scale * Q K^T restricted to layout & mask & key<valid_len) V,
  * one work-group per (batch, head, block-row), no S/P in memory.  Replaces the sequence
  * bst_sgemm_nt -> BlocksparseMaskedSoftmax -> bst_sgemm_xn (transformer_attention_optimize.cu:728-748)

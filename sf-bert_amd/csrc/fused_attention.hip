@@ -470,7 +470,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
 // ------------------------------------------------------------------------------------------------
 // One LDS buffer (K tile and V tile); the next block waits in registers.
 template <int BS, int D>
-__global__ __launch_bounds__(BS * 2, 2) void fused_attention_f32_kernel(FusedParams p) {
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_kernel(FusedParams p) {
     using T = F32Tiles<BS, D>;
     constexpr int KT = BS / 32;
     constexpr int NO = D / 32;
@@ -577,13 +577,29 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
     const uint32_t grid = p.groups * 8u * ranks;
     clear_stale_error();
     if (in_dtype == SFB_BF16) {
-        if (p.mask || p.valid_len)
-            fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-        else
-            fused_attention_bf16_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+        if constexpr (D == 64) {
+            if (p.mask || p.valid_len)
+                fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+            else
+                fused_attention_bf16_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+        } else {
+            return SFB_ERR_HEAD_STATE;   // the bf16 kernel is built for head size 64 only
+        }
     } else
         fused_attention_f32_kernel<BS, D><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
     return launch_status();
+}
+
+// head sizes: 64 for both input types; 32, 96 and 128 for fp32 inputs
+template <int BS>
+static int launch_fused_any(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks, uint32_t state_dim) {
+    switch (state_dim) {
+        case 64: return launch_fused<BS, 64>(stream, p, in_dtype, ranks);
+        case 32: return launch_fused<BS, 32>(stream, p, in_dtype, ranks);
+        case 96: return launch_fused<BS, 96>(stream, p, in_dtype, ranks);
+        case 128: return launch_fused<BS, 128>(stream, p, in_dtype, ranks);
+        default: return SFB_ERR_HEAD_STATE;
+    }
 }
 
 static int check_common(const void* q, const void* k, const void* v, const void* o, int in_dtype,
@@ -593,7 +609,8 @@ static int check_common(const void* q, const void* k, const void* v, const void*
     if (!q || !k || !v || !o || !nn_lut) return SFB_ERR_NULL_POINTER;
     if (in_dtype != SFB_F32 && in_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (state_dim != 64 && (in_dtype != SFB_F32 || (state_dim != 32 && state_dim != 96 && state_dim != 128)))
+        return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (batch_dim == 0 || ctx_blks == 0 || head_dim == 0 || lut_heads == 0 || mask_heads == 0)
         return SFB_ERR_SHAPE;
@@ -640,8 +657,8 @@ extern "C" int sfb_fused_attention(sfb_stream_t stream, const void* q, const voi
                 lut_heads, lut_dim, mask_heads, scale);
     p.row_order = row_order;
     hipStream_t s = (hipStream_t)stream;
-    if (block_size == 64) return launch_fused<64, 64>(s, p, in_dtype, ctx_blks);
-    return launch_fused<32, 64>(s, p, in_dtype, ctx_blks);
+    if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, ctx_blks, state_dim);
+    return launch_fused_any<32>(s, p, in_dtype, ctx_blks, state_dim);
 }
 
 extern "C" size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
@@ -683,8 +700,8 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
     p.counters = (uint32_t*)workspace;
     p.partials = (float*)((uint8_t*)workspace + counters);
     hipStream_t s = (hipStream_t)stream;
-    if (block_size == 64) return launch_fused<64, 64>(s, p, in_dtype, n_items);
-    return launch_fused<32, 64>(s, p, in_dtype, n_items);
+    if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, n_items, state_dim);
+    return launch_fused_any<32>(s, p, in_dtype, n_items, state_dim);
 }
 
 extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k,

@@ -34,7 +34,8 @@ namespace sfb {
 // No registers are spent on staging and no ds_write / v_perm instructions are needed.
 template <int BS, int D>
 struct Bf16DirectTiles {
-    static_assert(D == 64, "128-byte rows");
+    // the layout below is for D = 64 (128-byte rows); the loaders and fragment readers assert it, so that merely
+    // naming the type for another head size (in a branch that is not taken) stays legal
     static constexpr int NW = BS / 32;                 // waves per work-group
     static constexpr int TILE_BYTES = BS * D * 2;
     static constexpr int GROUPS = BS / 8;              // 8-row groups (one load instruction each)
@@ -60,6 +61,7 @@ struct Bf16DirectTiles {
     static constexpr int LOADS = GROUPS / NW;
     static __device__ __forceinline__ void load_rows(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
+        static_assert(D == 64, "128-byte rows");
         const uint32_t n = (uint32_t)(NW * i) + wave;   // 8-row group
         uint32_t src;
         if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's

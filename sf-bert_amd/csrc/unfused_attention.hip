@@ -1171,6 +1171,24 @@ static int check_dtype(int d) { return (d == SFB_F32 || d == SFB_BF16) ? SFB_OK 
 
 using namespace sfb;
 
+// Head sizes: 64 with every type combination; 32, 96 and 128 with fp32 dense tensors (Q, K, V and the like).
+static int check_head_state(uint32_t state_dim, int dense_dtype) {
+    if (state_dim == 64) return SFB_OK;
+    if (dense_dtype == SFB_F32 && (state_dim == 32 || state_dim == 96 || state_dim == 128)) return SFB_OK;
+    return SFB_ERR_HEAD_STATE;
+}
+// CALL(D, T) for a head size other than 64: dense type float, T = the sparse tensor's type
+#define SFB_DISPATCH_D(DV, TS, CALL)                                      \
+    do {                                                                  \
+        if ((TS) == SFB_F32) { CALL(DV, float); } else { CALL(DV, __bf16); } \
+    } while (0)
+#define SFB_DISPATCH_OTHER_D(STATE, TS, CALL)                              \
+    do {                                                                  \
+        if ((STATE) == 32) SFB_DISPATCH_D(32, TS, CALL);                   \
+        else if ((STATE) == 96) SFB_DISPATCH_D(96, TS, CALL);              \
+        else SFB_DISPATCH_D(128, TS, CALL);                                \
+    } while (0)
+
 #define SFB_DISPATCH_2(BSV, T0, T1, CALL)                                                  \
     do {                                                                                   \
         if ((T0) == SFB_F32 && (T1) == SFB_F32) { CALL(BSV, float, float); }               \
@@ -1186,7 +1204,7 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (!lut || !a || !b || !c) return SFB_ERR_NULL_POINTER;
     if (check_dtype(in_dtype) || check_dtype(out_dtype)) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (check_head_state(state_dim, in_dtype)) return SFB_ERR_HEAD_STATE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks_a || !ctx_blks_b || !lut_heads) return SFB_ERR_SHAPE;
     if (lut_heads > 1 && lut_heads != head_dim) return SFB_ERR_SHAPE;
     if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
@@ -1196,6 +1214,15 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     const dim3 grid(blocks, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim != 64) {
+#define SFB_CALL64(DV, TO) sdd_nt_kernel<64, DV, float, TO><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_CALL32(DV, TO) sdd_nt_kernel<32, DV, float, TO><<<grid, dim3(64), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, out_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, out_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
 #define SFB_CALL(BSV, TI, TO) sdd_nt_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, out_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, out_dtype, SFB_CALL);
@@ -1243,7 +1270,7 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (check_dtype(a_dtype) || check_dtype(b_dtype)) return SFB_ERR_DTYPE;
     if (op != SFB_NN_OP && op != SFB_TN_OP) return SFB_ERR_ARGUMENT;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (check_head_state(state_dim, b_dtype)) return SFB_ERR_HEAD_STATE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks_b || !ctx_blks_c || !lut_heads) return SFB_ERR_SHAPE;
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks_c + blocks)) return SFB_ERR_SHAPE;
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
@@ -1252,6 +1279,24 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     const dim3 grid(p.groups * 8u * ctx_blks_c);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim != 64) {
+#define SFB_TN64(DV, TA) dsd_tn_kernel<64, DV, TA, float><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_TN32(DV, TA) dsd_tn_kernel<32, DV, TA, float><<<grid, dim3(64), 0, s>>>(p)
+#define SFB_NN64(DV, TA) dsd_nn_kernel<64, DV, TA, float><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_NN32(DV, TA) dsd_nn_kernel<32, DV, TA, float><<<grid, dim3(64), 0, s>>>(p)
+        if (op == SFB_TN_OP) {
+            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_TN64);
+            else SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_TN32);
+        } else {
+            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_NN64);
+            else SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_NN32);
+        }
+#undef SFB_TN64
+#undef SFB_TN32
+#undef SFB_NN64
+#undef SFB_NN32
+        return launch_status();
+    }
     if (op == SFB_TN_OP) {
 #define SFB_CALL(BSV, TA, TB) dsd_tn_kernel<BSV, 64, TA, TB><<<grid, dim3(BSV * 2), 0, s>>>(p)
         if (block_size == 64) SFB_DISPATCH_2(64, a_dtype, b_dtype, SFB_CALL);
@@ -1306,7 +1351,7 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
     if (!nn_lut || !a || !b || !y) return SFB_ERR_NULL_POINTER;
     if (check_dtype(in_dtype) || check_dtype(y_dtype)) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (check_head_state(state_dim, in_dtype)) return SFB_ERR_HEAD_STATE;
     if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads || !mask_heads) return SFB_ERR_SHAPE;
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
@@ -1318,6 +1363,15 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
     const dim3 grid(p.groups * 8u * ctx_blks);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim != 64) {
+#define SFB_CALL64(DV, TO) sdd_softmax_kernel<64, DV, float, TO><<<grid, dim3(128 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+#define SFB_CALL32(DV, TO) sdd_softmax_kernel<32, DV, float, TO><<<grid, dim3(64 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, y_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, y_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
 #define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2 * kSddSoftmaxKeyGroups), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);

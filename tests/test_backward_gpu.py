@@ -172,3 +172,30 @@ def test_attention_backward(pattern, bs, bf16):
     tol = TOL_BF16 if bf16 else TOL_F32
     for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
         assert rel_err(got.cpu().numpy(), want) <= tol, name
+
+
+@pytest.mark.parametrize("d", [32, 96, 128])
+@pytest.mark.parametrize("bs,store_bf16", [(32, False), (64, False), (64, True)])
+def test_unfused_forward_and_backward_at_other_head_sizes(d, bs, store_bf16):
+    """fp32 Q/K/V/dO with head size 32, 96 or 128; S, P, dP, dS stored in fp32 or bf16: every product kernel
+    (NT, NN, TN) and the two-stage fusion (its per-block comparison variant stays at head size 64)."""
+    nb, B, H = 8, 2, 2
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    blocks = luts["blocks"]
+    scale = float(1.0 / np.sqrt(d))
+    Q, K, V = qkv(B, nb * bs, H, d, seed=3 * d + bs)
+    dO = orc.fill_normal((B, nb * bs, H, d), 90 + d)
+    dQ, dK, dV, P = orc.attention_backward(Q, K, V, dO, luts, bs, scale)
+    q, k, v, do = (dev(x) for x in (Q, K, V, dO))
+    ld = {name: sfb.to_device(luts[name]) for name in ("nt_lut", "nn_lut", "tn_lut")}
+    code = sfb.BF16 if store_bf16 else sfb.F32
+    tol = TOL_BF16 if store_bf16 else TOL_F32
+    p = sfb.fusion_attention2(ld["nn_lut"], q, k, bs, blocks, scale, out_dtype=code)
+    assert rel_err(p.float().cpu().numpy(), P) <= tol
+    S = sfb.bst_sgemm_nt(ld["nt_lut"], q, k, bs, blocks, out_dtype=code)
+    assert rel_err(S.float().cpu().numpy(), orc.sdd_nt(Q, K, luts["nt_lut"], bs)) <= tol
+    O = sfb.bst_sgemm_xn(ld["nn_lut"], p, v, nb)
+    assert rel_err(O.cpu().numpy(), orc.attention(Q, K, V, luts["nn_lut"], bs, scale)) <= tol
+    dq, dk, dv = sfb.attention_backward(q, k, v, do, p, ld, bs, blocks, scale)
+    for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+        assert rel_err(got.cpu().numpy(), want) <= tol, name
