@@ -140,7 +140,14 @@ def time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16):
     dense_bytes = q.numel() * q.element_size()
     tn = _time(torch, lambda: sfb.bst_sgemm_xn(ld["tn_lut"], p, d_out, nb, op=sfb.TN_OP, c=c), 200, 20)
     grad = _time(torch, lambda: sfb.BlocksparseMaskedSoftmaxGrad(ld["nn_lut"], dp, p, nb, scale, dx=ds), 200, 20)
+    o = sfb.bst_sgemm_xn(ld["nn_lut"], p, v, nb)
+    delta = sfb.row_dot(d_out, o)
     return {"ms_per_call": _time(torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale), 100, 20),
+            "ms_per_call_with_forward_output": _time(
+                torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale, o=o), 100, 20),
+            "row_dot_ms": _time(torch, lambda: sfb.row_dot(d_out, o), 200, 20),
+            "sdd_softmax_grad_ms": _time(
+                torch, lambda: sfb.sdd_softmax_grad(ld["nt_lut"], d_out, v, p, delta, bs, blocks, scale, ds=ds), 200, 20),
             "dsd_tn_ms": tn, "dsd_tn_hbm_GBs": (sparse_bytes + dense_bytes + c.numel() * 4) / tn / 1e6,
             "sdd_nt_ms": _time(torch, lambda: sfb.bst_sgemm_nt(ld["nt_lut"], d_out, v, bs, blocks, c=dp), 200, 20),
             "softmax_grad_ms": grad, "softmax_grad_hbm_GBs": 3 * sparse_bytes / grad / 1e6,

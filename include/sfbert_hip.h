@@ -212,6 +212,19 @@ int sfb_masked_softmax_grad(sfb_stream_t stream, const sfb_uint2* lut, const voi
                             uint32_t head_dim, uint32_t ctx_blks, uint32_t lut_heads, uint32_t lut_dim,
                             uint32_t max_lut, float scale);
 
+/* MI355X additions: the NT product dP = dO V^T and the softmax gradient of the backward pass
+ * (transformer_attention_optimize.cu:936, 945) in one kernel, dS = (dO V^T - delta) * P * scale per block, where
+ * delta[b][h][q] = sum_d dO[b][q][h][d] * O[b][q][h][d] (sfb_row_dot) replaces the gradient's sum over the sparse
+ * row (ewops.h:108-113): the two are equal because O = P V.  dP is never written.  d_out, v [dev] [batch, ctx,
+ * heads, state] of in_dtype; o [dev] fp32 (the forward output); p, ds [dev] sparse, of sparse_dtype; delta [dev]
+ * fp32 [batch][heads][ctx]; nt_lut [dev]. */
+int sfb_row_dot(sfb_stream_t stream, float* delta, const void* d_out, const float* o, int dtype, uint32_t batch_dim,
+                uint32_t ctx, uint32_t head_dim, uint32_t state_dim);
+int sfb_sdd_softmax_grad(sfb_stream_t stream, const sfb_uint2* nt_lut, const void* d_out, const void* v,
+                         const void* p, const float* delta, void* ds, int in_dtype, int sparse_dtype,
+                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                         uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads, float scale);
+
 /* bst_sgemm_xn (blocksparse.h:965-1014).  op = SFB_NN_OP: C_rowblk = sum over the row's blocks of
  * A_blk . B_colblk, lut = NN LUT.  op = SFB_TN_OP (the backward products dV = P^T dO, dK = dS^T Q;
  * matmul.h:81-99): C_colblk = sum over the column's blocks of A_blk^T . B_rowblk, lut = TN LUT.

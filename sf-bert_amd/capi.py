@@ -60,7 +60,7 @@ EXPORTED = [
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
-    "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split",
+    "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_gemm_bias", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
@@ -403,15 +403,45 @@ def fusion_attention2_split(nt_lut, nn_lut, a, b, block_size, blocks, scale, mas
     return y, scratch[nbytes - 256:nbytes - 252].view(torch.int32)
 
 
-def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None):
+def row_dot(d_out, o):
+    """delta [B, H, L] = sum_d dO * O (the row term of the softmax gradient, since O = P V)."""
+    import torch
+    B, L, H, d = d_out.shape
+    delta = torch.empty((B, H, L), device=d_out.device, dtype=torch.float32)
+    _check(lib.sfb_row_dot(_stream(), _dev(delta), _dev(d_out), _dev(o), _dtype_code(d_out), C.c_uint32(B),
+                           C.c_uint32(L), C.c_uint32(H), C.c_uint32(d)), "sfb_row_dot")
+    return delta
+
+
+def sdd_softmax_grad(nt_lut, d_out, v, p, delta, block_size, blocks, scale, lut_heads=1, ds=None):
+    """dS = (dO V^T - delta) * P * scale per block in one kernel (dP stays in registers)."""
+    import torch
+    B, L, H, d = d_out.shape
+    if ds is None:
+        ds = torch.empty_like(p)
+    _check(lib.sfb_sdd_softmax_grad(_stream(), _dev(nt_lut), _dev(d_out), _dev(v), _dev(p), _dev(delta), _dev(ds),
+                                    _dtype_code(d_out), _dtype_code(p), C.c_uint32(block_size), C.c_uint32(blocks),
+                                    C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d),
+                                    C.c_uint32(lut_heads), C.c_float(scale)), "sfb_sdd_softmax_grad")
+    return ds
+
+
+def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None, o=None):
     """Gradients of O = P V, P = masked softmax(scale * Q K^T) from the stored probabilities P, in the order of
     the reference's backward (transformer_attention_optimize.cu:924-965):
         dV = P^T dO (TN), dP = dO V^T (NT), dS = softmax grad, dK = dS^T Q (TN), dQ = dS K (NN).
     q, k, v, d_out [B, L, H, d]; p [B, H, blocks, bs, bs]; luts_dev: dict of device buffers nt_lut, nn_lut,
-    tn_lut.  dP / dS use p's dtype unless work_dtype says otherwise.  Returns (dq, dk, dv) fp32."""
+    tn_lut.  dP / dS use p's dtype unless work_dtype says otherwise.  o: the forward output O (fp32), optional; when
+    given, dP and the softmax gradient are computed by one kernel (sdd_softmax_grad).  Returns (dq, dk, dv) fp32."""
     nb = q.shape[1] // block_size
     code = _dtype_code(p) if work_dtype is None else work_dtype
     dv = bst_sgemm_xn(luts_dev["tn_lut"], p, d_out, nb, op=TN_OP)
+    if o is not None:
+        # with the forward output at hand the NT product and the softmax gradient are one kernel
+        ds = sdd_softmax_grad(luts_dev["nt_lut"], d_out, v, p, row_dot(d_out, o), block_size, blocks, scale)
+        dk = bst_sgemm_xn(luts_dev["tn_lut"], ds, q, nb, op=TN_OP)
+        dq = bst_sgemm_xn(luts_dev["nn_lut"], ds, k, nb, op=NN_OP)
+        return dq, dk, dv
     dp = bst_sgemm_nt(luts_dev["nt_lut"], d_out, v, block_size, blocks, out_dtype=code)
     if dp.dtype != p.dtype:
         p = p.to(dp.dtype)

@@ -127,17 +127,60 @@ __device__ __forceinline__ void score_tile(f32x16 (&s)[BS / 32], const KTile<BS,
         }
 }
 
-// Store this lane's part of a BS x BS block (row = its query): groups of 4 consecutive keys.
-template <int BS, typename TOut>
-__device__ __forceinline__ void store_block_row(TOut* row_ptr, const f32x16 (&s)[BS / 32], uint32_t half) {
+// A wave's 32 x BS part of a sparse block between registers (MFMA layout: a lane holds one query row in groups of
+// 4 keys) and memory, through a wave-private LDS slab so that memory sees whole rows: the 32 rows are contiguous
+// in memory (32 * BS elements); straight from the MFMA layout a store instruction would touch all 32 rows with 8
+// or 16 bytes each, here every instruction moves 1 KiB of consecutive bytes.
+template <int BS, typename T>
+struct RowSlab {
+    static constexpr int ROW_BYTES = BS * (int)sizeof(T);
+    static constexpr int PITCH = ROW_BYTES + 16;          // padded LDS row
+    static constexpr int BYTES = 32 * PITCH;              // per wave
+    static constexpr int CHUNKS = ROW_BYTES / 16;         // 16-byte chunks per row
+    static constexpr int ROWS_PER_PASS = 64 / CHUNKS, PASSES = 32 / ROWS_PER_PASS;
+
+    // registers (this lane's query row, groups of 4 keys) -> memory; rows: the wave's first row in memory
+    static __device__ __forceinline__ void store(T* rows, const f32x16 (&s)[BS / 32], uint8_t* slab, uint32_t lane) {
+        const uint32_t qn = lane & 31, half = lane >> 5;
+        T* mine = (T*)(slab + qn * PITCH);
 #pragma unroll
-    for (int kt = 0; kt < BS / 32; ++kt)
+        for (int kt = 0; kt < BS / 32; ++kt)
 #pragma unroll
-        for (int ig = 0; ig < 4; ++ig) {
-            const f32x4 v = {s[kt][ig * 4 + 0], s[kt][ig * 4 + 1], s[kt][ig * 4 + 2], s[kt][ig * 4 + 3]};
-            Elem<TOut>::store4(row_ptr + kt * 32 + ig * 8 + half * 4, v);
+            for (int ig = 0; ig < 4; ++ig) {
+                const f32x4 v = {s[kt][ig * 4 + 0], s[kt][ig * 4 + 1], s[kt][ig * 4 + 2], s[kt][ig * 4 + 3]};
+                Elem<T>::store4(mine + kt * 32 + ig * 8 + half * 4, v);
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+            const uint32_t row = pass * ROWS_PER_PASS + lane / CHUNKS, c = lane % CHUNKS;
+            const u32x4 v = *(const u32x4*)(slab + row * PITCH + c * 16);
+            *(u32x4*)((uint8_t*)rows + row * ROW_BYTES + c * 16) = v;
         }
-}
+    }
+    // memory -> registers in the same layout
+    static __device__ __forceinline__ void load(f32x16 (&s)[BS / 32], const T* rows, uint8_t* slab, uint32_t lane) {
+        const uint32_t qn = lane & 31, half = lane >> 5;
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+            const uint32_t row = pass * ROWS_PER_PASS + lane / CHUNKS, c = lane % CHUNKS;
+            *(u32x4*)(slab + row * PITCH + c * 16) = *(const u32x4*)((const uint8_t*)rows + row * ROW_BYTES + c * 16);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const T* mine = (const T*)(slab + qn * PITCH);
+#pragma unroll
+        for (int kt = 0; kt < BS / 32; ++kt)
+#pragma unroll
+            for (int ig = 0; ig < 4; ++ig) {
+                const f32x4 v = Elem<T>::load4(mine + kt * 32 + ig * 8 + half * 4);
+                s[kt][ig * 4 + 0] = v.x; s[kt][ig * 4 + 1] = v.y; s[kt][ig * 4 + 2] = v.z; s[kt][ig * 4 + 3] = v.w;
+            }
+    }
+};
 
 // ---------------------------------------------------------------------------------------------
 // sdd: grid (blocks, batch, heads), one BS x BS block per work-group (openai_blocksparse.h:224)
@@ -160,8 +203,74 @@ __global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
     const TIn* k_blk = (const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, D);
     f32x16 s[BS / 32];
     score_tile_direct<BS, D, TIn>(s, q_row, k_blk, row_stride, qn, half);
-    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32 + qn) * BS;
-    store_block_row<BS, TOut>(out, s, half);
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TOut>::BYTES];
+    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32) * BS;
+    RowSlab<BS, TOut>::store(out, s, slabs[wave], lane);
+}
+
+// ---------------------------------------------------------------------------------------------
+// dS = (dO V^T - delta) * P * scale per block: the NT product of the backward pass and the softmax gradient in
+// one kernel.  The row term of the gradient, sum_k dP_k P_k (ewops.h:108-113), equals delta_q = sum_d dO_qd O_qd
+// because O = P V, so no reduction over the sparse row is needed and dP never goes to memory.
+// Grid (blocks, batch, heads) as the sdd.
+// ---------------------------------------------------------------------------------------------
+struct SddGradParams {
+    const sfb_uint2* lut;    // NT LUT
+    const void* d_out;       // dO [batch, ctx, heads, D]
+    const void* v;           // V  [batch, ctx, heads, D]
+    const void* p;           // P  sparse
+    const float* delta;      // [batch][heads][ctx]
+    void* ds;                // dS sparse
+    uint32_t blocks, heads, ctx, lut_stride;
+    float scale;
+};
+
+template <int BS, int D, typename TIn, typename TS>
+__global__ __launch_bounds__(BS * 2) void sdd_softmax_grad_kernel(SddGradParams p) {
+    const uint32_t blk = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
+    const sfb_uint2 e = p.lut[(size_t)h * p.lut_stride + blk];
+    const uint32_t q = e.x * BS + wave * 32 + qn;
+    const TIn* do_row = (const TIn*)p.d_out + token_offset(b, q, h, p.ctx, p.heads, D);
+    const TIn* v_blk = (const TIn*)p.v + token_offset(b, e.y * BS, h, p.ctx, p.heads, D);
+    f32x16 s[BS / 32];
+    score_tile_direct<BS, D, TIn>(s, do_row, v_blk, p.heads * D, qn, half);   // dP^T: this lane's query, 16 keys per tile
+    const float delta = p.delta[((size_t)b * p.heads + h) * p.ctx + q];
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TS>::BYTES];
+    const size_t rows = ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32) * BS;   // the wave's 32 rows
+    f32x16 pv[BS / 32];
+    RowSlab<BS, TS>::load(pv, (const TS*)p.p + rows, slabs[wave], lane);
+#pragma unroll
+    for (int kt = 0; kt < BS / 32; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = (s[kt][i] - delta) * pv[kt][i] * p.scale;
+    // the slab is reused: every lane has taken its values out before any lane overwrites them
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    RowSlab<BS, TS>::store((TS*)p.ds + rows, s, slabs[wave], lane);
+}
+
+// delta[b][h][q] = sum_d dO[b][q][h][d] * O[b][q][h][d]; 16 lanes per (token, head) row of D elements
+template <int D, typename TIn>
+__global__ __launch_bounds__(256) void row_dot_kernel(float* delta, const TIn* d_out, const float* o, uint32_t batch,
+                                                      uint32_t ctx, uint32_t heads) {
+    constexpr int PER = D / 16;   // elements per lane
+    const uint64_t row = ((uint64_t)blockIdx.x * 256 + threadIdx.x) / 16;   // over batch * ctx * heads
+    const uint32_t part = threadIdx.x & 15;
+    if (row >= (uint64_t)batch * ctx * heads) return;
+    const TIn* a = d_out + row * D + part * PER;
+    const float* c = o + row * D + part * PER;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) sum += Elem<TIn>::load(a + i) * c[i];
+#pragma unroll
+    for (int d = 8; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
+    if (part == 0) {
+        const uint32_t hh = (uint32_t)(row % heads);
+        const uint64_t tok = row / heads;
+        const uint32_t bb = (uint32_t)(tok / ctx), qq = (uint32_t)(tok % ctx);
+        delta[((size_t)bb * heads + hh) * ctx + qq] = sum;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -970,6 +1079,7 @@ template <int BS, int D, typename TIn, typename TOut>
 __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_kernel(SddSoftmaxParams p) {
     constexpr int KT = BS / 32, QW = BS / 32, KG = kSddSoftmaxKeyGroups;
     __shared__ float stats[KG][BS][2];
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[QW * KG][RowSlab<BS, TOut>::BYTES];
     const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
@@ -1041,7 +1151,7 @@ __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_ker
                 for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) s[kt][i] = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc)) * inv;
-                store_block_row<BS, TOut>(Y + ((size_t)blk * BS + q_in_block) * BS, s, half);
+                RowSlab<BS, TOut>::store(Y + ((size_t)blk * BS + (wave % QW) * 32) * BS, s, slabs[wave], lane);
             }
         }
     }
@@ -1156,8 +1266,9 @@ __global__ __launch_bounds__(BS * 2) void sdd_softmax_split_kernel(SplitSoftmaxP
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[kt][i] *= inv;
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TOut>::BYTES];
     TOut* Y = (TOut*)p.y + (size_t)bh * p.blocks * BS * BS;
-    store_block_row<BS, TOut>(Y + ((size_t)blk * BS + q_in_block) * BS, s, half);
+    RowSlab<BS, TOut>::store(Y + ((size_t)blk * BS + wave * 32) * BS, s, slabs[wave], lane);
 }
 
 __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, uint32_t n) {
@@ -1423,6 +1534,64 @@ extern "C" int sfb_fused_sdd_softmax_split(sfb_stream_t stream, const sfb_uint2*
 #define SFB_CALL(BSV, TI, TO) sdd_softmax_split_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, y_dtype, SFB_CALL);
     else SFB_DISPATCH_2(32, in_dtype, y_dtype, SFB_CALL);
+#undef SFB_CALL
+    return launch_status();
+}
+
+extern "C" int sfb_row_dot(sfb_stream_t stream, float* delta, const void* d_out, const float* o, int dtype,
+                           uint32_t batch_dim, uint32_t ctx, uint32_t head_dim, uint32_t state_dim) {
+    if (!delta || !d_out || !o) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(dtype)) return SFB_ERR_DTYPE;
+    if (check_head_state(state_dim, dtype)) return SFB_ERR_HEAD_STATE;
+    if (!batch_dim || !ctx || !head_dim) return SFB_ERR_SHAPE;
+    const uint64_t rows = (uint64_t)batch_dim * ctx * head_dim;
+    if ((rows * 16 + 255) / 256 > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const dim3 grid((uint32_t)((rows * 16 + 255) / 256));
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+#define SFB_CALL(DV)                                                                                          \
+    do {                                                                                                      \
+        if (dtype == SFB_F32) row_dot_kernel<DV, float><<<grid, dim3(256), 0, s>>>(delta, (const float*)d_out, o, batch_dim, ctx, head_dim); \
+        else row_dot_kernel<DV, __bf16><<<grid, dim3(256), 0, s>>>(delta, (const __bf16*)d_out, o, batch_dim, ctx, head_dim);                 \
+    } while (0)
+    if (state_dim == 64) SFB_CALL(64);
+    else if (state_dim == 32) SFB_CALL(32);
+    else if (state_dim == 96) SFB_CALL(96);
+    else SFB_CALL(128);
+#undef SFB_CALL
+    return launch_status();
+}
+
+extern "C" int sfb_sdd_softmax_grad(sfb_stream_t stream, const sfb_uint2* nt_lut, const void* d_out, const void* v,
+                                    const void* p, const float* delta, void* ds, int in_dtype, int sparse_dtype,
+                                    uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                    uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads, float scale) {
+    if (!nt_lut || !d_out || !v || !p || !delta || !ds) return SFB_ERR_NULL_POINTER;
+    if (check_dtype(in_dtype) || check_dtype(sparse_dtype)) return SFB_ERR_DTYPE;
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (check_head_state(state_dim, in_dtype)) return SFB_ERR_HEAD_STATE;
+    if (!blocks || !batch_dim || !head_dim || !ctx_blks || !lut_heads) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && lut_heads != head_dim) return SFB_ERR_SHAPE;
+    if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)d_out | (uintptr_t)v | (uintptr_t)p | (uintptr_t)ds) & 15u) return SFB_ERR_ALIGNMENT;
+    SddGradParams g = {nt_lut, d_out, v, p, delta, ds, blocks, head_dim, ctx_blks * block_size,
+                       lut_heads > 1 ? blocks : 0, scale};
+    const dim3 grid(blocks, batch_dim, head_dim);
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+    if (state_dim != 64) {
+#define SFB_CALL64(DV, TS) sdd_softmax_grad_kernel<64, DV, float, TS><<<grid, dim3(128), 0, s>>>(g)
+#define SFB_CALL32(DV, TS) sdd_softmax_grad_kernel<32, DV, float, TS><<<grid, dim3(64), 0, s>>>(g)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, sparse_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, sparse_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
+#define SFB_CALL(BSV, TI, TS) sdd_softmax_grad_kernel<BSV, 64, TI, TS><<<grid, dim3(BSV * 2), 0, s>>>(g)
+    if (block_size == 64) SFB_DISPATCH_2(64, in_dtype, sparse_dtype, SFB_CALL);
+    else SFB_DISPATCH_2(32, in_dtype, sparse_dtype, SFB_CALL);
 #undef SFB_CALL
     return launch_status();
 }

@@ -172,6 +172,16 @@ def test_attention_backward(pattern, bs, bf16):
     tol = TOL_BF16 if bf16 else TOL_F32
     for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
         assert rel_err(got.cpu().numpy(), want) <= tol, name
+    # with the forward output: dP and the softmax gradient in one kernel, the row term taken from dO . O
+    o = sfb.fused_attention(q, k, v, luts_dev["nn_lut"], bs, blocks, 0.125,
+                            mask=None if mask is None else sfb.to_device(mask))
+    delta = sfb.row_dot(do, o).cpu().numpy()
+    want_delta = np.einsum("blhd,blhd->bhl", dO.astype(np.float64), orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125,
+                                                                                    mask=mask).astype(np.float64))
+    assert np.abs(delta - want_delta).max() <= tol * np.abs(want_delta).max()
+    dq2, dk2, dv2 = sfb.attention_backward(q, k, v, do, p, luts_dev, bs, blocks, 0.125, o=o)
+    for name, got, want in (("dq", dq2, dQ), ("dk", dk2, dK), ("dv", dv2, dV)):
+        assert rel_err(got.cpu().numpy(), want) <= tol, name
 
 
 @pytest.mark.parametrize("d", [32, 96, 128])
@@ -197,5 +207,8 @@ def test_unfused_forward_and_backward_at_other_head_sizes(d, bs, store_bf16):
     O = sfb.bst_sgemm_xn(ld["nn_lut"], p, v, nb)
     assert rel_err(O.cpu().numpy(), orc.attention(Q, K, V, luts["nn_lut"], bs, scale)) <= tol
     dq, dk, dv = sfb.attention_backward(q, k, v, do, p, ld, bs, blocks, scale)
+    for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+        assert rel_err(got.cpu().numpy(), want) <= tol, name
+    dq, dk, dv = sfb.attention_backward(q, k, v, do, p, ld, bs, blocks, scale, o=O)
     for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
         assert rel_err(got.cpu().numpy(), want) <= tol, name
