@@ -155,6 +155,28 @@ def time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16):
             "sp_storage": "bf16" if bf16 else "f32"}
 
 
+def time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, max_blocks, flops_forward):
+    """Training pair of the fused path: forward with log-sum-exp output, then dQ, dK, dV in two kernels that keep
+    P, dP and dS on chip.  Backward FLOPs counted as 2.5 x forward (five block products instead of two)."""
+    B, L, H, d = q.shape
+    nb = L // bs
+    sched = sfb.build_schedule(luts["nn_lut"], nb, max_blocks)
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    nn, tn, items = sfb.to_device(luts["nn_lut"]), sfb.to_device(luts["tn_lut"]), sfb.to_device(sched["items"])
+    d_out = torch.randn((B, L, H, d), device="cuda").to(q.dtype)
+    fwd = lambda: sfb.fused_attention_forward_lse(q, k, v, nn, items, sched, ws, bs, blocks, scale)
+    o, lse = fwd()
+    rs, cs = sched, sfb.build_schedule(luts["tn_lut"], nb, max_blocks)
+    rs["items_dev"], cs["items_dev"] = items, sfb.to_device(cs["items"])
+    nbytes = int(sfb.lib.sfb_backward_workspace_bytes(rs["n_parts"], cs["n_parts"], B, H, bs, d))
+    bws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device="cuda")
+    bwd = lambda: sfb.fused_attention_backward(q, k, v, o, d_out, lse, nn, tn, bs, blocks, scale, row_sched=rs,
+                                               col_sched=cs, workspace=bws)
+    ms_b = _time(torch, bwd, 200, 20)
+    return {"forward_with_lse_ms": _time(torch, fwd, 200, 20), "backward_ms": ms_b,
+            "backward_TFLOPs": 2.5 * flops_forward / (ms_b * 1e-3) / 1e12}
+
+
 def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
     """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
     B, L, ffn = 8, 4096, 3072
@@ -328,6 +350,9 @@ def main():
     if not args.skip_extras:
         result["unfused"] = time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
         result["backward_unfused"] = time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
+        if bf16:
+            result["backward_fused"] = time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale,
+                                                           args.max_blocks, flops)
         if args.workload == "c4":
             result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, args.max_blocks)
             result["model_forward"] = time_model(sfb, torch, luts, bs, H, d, args.max_blocks)

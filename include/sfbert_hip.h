@@ -178,6 +178,42 @@ int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const v
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
+/* The same launch for a training step: additionally writes lse [dev] fp32 [batch][heads][ctx], the base-2
+ * logarithm of each query row's softmax denominator in units where the normalised probability of a key with raw
+ * score s is exp2(s * scale * log2(e) - lse).  sfb_fused_attention_backward rebuilds P from it. */
+int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                      float* lse, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
+                                      const void* mask, const int32_t* valid_len, const sfb_work_item* items,
+                                      uint32_t n_items, uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts,
+                                      void* workspace, size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                      uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                      uint32_t mask_heads, float scale);
+
+/* MI355X addition: the whole backward of the attention in two kernels, with P, dP and dS kept on chip.  Same
+ * arithmetic as the reference's sequence TN, NT, softmax gradient, TN, NN (transformer_attention_optimize.cu:
+ * 924-965; ewops.h:101-124; matmul.h:81-99): P = exp2(S scale log2e - lse), dV = P^T dO, dS = P (dO V^T - delta)
+ * scale, dK = dS^T Q, dQ = dS K, where delta = rowsum(dO * O) (computed here into the caller's buffer) stands for
+ * the gradient's sum over the sparse row.  q, k, v, d_out [dev] bf16 [batch, ctx, heads, 64]; o [dev] fp32, the
+ * forward output; lse [dev] from sfb_fused_attention_scheduled_lse; delta [dev] fp32 [batch][heads][ctx]
+ * (scratch, overwritten); dq, dk, dv [dev] fp32; nn_lut, tn_lut [dev] (one layout for all heads); mask
+ * block-major.  row_items / col_items [dev] (may be NULL: one work-group per block-row / block-column in index
+ * order): work items of sfb_build_schedule over nn_lut / over tn_lut, longest first, with lines of more than
+ * max_blocks blocks cut into chunks; the chunks of a split line write partial records into workspace ([dev],
+ * 256-byte aligned, sfb_backward_workspace_bytes() bytes; n_*_parts as returned by sfb_build_schedule) and a
+ * follow-up kernel adds them in chunk order, so results do not depend on timing.  dtype must be SFB_BF16 (fp32
+ * tensors: use the unfused sequence). */
+size_t sfb_backward_workspace_bytes(uint32_t n_row_parts, uint32_t n_col_parts, uint32_t batch_dim,
+                                    uint32_t head_dim, uint32_t block_size, uint32_t state_dim);
+int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, const void* k, const void* v, const float* o,
+                                 const void* d_out, const float* lse, float* delta, float* dq, float* dk, float* dv,
+                                 int dtype, const sfb_uint2* nn_lut, const sfb_uint2* tn_lut, const void* mask,
+                                 const int32_t* valid_len, const sfb_work_item* row_items, uint32_t n_row_items,
+                                 uint32_t n_row_heavy, uint32_t n_row_parts, const sfb_work_item* col_items,
+                                 uint32_t n_col_items, uint32_t n_col_heavy, uint32_t n_col_parts, void* workspace,
+                                 size_t workspace_bytes, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                 uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
+                                 float scale);
+
 
 /* ---- the unfused trio (kept as the no_fusion comparison) ------------------------------------ */
 

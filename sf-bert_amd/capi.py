@@ -49,6 +49,7 @@ lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
 lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
+lib.sfb_backward_workspace_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -59,6 +60,7 @@ EXPORTED = [
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
+    "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
@@ -254,6 +256,53 @@ def fused_attention(q, k, v, nn_lut, block_size, blocks, scale, mask=None, valid
                                    C.c_uint32(nb + blocks), C.c_uint32(mask_heads), C.c_float(scale)),
            "sfb_fused_attention")
     return out
+
+
+def fused_attention_forward_lse(q, k, v, nn_lut, items, sched, workspace, block_size, blocks, scale,
+                                mask=None, valid_len=None, mask_heads=1):
+    """Forward of a training step: (O fp32, lse [B, H, L]) through sfb_fused_attention_scheduled_lse."""
+    import torch
+    B, L, H, d = q.shape
+    out = torch.empty((B, L, H, d), dtype=torch.float32, device=q.device)
+    lse = torch.empty((B, H, L), dtype=torch.float32, device=q.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(lib.sfb_fused_attention_scheduled_lse(
+        _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dev(lse), _dtype_code(q), F32, _dev(nn_lut), _dev(mask),
+        _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]),
+        C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes),
+        C.c_uint32(block_size), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H),
+        C.c_uint32(d), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled_lse")
+    return out, lse
+
+
+def fused_attention_backward(q, k, v, o, d_out, lse, nn_lut, tn_lut, block_size, blocks, scale, mask=None,
+                             valid_len=None, mask_heads=1, row_sched=None, col_sched=None, workspace=None):
+    """(dq, dk, dv) fp32 from bf16 q, k, v, d_out, the forward output o and lse, in two kernels
+    (sfb_fused_attention_backward); nothing sparse goes through memory.  row_sched / col_sched: build_schedule()
+    over the NN / TN look-up table with its "items" already on the device under "items_dev" (None: one
+    work-group per block-row / block-column)."""
+    import torch
+    B, L, H, d = q.shape
+    dq, dk, dv = (torch.empty((B, L, H, d), dtype=torch.float32, device=q.device) for _ in range(3))
+    delta = torch.empty((B, H, L), dtype=torch.float32, device=q.device)
+    for t in (q, k, v, o, d_out):
+        if not t.is_contiguous():
+            raise SfbError(4, "non-contiguous tensor")
+    rs, cs = row_sched or {}, col_sched or {}
+    nbytes = int(lib.sfb_backward_workspace_bytes(C.c_uint32(rs.get("n_parts", 0)), C.c_uint32(cs.get("n_parts", 0)),
+                                                  C.c_uint32(B), C.c_uint32(H), C.c_uint32(block_size), C.c_uint32(d)))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    _check(lib.sfb_fused_attention_backward(
+        _stream(), _dev(q), _dev(k), _dev(v), _dev(o), _dev(d_out), _dev(lse), _dev(delta), _dev(dq), _dev(dk),
+        _dev(dv), _dtype_code(q), _dev(nn_lut), _dev(tn_lut), _dev(mask), _dev(valid_len),
+        _dev(rs.get("items_dev")), C.c_uint32(rs.get("n_items", 0)), C.c_uint32(rs.get("n_heavy", 0)),
+        C.c_uint32(rs.get("n_parts", 0)), _dev(cs.get("items_dev")), C.c_uint32(cs.get("n_items", 0)),
+        C.c_uint32(cs.get("n_heavy", 0)), C.c_uint32(cs.get("n_parts", 0)), _dev(workspace),
+        C.c_size_t(workspace.numel() if workspace is not None else 0), C.c_uint32(block_size), C.c_uint32(blocks),
+        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(mask_heads),
+        C.c_float(scale)), "sfb_fused_attention_backward")
+    return dq, dk, dv
 
 
 def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_size, blocks, scale,

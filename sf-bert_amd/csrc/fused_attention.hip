@@ -24,6 +24,7 @@ struct FusedParams {
     const void* k;
     const void* v;
     float* o;                       // fp32, or bf16 (o_bf16 != 0) behind the same pointer
+    float* lse;                     // [batch][heads][ctx] base-2 log of each row's softmax denominator, or nullptr
     const sfb_uint2* nn_lut;
     const void* mask;               // block-major keep words, or nullptr
     const int32_t* valid_len;       // per batch, or nullptr
@@ -148,11 +149,14 @@ __device__ __forceinline__ float* output_row(const FusedParams& p, size_t elemen
     return (float*)((uint8_t*)p.o + element_offset * (p.o_bf16 ? 2u : 4u));
 }
 
+// lse_row (may be null): receives m_used c + log2(total + 1e-6 f), so that the normalised probability of a key
+// with raw score s is exp2(s c - lse) -- what a backward pass needs to rebuild P without the row's other keys.
 template <int NO>
-__device__ __forceinline__ void store_output(float* o_row, uint32_t as_bf16, f32x16 (&o)[NO], float m_used,
-                                             float m_true, float total, float c, uint32_t half) {
+__device__ __forceinline__ void store_output(float* o_row, uint32_t as_bf16, float* lse_row, f32x16 (&o)[NO],
+                                             float m_used, float m_true, float total, float c, uint32_t half) {
     const float f = exp2_fast((m_true - m_used) * c);
     const float inv = 1.0f / (total + 1e-6f * f);
+    if (lse_row != nullptr && half == 0) *lse_row = __builtin_fmaf(m_used, c, __builtin_log2f(total + 1e-6f * f));
     for_each_out_vec<NO>([&](int mt, int ig) {
         const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
                            o[mt][ig * 4 + 3] * inv};
@@ -186,7 +190,8 @@ __device__ __forceinline__ uint32_t partial_offset(int mt, int ig, uint32_t half
 
 template <int BS, int D>
 __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
-                                               uint32_t as_bf16, float c, uint32_t q_in_block, uint32_t half);
+                                               uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
+                                               uint32_t half);
 
 // End of a work item.  Unsplit rows are normalised and stored.  A chunk of a split row writes its
 // partial (unnormalised O, reference maximum, true maximum, sum) and bumps the row's counter; the
@@ -196,11 +201,12 @@ template <int BS, int D>
 __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& w, float* o_row,
                                            f32x16 (&o)[D / 32], const RowState& st, float c,
                                            uint32_t q_in_block, uint32_t half, uint32_t t) {
+    float* const lse_row = p.lse ? p.lse + ((size_t)w.bh * p.nb + w.row) * BS + q_in_block : nullptr;
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;   // floats per partial
     const float total = st.l + __shfl_xor(st.l, 32);
     if (w.nchunks <= 1) {
-        store_output<NO>(o_row, p.o_bf16, o, st.m_used, st.m_true, total, c, half);
+        store_output<NO>(o_row, p.o_bf16, lse_row, o, st.m_used, st.m_true, total, c, half);
         return;
     }
     float* base = p.partials + ((size_t)w.bh * p.n_parts + w.part) * PART;
@@ -226,14 +232,15 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     }
     __syncthreads();
     if (!last_flag) return;
-    merge_partials<BS, D>(base, w.nchunks, o_row, p.o_bf16, c, q_in_block, half);
+    merge_partials<BS, D>(base, w.nchunks, o_row, p.o_bf16, lse_row, c, q_in_block, half);
     if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Merge of the partial records of a split row (run by the chunk that arrived last).
 template <int BS, int D>
 __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
-                                               uint32_t as_bf16, float c, uint32_t q_in_block, uint32_t half) {
+                                               uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
+                                               uint32_t half) {
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -260,7 +267,7 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchun
             for (int e = 0; e < 4; ++e) acc[mt][ig * 4 + e] += coherent_load(src + e) * wgt;
         });
     }
-    store_output<NO>(o_row, as_bf16, acc, m_used, m_true, sum, c, half);
+    store_output<NO>(o_row, as_bf16, lse_row, acc, m_used, m_true, sum, c, half);
 }
 
 template <int D>
@@ -329,6 +336,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
 
     if (count == 0) {
         store_zero_row<D>(o_row, p.o_bf16, half);
+        if (p.lse && half == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
         return;
     }
 
@@ -493,6 +501,7 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_ke
 
     if (count == 0) {
         store_zero_row<D>(o_row, p.o_bf16, half);
+        if (p.lse && half == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
         return;
     }
 
@@ -628,6 +637,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
                         uint32_t head_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
                         float scale) {
     p.q = q; p.k = k; p.v = v; p.o = (float*)o; p.o_bf16 = out_dtype == SFB_BF16 ? 1u : 0u;
+    p.lse = nullptr;
     p.nn_lut = nn_lut; p.mask = mask; p.valid_len = valid_len;
     p.row_order = nullptr; p.items = nullptr; p.counters = nullptr; p.partials = nullptr;
     p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
@@ -671,7 +681,7 @@ extern "C" size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_part
 }
 
 static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const void* k,
-                                             const void* v, void* o, int in_dtype, int out_dtype,
+                                             const void* v, void* o, float* lse, int in_dtype, int out_dtype,
                                              const sfb_uint2* nn_lut, const void* mask,
                                              const int32_t* valid_len, const sfb_work_item* items,
                                              uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
@@ -694,6 +704,7 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
     fill_common(p, q, k, v, o, out_dtype, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
                 1, ctx_blks + blocks, mask_heads, scale);
     p.items = items;
+    p.lse = lse;
     p.n_slots = n_slots; p.n_parts = n_parts; p.heavy = n_heavy;
     const size_t bh = (size_t)batch_dim * head_dim;
     const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
@@ -713,7 +724,7 @@ extern "C" int sfb_fused_attention_scheduled(sfb_stream_t stream, const void* q,
                                              uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                              uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                              uint32_t mask_heads, float scale) {
-    return fused_attention_scheduled(stream, q, k, v, o, in_dtype, SFB_F32, nn_lut, mask, valid_len, items, n_items,
+    return fused_attention_scheduled(stream, q, k, v, o, nullptr, in_dtype, SFB_F32, nn_lut, mask, valid_len, items, n_items,
                                      n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
 }
@@ -727,7 +738,22 @@ extern "C" int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void*
                                                 uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                                 uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                                 uint32_t mask_heads, float scale) {
-    return fused_attention_scheduled(stream, q, k, v, o, in_dtype, out_dtype, nn_lut, mask, valid_len, items, n_items,
+    return fused_attention_scheduled(stream, q, k, v, o, nullptr, in_dtype, out_dtype, nn_lut, mask, valid_len, items, n_items,
                                      n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
+}
+
+extern "C" int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const void* k,
+                                                 const void* v, void* o, float* lse, int in_dtype, int out_dtype,
+                                                 const sfb_uint2* nn_lut, const void* mask,
+                                                 const int32_t* valid_len, const sfb_work_item* items,
+                                                 uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                                 uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                                 uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                                 uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                                 uint32_t mask_heads, float scale) {
+    if (!lse) return SFB_ERR_NULL_POINTER;
+    return fused_attention_scheduled(stream, q, k, v, o, lse, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
+                                     n_items, n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
 }

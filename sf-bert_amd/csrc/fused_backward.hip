@@ -1,0 +1,430 @@
+// Fused backward of the block-sparse attention: dQ, dK, dV from Q, K, V, dO, the forward output O and the
+// forward's row statistics, without P, dP or dS ever reaching memory.  The reference's backward is the unfused
+// sequence TN, NT, softmax gradient, TN, NN over sparse tensors in memory
+// (transformer_attention_optimize.cu:924-965); the arithmetic here is the same (ewops.h:101-124, matmul.h:81-99):
+//     P  = exp2(S c - lse)                  S = Q K^T, lse from the forward (sfb_fused_attention_scheduled_lse)
+//     dV = P^T dO      dP = dO V^T      dS = P (dP - delta) scale      dK = dS^T Q      dQ = dS K
+// with delta_q = sum_d dO_qd O_qd in place of the gradient's sum over the sparse row (equal, since O = P V).
+//
+// Two kernels, both with the tile machinery of the forward kernel (LDS-direct loads into swizzled tiles, see
+// Bf16DirectTiles; k_frag reads a tile row-wise, v_frag reads it transposed):
+//   * dq kernel, one work-group per (batch, head, block-row), a lane owns one query: per key block
+//         S^T = K Q^T, dP^T = V dO^T (row-wise reads of the K and V tiles), dS^T lane-local,
+//         dQ^T += K^T dS^T (transposed read of the K tile);
+//   * dkdv kernel, one work-group per (batch, head, key-block column), a lane owns one key: per query block
+//         S = Q K^T, dP = dO V^T (row-wise reads of the Q and dO tiles; lse and delta per accumulator element),
+//         dV^T += dO^T P, dK^T += Q^T dS (transposed reads of the dO and Q tiles).
+// bf16 tensors, head size 64, block size 32 or 64; fp32 accumulation and fp32 gradients.
+#include "tiles.hip.h"
+
+namespace sfb {
+
+struct BackwardParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* d_out;
+    const float* lse;           // [batch][heads][ctx]
+    const float* delta;         // [batch][heads][ctx]
+    float* dq;
+    float* dk;
+    float* dv;
+    const sfb_uint2* nn_lut;
+    const sfb_uint2* tn_lut;
+    const void* mask;           // block-major keep words, or nullptr
+    const int32_t* valid_len;
+    const sfb_work_item* items; // rank -> chunk of a block-row (dq) / block-column (dkdv), or nullptr: whole rows
+    float* partials;            // partial results of split rows / columns, or nullptr
+    uint32_t ranks, heavy, n_parts;
+    uint32_t batch, heads, nb, blocks, mask_stride;
+    float scale, scale_log2e;
+};
+
+// What a work-group does: key (query) blocks [first, first + count) of the LUT segment of block-row (column)
+// `line`; the result goes to the output rows, or, for a chunk of a split line, to partial record `slot`.
+struct LineWork {
+    uint32_t bh, line, first, count;
+    int32_t slot;   // -1: write the output directly
+    bool valid;
+};
+__device__ __forceinline__ LineWork decode_line_work(const BackwardParams& p, const sfb_uint2* lut) {
+    const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.ranks, p.heavy);
+    LineWork w;
+    w.valid = id.valid;
+    w.bh = id.bh;
+    w.slot = -1;
+    if (p.items) {
+        const sfb_work_item it = p.items[id.rank];
+        w.line = it.row;
+        w.first = it.lut_first;
+        w.count = it.count;
+        if (it.nchunks > 1) w.slot = (int32_t)(it.part + it.chunk);
+    } else {
+        w.line = id.rank;
+        w.first = lut[id.valid ? id.rank : 0u].x;
+        w.count = id.valid ? lut[id.rank].y : 0u;
+    }
+    return w;
+}
+
+// acc element i of tile kt <-> index kt*32 + (i/4)*8 + half*4 + i%4 along the block; chunk u (16 indices) of the
+// packed bf16 operand takes elements i0 .. i0+7 of tile u/2 with i0 = (u%2)*8
+template <int KT>
+__device__ __forceinline__ void pack_chunks(uint32_t (&pk)[KT * 8], const f32x16 (&x)[KT]) {
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) pk[kt * 8 + i / 2] = pack_bf16(x[kt][i], x[kt][i + 1]);
+}
+
+template <int NO>
+__device__ __forceinline__ void store_rows_f32(float* row, const f32x16 (&acc)[NO], uint32_t half) {
+#pragma unroll
+    for (int mt = 0; mt < NO; ++mt)
+#pragma unroll
+        for (int ig = 0; ig < 4; ++ig) {
+            const f32x4 out = {acc[mt][ig * 4 + 0], acc[mt][ig * 4 + 1], acc[mt][ig * 4 + 2], acc[mt][ig * 4 + 3]};
+            *(f32x4*)(row + mt * 32 + ig * 8 + half * 4) = out;
+        }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dQ: row owner
+// ------------------------------------------------------------------------------------------------
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 2) void attention_dq_kernel(BackwardParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+
+    const LineWork work = decode_line_work(p, p.nn_lut);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t r = work.line;
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t row_bytes = p.heads * D * 2;
+    const uint32_t off = __builtin_amdgcn_readfirstlane(work.first), count = __builtin_amdgcn_readfirstlane(work.count);
+    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+
+    f32x16 dq_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dq_acc[n][i] = 0.f;
+
+    if (count > 0) {
+        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
+        const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
+        const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
+        const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+        const uint32_t lds0 = T::lds_address(smem);
+        const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
+        const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+        const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+        const float c = p.scale_log2e;
+
+        bf16x8 qf[KS], dof[KS];
+        T::load_q(qf, (const __bf16*)p.q + my_row, half);
+        T::load_q(dof, (const __bf16*)p.d_out + my_row, half);
+        const size_t stat = ((size_t)work.bh * p.nb + r) * BS + q_in_block;
+        const float lse = p.lse[stat], delta = p.delta[stat];
+
+        auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
+            const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
+            return u;
+        };
+        auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
+            T::load_tile(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+            T::load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+        };
+        sfb_uint2 e = uniform(p.nn_lut[off]);
+        fetch(e, 0);
+        for (uint32_t j = 0; j < count; ++j) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();   // tiles of block j have landed for every wave; every wave is done with block j-1
+            const sfb_uint2 e_next = uniform(p.nn_lut[off + (j + 1 < count ? j + 1 : j)]);
+            fetch(e_next, (j + 1) & 1);
+            const uint8_t* k_tile = smem + (j & 1) * TILE;
+            const uint8_t* v_tile = smem + (2 + (j & 1)) * TILE;
+
+            f32x16 s[KT], dp[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { s[kt][i] = 0.f; dp[kt][i] = 0.f; }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_tile, k_lane, kt, ks), qf[ks], s[kt], 0, 0, 0);
+                    dp[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(v_tile, k_lane, kt, ks), dof[ks], dp[kt], 0, 0, 0);
+                }
+            }
+            if (MASKED) {
+                const int limit = valid - (int)(e.y * BS);
+                if ((mask != nullptr) || (limit < BS))
+                    apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)e.x * BS + q_in_block, limit), half);
+            }
+            // dS^T for this lane's query: P (dP - delta) scale; a masked score is -3e38, its probability an exact 0
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float prob = exp2_fast(__builtin_fmaf(s[kt][i], c, -lse));
+                    s[kt][i] = prob * (dp[kt][i] - delta) * p.scale;
+                }
+            uint32_t pk[KT * 8];
+            pack_chunks<KT>(pk, s);
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
+                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    dq_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(k_tile, v_lane, mt, u), bfrag, dq_acc[mt], 0, 0, 0);
+            }
+            e = e_next;
+        }
+    }
+    if (work.slot < 0) store_rows_f32<NO>(p.dq + my_row, dq_acc, half);
+    else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK, dV: column owner
+// ------------------------------------------------------------------------------------------------
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 2) void attention_dkdv_kernel(BackwardParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // Q0 Q1 dO0 dO1
+
+    const LineWork work = decode_line_work(p, p.tn_lut);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t col = work.line;
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t kn = lane & 31, half = lane >> 5;
+    const uint32_t key_in_block = wave * 32 + kn;
+    const uint32_t row_bytes = p.heads * D * 2;
+    const uint32_t off = __builtin_amdgcn_readfirstlane(work.first), count = __builtin_amdgcn_readfirstlane(work.count);
+    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, D);
+
+    f32x16 dk_acc[NO], dv_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { dk_acc[n][i] = 0.f; dv_acc[n][i] = 0.f; }
+
+    if (count > 0) {
+        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
+        const uint8_t* const q_base = (const uint8_t*)p.q + bh_bytes;
+        const uint8_t* const do_base = (const uint8_t*)p.d_out + bh_bytes;
+        const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+        const uint32_t lds0 = T::lds_address(smem);
+        const uint32_t k_lane = T::k_lane_base(kn, half), v_lane = T::v_lane_base(lane);
+        const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+        const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+        const bool key_valid = (int)(col * BS + key_in_block) < valid;
+        const float c = p.scale_log2e;
+        const float* lse_bh = p.lse + (size_t)work.bh * L;
+        const float* delta_bh = p.delta + (size_t)work.bh * L;
+
+        bf16x8 kf[KS], vf[KS];   // this lane's key as the B operand of both score-like products
+        T::load_q(kf, (const __bf16*)p.k + my_row, half);
+        T::load_q(vf, (const __bf16*)p.v + my_row, half);
+
+        auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
+            const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
+            return u;
+        };
+        auto fetch = [&](const sfb_uint2 e, uint32_t buf) {   // e = {block id, row block}
+            T::load_tile(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+            T::load_tile(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+        };
+        sfb_uint2 e = uniform(p.tn_lut[off]);
+        fetch(e, 0);
+        for (uint32_t j = 0; j < count; ++j) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            const sfb_uint2 e_next = uniform(p.tn_lut[off + (j + 1 < count ? j + 1 : j)]);
+            fetch(e_next, (j + 1) & 1);
+            const uint8_t* q_tile = smem + (j & 1) * TILE;
+            const uint8_t* do_tile = smem + (2 + (j & 1)) * TILE;
+
+            // S[query][key], dP[query][key]: element i of tile kt is query kt*32 + (i/4)*8 + half*4 + i%4, key = lane's
+            f32x16 s[KT], dp[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { s[kt][i] = 0.f; dp[kt][i] = 0.f; }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(q_tile, k_lane, kt, ks), kf[ks], s[kt], 0, 0, 0);
+                    dp[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(do_tile, k_lane, kt, ks), vf[ks], dp[kt], 0, 0, 0);
+                }
+            }
+            const float* lse_blk = lse_bh + (size_t)e.y * BS;
+            const float* delta_blk = delta_bh + (size_t)e.y * BS;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ig = 0; ig < 4; ++ig) {
+                    const uint32_t q0 = kt * 32 + ig * 8 + half * 4;
+                    const f32x4 lse4 = *(const f32x4*)(lse_blk + q0), delta4 = *(const f32x4*)(delta_blk + q0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int i = ig * 4 + x;
+                        float prob = exp2_fast(__builtin_fmaf(s[kt][i], c, -lse4[x]));
+                        if (MASKED) {
+                            bool keep = key_valid;
+                            if (mask != nullptr) {
+                                const size_t word = (size_t)e.x * BS + q0 + x;
+                                const uint64_t bits = (BS == 64) ? ((const uint64_t*)mask)[word] : ((const uint32_t*)mask)[word];
+                                keep = keep && ((bits >> key_in_block) & 1u);
+                            }
+                            prob = keep ? prob : 0.f;
+                        }
+                        s[kt][i] = prob;
+                        dp[kt][i] = prob * (dp[kt][i] - delta4[x]) * p.scale;
+                    }
+                }
+            uint32_t pk_p[KT * 8], pk_ds[KT * 8];
+            pack_chunks<KT>(pk_p, s);
+            pack_chunks<KT>(pk_ds, dp);
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                const u32x4 pb = {pk_p[u * 4 + 0], pk_p[u * 4 + 1], pk_p[u * 4 + 2], pk_p[u * 4 + 3]};
+                const u32x4 db = {pk_ds[u * 4 + 0], pk_ds[u * 4 + 1], pk_ds[u * 4 + 2], pk_ds[u * 4 + 3]};
+                const bf16x8 pfrag = __builtin_bit_cast(bf16x8, pb), dsfrag = __builtin_bit_cast(bf16x8, db);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt) {
+                    dv_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(do_tile, v_lane, mt, u), pfrag, dv_acc[mt], 0, 0, 0);
+                    dk_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(q_tile, v_lane, mt, u), dsfrag, dk_acc[mt], 0, 0, 0);
+                }
+            }
+            e = e_next;
+        }
+    }
+    if (work.slot < 0) {
+        store_rows_f32<NO>(p.dk + my_row, dk_acc, half);
+        store_rows_f32<NO>(p.dv + my_row, dv_acc, half);
+    } else {   // partial record of a split column: dK rows, then dV rows
+        float* part = p.partials + (((size_t)work.bh * p.n_parts + work.slot) * 2 * BS + key_in_block) * D;
+        store_rows_f32<NO>(part, dk_acc, half);
+        store_rows_f32<NO>(part + (size_t)BS * D, dv_acc, half);
+    }
+}
+
+// Sum of the partial records of split block-rows (TENSORS = 1: dQ) or block-columns (TENSORS = 2: dK, dV), in chunk
+// order, by the work-group of the line's first chunk; all other work-groups leave at once.  A separate launch: the
+// partials are complete when it starts, nobody has to wait for anybody.
+template <int BS, int D, int TENSORS>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(float* out0, float* out1, const float* partials,
+                                                              const sfb_work_item* items, uint32_t n_parts,
+                                                              uint32_t heads, uint32_t ctx) {
+    const sfb_work_item it = items[blockIdx.x];
+    if (it.nchunks <= 1 || it.chunk != 0) return;
+    const uint32_t bh = blockIdx.y, b = bh / heads, h = bh % heads;
+    constexpr int VECS = BS * D / 4;
+    for (int tensor = 0; tensor < TENSORS; ++tensor) {
+        float* out = tensor == 0 ? out0 : out1;
+        for (uint32_t vec = threadIdx.x; vec < VECS; vec += 256) {
+            const uint32_t row = vec / (D / 4), c4 = vec % (D / 4);
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            for (uint32_t ch = 0; ch < it.nchunks; ++ch)
+                sum += *(const f32x4*)(partials + ((((size_t)bh * n_parts + it.part + ch) * TENSORS + tensor) * BS + row) * D + c4 * 4);
+            *(f32x4*)(out + token_offset(b, it.row * BS + row, h, ctx, heads, D) + c4 * 4) = sum;
+        }
+    }
+}
+
+template <int BS>
+static int launch_backward(hipStream_t stream, const BackwardParams& p, const sfb_work_item* row_items,
+                           uint32_t n_row_items, uint32_t n_row_heavy, uint32_t n_row_parts,
+                           const sfb_work_item* col_items, uint32_t n_col_items, uint32_t n_col_heavy,
+                           uint32_t n_col_parts, float* row_partials, float* col_partials) {
+    const bool masked = p.mask != nullptr || p.valid_len != nullptr;
+    const uint32_t groups = bh_groups(p.batch * p.heads);
+    BackwardParams rows = p, cols = p;
+    rows.items = row_items; rows.ranks = row_items ? n_row_items : p.nb; rows.heavy = row_items ? n_row_heavy : 0;
+    rows.n_parts = n_row_parts; rows.partials = row_partials;
+    cols.items = col_items; cols.ranks = col_items ? n_col_items : p.nb; cols.heavy = col_items ? n_col_heavy : 0;
+    cols.n_parts = n_col_parts; cols.partials = col_partials;
+    clear_stale_error();
+    if (masked) {
+        attention_dkdv_kernel<BS, 64, true><<<dim3(groups * 8u * cols.ranks), dim3(BS * 2), 0, stream>>>(cols);
+        attention_dq_kernel<BS, 64, true><<<dim3(groups * 8u * rows.ranks), dim3(BS * 2), 0, stream>>>(rows);
+    } else {
+        attention_dkdv_kernel<BS, 64, false><<<dim3(groups * 8u * cols.ranks), dim3(BS * 2), 0, stream>>>(cols);
+        attention_dq_kernel<BS, 64, false><<<dim3(groups * 8u * rows.ranks), dim3(BS * 2), 0, stream>>>(rows);
+    }
+    if (col_items && n_col_parts)
+        reduce_partials_kernel<BS, 64, 2><<<dim3(n_col_items, p.batch * p.heads), dim3(256), 0, stream>>>(
+            p.dk, p.dv, col_partials, col_items, n_col_parts, p.heads, p.nb * BS);
+    if (row_items && n_row_parts)
+        reduce_partials_kernel<BS, 64, 1><<<dim3(n_row_items, p.batch * p.heads), dim3(256), 0, stream>>>(
+            p.dq, nullptr, row_partials, row_items, n_row_parts, p.heads, p.nb * BS);
+    return launch_status();
+}
+
+}  // namespace sfb
+
+extern "C" size_t sfb_backward_workspace_bytes(uint32_t n_row_parts, uint32_t n_col_parts, uint32_t batch_dim,
+                                               uint32_t head_dim, uint32_t block_size, uint32_t state_dim) {
+    const size_t record = (size_t)block_size * state_dim * sizeof(float);
+    return (size_t)batch_dim * head_dim * ((size_t)n_row_parts + 2 * (size_t)n_col_parts) * record;
+}
+
+extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, const void* k, const void* v,
+                                            const float* o, const void* d_out, const float* lse, float* delta,
+                                            float* dq, float* dk, float* dv, int dtype, const sfb_uint2* nn_lut,
+                                            const sfb_uint2* tn_lut, const void* mask, const int32_t* valid_len,
+                                            const sfb_work_item* row_items, uint32_t n_row_items,
+                                            uint32_t n_row_heavy, uint32_t n_row_parts,
+                                            const sfb_work_item* col_items, uint32_t n_col_items,
+                                            uint32_t n_col_heavy, uint32_t n_col_parts, void* workspace,
+                                            size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                            uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                            uint32_t state_dim, uint32_t mask_heads, float scale) {
+    using namespace sfb;
+    if (!q || !k || !v || !o || !d_out || !lse || !delta || !dq || !dk || !dv || !nn_lut || !tn_lut)
+        return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_BF16) return SFB_ERR_DTYPE;   // fp32 tensors take the unfused sequence
+    if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
+    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
+    if (!batch_dim || !ctx_blks || !head_dim || !mask_heads) return SFB_ERR_SHAPE;
+    if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
+    if ((row_items && (!n_row_items || n_row_heavy >= n_row_items)) ||
+        (col_items && (!n_col_items || n_col_heavy >= n_col_items)))
+        return SFB_ERR_SHAPE;
+    const uint64_t most = (row_items ? n_row_items : ctx_blks) > (col_items ? n_col_items : ctx_blks)
+                              ? (row_items ? n_row_items : ctx_blks) : (col_items ? n_col_items : ctx_blks);
+    if ((uint64_t)batch_dim * head_dim * most > 0x7fffffffull / 64) return SFB_ERR_SHAPE;
+    if (!row_items) n_row_parts = 0;
+    if (!col_items) n_col_parts = 0;
+    const size_t need = sfb_backward_workspace_bytes(n_row_parts, n_col_parts, batch_dim, head_dim, block_size, state_dim);
+    if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u))) return SFB_ERR_WORKSPACE;
+    const uintptr_t align = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_out |
+                            (uintptr_t)lse | (uintptr_t)delta | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv;
+    if (align & 15u) return SFB_ERR_ALIGNMENT;
+    const int rc = sfb_row_dot(stream, delta, d_out, o, dtype, batch_dim, ctx_blks * block_size, head_dim, state_dim);
+    if (rc != SFB_OK) return rc;
+    BackwardParams p = {};
+    p.q = q; p.k = k; p.v = v; p.d_out = d_out; p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
+    p.nn_lut = nn_lut; p.tn_lut = tn_lut; p.mask = mask; p.valid_len = valid_len;
+    p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
+    p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
+    p.scale = scale; p.scale_log2e = scale * kLog2e;
+    float* row_partials = (float*)workspace;
+    float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * state_dim;
+    hipStream_t s = (hipStream_t)stream;
+    if (block_size == 64)
+        return launch_backward<64>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items,
+                                   n_col_heavy, n_col_parts, row_partials, col_partials);
+    return launch_backward<32>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items,
+                               n_col_heavy, n_col_parts, row_partials, col_partials);
+}

@@ -1,0 +1,96 @@
+"""Fused backward of the attention (two kernels, nothing sparse in memory) and the forward's log-sum-exp output
+against the CPU oracle's backward chain, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as orc
+from gpu_common import PATTERNS, TOL_BF16, dev, qkv, rel_err
+from sfb import sfb
+
+pytestmark = pytest.mark.gpu
+
+
+def forward(q, k, v, luts, bs, scale, mask=None, valid=None, max_blocks=4):
+    B, L, H, d = q.shape
+    sched = sfb.build_schedule(luts["nn_lut"], L // bs, max_blocks)
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    return sfb.fused_attention_forward_lse(q, k, v, sfb.to_device(luts["nn_lut"]), sfb.to_device(sched["items"]), sched,
+                                           ws, bs, luts["blocks"], scale, mask=mask, valid_len=valid)
+
+
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("pattern,masked", [("causal", True), ("bigbird", False), ("bigbird", True), ("strided", False)])
+def test_fused_backward_matches_oracle(pattern, masked, bs):
+    nb, B, H, d = 16, 2, 3, 64
+    lay = PATTERNS[pattern](nb).copy()
+    if pattern == "bigbird":
+        lay[5] = 0      # a block-row without blocks
+        lay[:, 9] = 0   # a block-column without blocks
+    luts = sfb.build_luts(lay)
+    mask = valid = None
+    if masked:
+        if pattern == "causal":
+            mask = sfb.pack_mask(sfb.element_mask(luts["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG))
+        else:
+            keep = (np.random.default_rng(bs).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
+            mask = sfb.pack_mask(keep)
+        valid = np.array([nb * bs, nb * bs - bs - 7], np.int32)
+    Q, K, V = qkv(B, nb * bs, H, d, seed=200 + bs, bf16=True)
+    dO = orc.round_bf16(orc.fill_normal((B, nb * bs, H, d), 210))
+    dQ, dK, dV, P = orc.attention_backward(Q, K, V, dO, luts, bs, 0.125, mask=mask, valid_len=valid)
+    q, k, v, do = (dev(x, True) for x in (Q, K, V, dO))
+    m = None if mask is None else sfb.to_device(mask)
+    vl = None if valid is None else sfb.to_device(valid)
+    o, lse = forward(q, k, v, luts, bs, 0.125, mask=m, valid=vl)
+    want_o = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, mask=mask, valid_len=valid)
+    assert rel_err(o.cpu().numpy(), want_o) <= TOL_BF16
+
+    # the log-sum-exp rebuilds the oracle's probabilities: P = exp2(S scale log2e - lse)
+    S = orc.sdd_nt(Q, K, luts["nt_lut"], bs)
+    lse_np = lse.cpu().numpy()
+    worst = 0.0
+    for blk, (r, _) in enumerate(luts["nt_lut"]):
+        rebuilt = np.exp2(S[:, :, blk] * (0.125 * np.log2(np.e)) - lse_np[:, :, r * bs:(r + 1) * bs, None])
+        kept = P[:, :, blk] > 0
+        worst = max(worst, float(np.abs(np.where(kept, rebuilt - P[:, :, blk], 0)).max()))
+    # the bf16 kernel sums the probabilities as it uses them, rounded to bf16: its denominator carries that noise
+    assert worst <= 2e-3 * P.max()
+
+    nn, tn = sfb.to_device(luts["nn_lut"]), sfb.to_device(luts["tn_lut"])
+    results = []
+    for max_blocks in (None, 3, 100):   # whole lines in index order; lines cut into chunks of 3 blocks; sorted only
+        rs = cs = None
+        if max_blocks:
+            rs, cs = sfb.build_schedule(luts["nn_lut"], nb, max_blocks), sfb.build_schedule(luts["tn_lut"], nb, max_blocks)
+            rs["items_dev"], cs["items_dev"] = sfb.to_device(rs["items"]), sfb.to_device(cs["items"])
+            assert (max_blocks == 3) == (rs["n_parts"] > 0 and cs["n_parts"] > 0)
+        dq, dk, dv = sfb.fused_attention_backward(q, k, v, o, do, lse, nn, tn, bs, luts["blocks"], 0.125, mask=m,
+                                                  valid_len=vl, row_sched=rs, col_sched=cs)
+        torch.cuda.synchronize()
+        for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+            got = got.cpu().numpy()
+            assert np.isfinite(got).all()
+            assert rel_err(got, want) <= TOL_BF16, (name, max_blocks)
+        if pattern == "bigbird":
+            assert (dq.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
+            assert (dk.cpu().numpy()[:, 9 * bs:10 * bs] == 0).all() and (dv.cpu().numpy()[:, 9 * bs:10 * bs] == 0).all()
+        results.append((dq, dk, dv))
+    # the order in which whole lines are handed out does not change a bit; and a second call with split lines
+    # gives the same bits as the first (the partial records are added in chunk order)
+    for x, y in zip(results[0], results[2]):
+        assert torch.equal(x, y)
+    rs, cs = sfb.build_schedule(luts["nn_lut"], nb, 3), sfb.build_schedule(luts["tn_lut"], nb, 3)
+    rs["items_dev"], cs["items_dev"] = sfb.to_device(rs["items"]), sfb.to_device(cs["items"])
+    again = sfb.fused_attention_backward(q, k, v, o, do, lse, nn, tn, bs, luts["blocks"], 0.125, mask=m, valid_len=vl,
+                                         row_sched=rs, col_sched=cs)
+    for x, y in zip(results[1], again):
+        assert torch.equal(x, y)
+
+
+def test_fused_backward_rejects_fp32():
+    q = torch.zeros((1, 64, 1, 64), device="cuda")
+    lut = sfb.to_device(np.zeros((2, 2), np.uint32))
+    with pytest.raises(sfb.SfbError) as e:
+        sfb.fused_attention_backward(q, q, q, q, q, torch.zeros((1, 1, 64), device="cuda"), lut, lut, 64, 1, 0.125)
+    assert e.value.status == 5
