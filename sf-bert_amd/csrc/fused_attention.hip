@@ -417,8 +417,13 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
             const sfb_uint2 here = {(uint32_t)__builtin_amdgcn_readlane(entries.x, j - win),
                                     (uint32_t)__builtin_amdgcn_readlane(entries.y, j - win)};
             const int limit = valid - (int)(here.y * BS);
-            if ((mask != nullptr) || (limit < BS))
-                apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit), half);
+            if ((mask != nullptr) || (limit < BS)) {
+                // most blocks of a causal or padded layout keep every key: the per-element selection is only done
+                // when some lane of the wave has a key to drop
+                const uint64_t keep = load_keep_word<BS>(mask, (size_t)here.x * BS + q_in_block, limit);
+                constexpr uint64_t kAll = BS == 64 ? ~0ull : 0xffffffffull;
+                if (__builtin_amdgcn_ballot_w64((keep & kAll) != kAll) != 0) apply_keep<KT>(s, keep, half);
+            }
         }
         const float mloc = block_row_max<KT>(s);
         st.m_true = fmaxf(st.m_true, mloc);
