@@ -94,3 +94,32 @@ def test_fused_backward_rejects_fp32():
     with pytest.raises(sfb.SfbError) as e:
         sfb.fused_attention_backward(q, q, q, q, q, torch.zeros((1, 1, 64), device="cuda"), lut, lut, 64, 1, 0.125)
     assert e.value.status == 5
+
+
+def test_fused_backward_full_size_identities():
+    """C4 workload (BigBird B4 H12 L4096, 622 blocks), scheduled with split global rows and columns: O is linear in V
+    and S is bilinear in Q, K, hence <dV, V> = <dO, O> and <dQ, Q> = <dK, K>; every gradient row is written."""
+    import bench
+    pattern, B, H, L, d, bs, _ = bench.WORKLOADS["c4"]
+    nb = L // bs
+    luts = sfb.build_luts(bench.make_layout(sfb, pattern, nb))
+    torch.manual_seed(5)
+    q, k, v, do = (torch.randn((B, L, H, d), device="cuda").to(torch.bfloat16) for _ in range(4))
+    o, lse = forward(q, k, v, luts, bs, 0.125, max_blocks=16)
+    rs, cs = sfb.build_schedule(luts["nn_lut"], nb, 16), sfb.build_schedule(luts["tn_lut"], nb, 16)
+    assert rs["n_parts"] > 0 and cs["n_parts"] > 0
+    rs["items_dev"], cs["items_dev"] = sfb.to_device(rs["items"]), sfb.to_device(cs["items"])
+    dq, dk, dv = sfb.fused_attention_backward(q, k, v, o, do, lse, sfb.to_device(luts["nn_lut"]),
+                                              sfb.to_device(luts["tn_lut"]), bs, luts["blocks"], 0.125, row_sched=rs,
+                                              col_sched=cs)
+    torch.cuda.synchronize()
+    dot = lambda a, b: float((a.double() * b.double()).sum())
+    dv_v, do_o = dot(dv, v), dot(do, o)
+    dq_q, dk_k = dot(dq, q), dot(dk, k)
+    scale_v = float((dv.double() * v.double()).abs().sum())
+    scale_q = float((dq.double() * q.double()).abs().sum())
+    # P is rounded to bf16 inside both kernels and O inside the forward: the identities hold to that rounding
+    assert abs(dv_v - do_o) <= 2e-3 * scale_v
+    assert abs(dq_q - dk_k) <= 2e-3 * scale_q
+    for g in (dq, dk, dv):
+        assert torch.isfinite(g).all() and float(g.abs().amax(dim=(0, 2, 3)).min()) > 0
