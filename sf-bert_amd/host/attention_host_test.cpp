@@ -5,7 +5,8 @@
 // reference's timing harnesses it checks results: all-ones Q, K (the reference's inputs,
 // fixed_fusion_test.cu:263-268) give uniform probabilities in closed form, and on random inputs the
 // fused and unfused paths must agree; the backward stages (bst_sgemm_xn with TN_OP, BlocksparseMaskedSoftmaxGrad)
-// are checked through the inner-product identities of a linear and a bilinear map.  Exit code 0 = all passed.
+// are checked through the inner-product identities of a linear and a bilinear map, and so is the fused training pair
+// (sfb_fused_attention_scheduled_lse, sfb_fused_attention_backward).  Exit code 0 = all passed.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -189,7 +190,81 @@ int main() {
         if (!(std::fabs(dq_q - dk_k) <= 1e-4 * dq_abs)) ++failures;
     }
 
-    // ---- 4. a block size the kernels do not implement is an error, not a silent no-op ----
+    // ---- 4. training pair of the fused path on bf16 tensors: forward with log-sum-exp, fused backward ----
+    // the same identities, and agreement of dV with the unfused sequence above (same P up to bf16 rounding)
+    {
+        const size_t n = tokens * state;
+        bhalf *q16 = nullptr, *k16 = nullptr, *v16 = nullptr, *do16 = nullptr;
+        float *d_do = nullptr, *o = nullptr, *lse = nullptr, *delta = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr;
+        for (bhalf** ptr : {&q16, &k16, &v16, &do16}) HIP_OK(hipMalloc((void**)ptr, n * sizeof(bhalf)));
+        for (float** ptr : {&d_do, &o, &dq, &dk, &dv}) HIP_OK(hipMalloc((void**)ptr, n * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&lse, (size_t)batch_dim * heads_ * seq_len * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&delta, (size_t)batch_dim * heads_ * seq_len * sizeof(float)));
+        std::vector<float> d_out(n);
+        for (size_t i = 0; i < n; ++i) d_out[i] = (rand() % 2001 - 1000) * 1e-3f;
+        HIP_OK(hipMemcpy(d_do, d_out.data(), n * sizeof(float), hipMemcpyHostToDevice));
+        int rc = sfb_cast_f32_bf16(stream, q16, d_q, n);
+        rc = rc ? rc : sfb_cast_f32_bf16(stream, k16, d_k, n);
+        rc = rc ? rc : sfb_cast_f32_bf16(stream, v16, d_v, n);
+        rc = rc ? rc : sfb_cast_f32_bf16(stream, do16, d_do, n);
+        // schedules over the NN table (rows) and the TN table (columns), lines longer than 2 blocks split
+        std::vector<uint2> tn_lut(ctx_blks + blocks);
+        sfb_build_tn_lut((sfb_uint2*)tn_lut.data(), (const sfb_uint2*)nt_lut.data(), blocks, ctx_blks, nullptr);
+        uint2* d_tn = upload(tn_lut);
+        struct Sched { std::vector<sfb_work_item> items; uint32_t n = 0, heavy = 0, slots = 0, parts = 0; sfb_work_item* dev = nullptr; };
+        Sched rows, cols;
+        const sfb_uint2* tables[2] = {(const sfb_uint2*)nn_lut.data(), (const sfb_uint2*)tn_lut.data()};
+        Sched* scheds[2] = {&rows, &cols};
+        for (int i = 0; i < 2; ++i) {
+            Sched& sc = *scheds[i];
+            sfb_build_schedule(nullptr, &sc.n, &sc.heavy, &sc.slots, &sc.parts, tables[i], ctx_blks, 2);
+            sc.items.resize(sc.n);
+            sfb_build_schedule(sc.items.data(), &sc.n, &sc.heavy, &sc.slots, &sc.parts, tables[i], ctx_blks, 2);
+            sc.dev = upload(sc.items);
+        }
+        size_t fwd_bytes = sfb_schedule_workspace_bytes(rows.slots, rows.parts, batch_dim, heads_, blk_size_, head_state_);
+        size_t bwd_bytes = sfb_backward_workspace_bytes(rows.parts, cols.parts, batch_dim, heads_, blk_size_, head_state_);
+        void *fwd_ws = nullptr, *bwd_ws = nullptr;
+        HIP_OK(hipMalloc(&fwd_ws, fwd_bytes + 256));
+        HIP_OK(hipMemset(fwd_ws, 0, fwd_bytes + 256));
+        HIP_OK(hipMalloc(&bwd_ws, bwd_bytes + 256));
+        rc = rc ? rc : sfb_fused_attention_scheduled_lse(stream, q16, k16, v16, o, lse, SFB_BF16, SFB_F32,
+                                                         (const sfb_uint2*)d_nn, d_mask_np, nullptr, rows.dev, rows.n,
+                                                         rows.heavy, rows.slots, rows.parts, fwd_ws, fwd_bytes + 256,
+                                                         blk_size_, blocks, batch_dim, ctx_blks, heads_, head_state_, 1,
+                                                         scale);
+        rc = rc ? rc : sfb_fused_attention_backward(stream, q16, k16, v16, o, do16, lse, delta, dq, dk, dv, SFB_BF16,
+                                                    (const sfb_uint2*)d_nn, (const sfb_uint2*)d_tn, d_mask_np, nullptr,
+                                                    rows.dev, rows.n, rows.heavy, rows.parts, cols.dev, cols.n,
+                                                    cols.heavy, cols.parts, bwd_ws, bwd_bytes + 256, blk_size_, blocks,
+                                                    batch_dim, ctx_blks, heads_, head_state_, 1, scale);
+        if (rc != SFB_OK) {
+            std::fprintf(stderr, "fused training pair failed: %s\n", sfb_status_string(rc));
+            return 1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<float> h_o(n), h_dq(n), h_dk(n), h_dv(n);
+        HIP_OK(hipMemcpy(h_o.data(), o, n * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(h_dq.data(), dq, n * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(h_dk.data(), dk, n * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(h_dv.data(), dv, n * sizeof(float), hipMemcpyDeviceToHost));
+        auto bf = [](float x) {   // the value the device sees: rounded to bf16, nearest even
+            uint32_t u; std::memcpy(&u, &x, 4);
+            u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+            float y; std::memcpy(&y, &u, 4); return y;
+        };
+        double dv_v = 0, do_o = 0, dq_q = 0, dk_k = 0, abs_v = 0, abs_q = 0;
+        for (size_t i = 0; i < n; ++i) {
+            dv_v += (double)h_dv[i] * bf(v[i]);  do_o += (double)bf(d_out[i]) * h_o[i];
+            dq_q += (double)h_dq[i] * bf(q[i]);  dk_k += (double)h_dk[i] * bf(k[i]);
+            abs_v += std::fabs((double)h_dv[i] * bf(v[i]));  abs_q += std::fabs((double)h_dq[i] * bf(q[i]));
+        }
+        std::printf("fused backward: <dV,V> = %.5f, <dO,O> = %.5f; <dQ,Q> = %.5f, <dK,K> = %.5f\n", dv_v, do_o, dq_q, dk_k);
+        if (!(std::fabs(dv_v - do_o) <= 2e-3 * abs_v)) ++failures;
+        if (!(std::fabs(dq_q - dk_k) <= 2e-3 * abs_q)) ++failures;
+    }
+
+    // ---- 5. a block size the kernels do not implement is an error, not a silent no-op ----
     if (bst_sgemm_nt(stream, d_nt, d_q, d_k, d_s, 16, blocks, batch_dim, ctx_blks, ctx_blks, heads_, head_state_, 1,
                      blocks) || sfb_host::last_status() != SFB_ERR_BLOCK_SIZE)
         ++failures;
