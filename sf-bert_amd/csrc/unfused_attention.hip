@@ -858,25 +858,43 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_tn_kernel(DsdParams p) {
     } else {
         // generic path: fp32 MFMA (k = 2 per step, one element per lane and operand); the X row block is staged
         // in LDS as fp32, the sparse block is read from memory, 32 consecutive keys per half-wave
+        // The next block's X tile and this lane's column of the next sparse block wait in registers while the
+        // current block is multiplied.
         float* x_lds = (float*)smem;
-        for (uint32_t j = 0; j < count; ++j) {
+        constexpr int XV = D / 8;   // float4 of the X tile per thread: BS * D / 4 over BS * 2 threads
+        f32x4 xr[XV];
+        float a_cur[BS / 2], a_next[BS / 2];
+        auto fetch_block = [&](uint32_t j, float (&adst)[BS / 2]) {
             const sfb_uint2 e = lut[off + j];
             const TB* x_blk = X + token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
             const TA* a_blk = A + (size_t)e.x * BS * BS;
-            for (uint32_t cid = t; cid < BS * (D / 4); cid += BS * 2) {
-                const uint32_t row = cid / (D / 4), cc = cid % (D / 4);
-                *(f32x4*)(x_lds + row * X_STRIDE + cc * 4) = Elem<TB>::load4(x_blk + (size_t)row * row_stride + cc * 4);
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                const uint32_t cid = i * BS * 2 + t, row = cid / (D / 4), cc = cid % (D / 4);
+                xr[i] = Elem<TB>::load4(x_blk + (size_t)row * row_stride + cc * 4);
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < BS / 2; ++s2) adst[s2] = Elem<TA>::load(a_blk + (size_t)(2 * s2 + half) * BS + key_in_block);
+        };
+        if (count > 0) fetch_block(0, a_cur);
+        for (uint32_t j = 0; j < count; ++j) {
+#pragma unroll
+            for (int i = 0; i < XV; ++i) {
+                const uint32_t cid = i * BS * 2 + t, row = cid / (D / 4), cc = cid % (D / 4);
+                *(f32x4*)(x_lds + row * X_STRIDE + cc * 4) = xr[i];
             }
             __syncthreads();
-#pragma unroll 4
+            if (j + 1 < count) fetch_block(j + 1, a_next);
+#pragma unroll
             for (int s2 = 0; s2 < BS / 2; ++s2) {
                 const uint32_t q = 2 * s2 + half;
-                const float av = Elem<TA>::load(a_blk + (size_t)q * BS + key_in_block);
 #pragma unroll
                 for (int mt = 0; mt < NO; ++mt)
-                    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(x_lds[q * X_STRIDE + mt * 32 + kn], av, acc[mt], 0, 0, 0);
+                    acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(x_lds[q * X_STRIDE + mt * 32 + kn], a_cur[s2], acc[mt], 0, 0, 0);
             }
             __syncthreads();
+#pragma unroll
+            for (int s2 = 0; s2 < BS / 2; ++s2) a_cur[s2] = a_next[s2];
         }
     }
     // accumulator element i of column tile mt is column mt*32 + (i/4)*8 + half*4 + i%4 of this lane's key row;
@@ -1016,28 +1034,40 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
             for (int x = 0; x < 2 * PU; ++x) pc[x] = pn[x];
         }
     } else {
-        for (uint32_t j = 0; j < count; ++j) {
+        // fp32 V: the tile goes through registers into LDS; the next block's V tile and P values are fetched while
+        // this block is multiplied
+        float* v_lds = (float*)smem;
+        typename TF::Regs gv;
+        f32x4 pc[KT][4], pn[KT][4];
+        auto fetch_block = [&](uint32_t j, f32x4 (&pdst)[KT][4]) {
             const sfb_uint2 e = lut[off + j];
-            const size_t base = token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
+            TF::fetch(gv, (const float*)V, token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D), row_stride, t);
             const TP* p_row = P + ((size_t)e.x * BS + q_in_block) * BS;
-            float* v_lds = (float*)smem;
-            typename TF::Regs gv;
-            TF::fetch(gv, (const float*)V, base, row_stride, t);
-            TF::template stage<TF::V_STRIDE>(v_lds, gv, t);
-            __syncthreads();
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int ig = 0; ig < 4; ++ig) {
-                    const f32x4 pv = Elem<TP>::load4(p_row + kt * 32 + ig * 8 + half * 4);
+                for (int ig = 0; ig < 4; ++ig) pdst[kt][ig] = Elem<TP>::load4(p_row + kt * 32 + ig * 8 + half * 4);
+        };
+        if (count > 0) fetch_block(0, pc);
+        for (uint32_t j = 0; j < count; ++j) {
+            TF::template stage<TF::V_STRIDE>(v_lds, gv, t);
+            __syncthreads();
+            if (j + 1 < count) fetch_block(j + 1, pn);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ig = 0; ig < 4; ++ig)
 #pragma unroll
                     for (int e4 = 0; e4 < 4; ++e4)
 #pragma unroll
                         for (int mt = 0; mt < NO; ++mt)
                             o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                                TF::v_elem(v_lds, kt, ig * 4 + e4, mt, qn, half), pv[e4], o_acc[mt], 0, 0, 0);
-                }
+                                TF::v_elem(v_lds, kt, ig * 4 + e4, mt, qn, half), pc[kt][ig][e4], o_acc[mt], 0, 0, 0);
             __syncthreads();
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ig = 0; ig < 4; ++ig) pc[kt][ig] = pn[kt][ig];
         }
     }
     // block-rows without blocks write zeros (blocksparse.h:949-962)
