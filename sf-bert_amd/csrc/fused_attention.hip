@@ -407,8 +407,10 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         const uint8_t* const k_read = smem + (par ^ 1) * TILE;       // K(j+1)
         const uint8_t* const v_read = smem + (2 + par) * TILE;       // V(j)
         if (j + 2 >= win + 64) refill(j);
-        // K(j+2) replaces K(j), V(j+1) replaces V(j-1); the loads are issued a few at a time between the
-        // chunks below so that they never queue up in front of the arithmetic
+        // K(j+2) replaces K(j), V(j+1) replaces V(j-1); the loads are issued right after the first exponentials
+        // (behind the row maximum, which the next instructions depend on) so that they have the whole
+        // iteration to land: issued later, spread over the chunks, the last of them were still in flight at
+        // the end of the iteration and every wave waited for them there
         const uint8_t* const k_src = k_base + (size_t)column_of(j + 2) * BS * row_bytes;
         const uint8_t* const v_src = v_base + (size_t)column_of(j + 1) * BS * row_bytes;
         const uint32_t k_dst = lds0 + par * TILE, v_dst = lds0 + (2 + (par ^ 1)) * TILE;
@@ -443,7 +445,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         for (int u = 0; u < PU; ++u) {
             if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
 #pragma unroll
-            for (int i = u * (T::LOADS / PU); i < (u + 1) * (T::LOADS / PU); ++i) {
+            for (int i = 0; i < (u == 0 ? T::LOADS : 0); ++i) {
                 T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
                 T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
             }
