@@ -151,23 +151,55 @@ __device__ __forceinline__ float* output_row(const FusedParams& p, size_t elemen
 
 // lse_row (may be null): receives m_used c + log2(total + 1e-6 f), so that the normalised probability of a key
 // with raw score s is exp2(s c - lse) -- what a backward pass needs to rebuild P without the row's other keys.
+//
+// The rows go to memory through a wave-private LDS slab (32 padded rows): straight from the accumulator layout a
+// store instruction would touch all 32 rows of the wave with 32 bytes each; from the slab every instruction writes
+// whole rows (1 KiB of 256-byte or 128-byte rows), as streaming (non-temporal) stores: O is written once and never
+// read by this launch, so it should not displace the K and V blocks that later work-groups of the head find in the
+// L2.  (Streaming stores of the 32-byte pieces were slower than cached ones; of whole rows they are faster.)
+// o_row is this lane's own row, o_row_bytes the distance between the rows of consecutive queries; slab must hold
+// 32 * (row size + 16) bytes and be free of other users.
 template <int NO>
-__device__ __forceinline__ void store_output(float* o_row, uint32_t as_bf16, float* lse_row, f32x16 (&o)[NO],
-                                             float m_used, float m_true, float total, float c, uint32_t half) {
+__device__ __forceinline__ void store_output(float* o_row, uint32_t o_row_bytes, uint32_t as_bf16, float* lse_row,
+                                             f32x16 (&o)[NO], float m_used, float m_true, float total, float c,
+                                             uint32_t lane, uint8_t* slab) {
+    constexpr int D = NO * 32;
+    const uint32_t qn = lane & 31, half = lane >> 5;
     const float f = exp2_fast((m_true - m_used) * c);
     const float inv = 1.0f / (total + 1e-6f * f);
     if (lse_row != nullptr && half == 0) *lse_row = __builtin_fmaf(m_used, c, __builtin_log2f(total + 1e-6f * f));
+    uint8_t* const wave_rows = (uint8_t*)o_row - (size_t)qn * o_row_bytes;   // row of the wave's first query
+    const uint32_t pitch = as_bf16 ? D * 2 + 16 : D * 4 + 16;
+    uint8_t* const mine = slab + qn * pitch;
     for_each_out_vec<NO>([&](int mt, int ig) {
         const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
                            o[mt][ig * 4 + 3] * inv};
         const uint32_t col = mt * 32 + ig * 8 + half * 4;
         if (as_bf16) {
             const u32x2 packed = {pack_bf16(out.x, out.y), pack_bf16(out.z, out.w)};
-            *(u32x2*)((uint8_t*)o_row + col * 2) = packed;
+            *(u32x2*)(mine + col * 2) = packed;
         } else {
-            *(f32x4*)(o_row + col) = out;
+            *(f32x4*)(mine + col * 4) = out;
         }
     });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (as_bf16) {
+        constexpr int CHUNKS = D / 8;   // 16-byte chunks per row
+#pragma unroll
+        for (int pass = 0; pass < CHUNKS / 2; ++pass) {
+            const uint32_t idx = pass * 64 + lane, row = idx / CHUNKS, ch = idx % CHUNKS;
+            __builtin_nontemporal_store(*(const u32x4*)(slab + row * pitch + ch * 16), (u32x4*)(wave_rows + (size_t)row * o_row_bytes + ch * 16));
+        }
+    } else {
+        constexpr int CHUNKS = D / 4;
+#pragma unroll
+        for (int pass = 0; pass < CHUNKS / 2; ++pass) {
+            const uint32_t idx = pass * 64 + lane, row = idx / CHUNKS, ch = idx % CHUNKS;
+            __builtin_nontemporal_store(*(const u32x4*)(slab + row * pitch + ch * 16), (u32x4*)(wave_rows + (size_t)row * o_row_bytes + ch * 16));
+        }
+    }
 }
 
 // Partial records are exchanged between work-groups of one launch.  They are written with
@@ -189,24 +221,27 @@ __device__ __forceinline__ uint32_t partial_offset(int mt, int ig, uint32_t half
 }
 
 template <int BS, int D>
-__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, uint32_t o_row_bytes,
                                                uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
-                                               uint32_t half);
+                                               uint32_t lane, uint8_t* slab);
 
 // End of a work item.  Unsplit rows are normalised and stored.  A chunk of a split row writes its
 // partial (unnormalised O, reference maximum, true maximum, sum) and bumps the row's counter; the
 // chunk that finds every other chunk already arrived merges all partials, stores O and resets the
-// counter for the next launch.  Nobody waits.
+// counter for the next launch.  Nobody waits.  lds: shared memory of the work-group that nobody uses any more, at
+// least 32 * (row size + 16) bytes per wave (the output rows pass through it).
 template <int BS, int D>
 __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& w, float* o_row,
                                            f32x16 (&o)[D / 32], const RowState& st, float c,
-                                           uint32_t q_in_block, uint32_t half, uint32_t t) {
+                                           uint32_t q_in_block, uint32_t half, uint32_t t, uint8_t* lds) {
+    const uint32_t lane = t & 63, o_row_bytes = p.heads * D * (p.o_bf16 ? 2u : 4u);
+    uint8_t* const slab = lds + (t >> 6) * (32u * (D * 4 + 16));
     float* const lse_row = p.lse ? p.lse + ((size_t)w.bh * p.nb + w.row) * BS + q_in_block : nullptr;
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;   // floats per partial
     const float total = st.l + __shfl_xor(st.l, 32);
     if (w.nchunks <= 1) {
-        store_output<NO>(o_row, p.o_bf16, lse_row, o, st.m_used, st.m_true, total, c, half);
+        store_output<NO>(o_row, o_row_bytes, p.o_bf16, lse_row, o, st.m_used, st.m_true, total, c, lane, slab);
         return;
     }
     float* base = p.partials + ((size_t)w.bh * p.n_parts + w.part) * PART;
@@ -232,15 +267,16 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     }
     __syncthreads();
     if (!last_flag) return;
-    merge_partials<BS, D>(base, w.nchunks, o_row, p.o_bf16, lse_row, c, q_in_block, half);
+    merge_partials<BS, D>(base, w.nchunks, o_row, o_row_bytes, p.o_bf16, lse_row, c, q_in_block, lane, slab);
     if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Merge of the partial records of a split row (run by the chunk that arrived last).
 template <int BS, int D>
-__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row,
+__device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, uint32_t o_row_bytes,
                                                uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
-                                               uint32_t half) {
+                                               uint32_t lane, uint8_t* slab) {
+    const uint32_t half = lane >> 5;
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -267,7 +303,7 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchun
             for (int e = 0; e < 4; ++e) acc[mt][ig * 4 + e] += coherent_load(src + e) * wgt;
         });
     }
-    store_output<NO>(o_row, as_bf16, lse_row, acc, m_used, m_true, sum, c, half);
+    store_output<NO>(o_row, o_row_bytes, as_bf16, lse_row, acc, m_used, m_true, sum, c, lane, slab);
 }
 
 template <int D>
@@ -320,6 +356,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     constexpr int SC = PU >= 2 ? PU / 2 : 1;   // chunks that carry a slice of the next block's scores
 
     __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+    static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
 
     const RowWork w = decode_row_work(p);
     if (!w.valid) return;
@@ -477,7 +514,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         if (j + 1 < count) iteration(j + 1, s_odd, s_even);
     }
 
-    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
+    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, smem);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -493,6 +530,7 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_ke
 
     __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
     __shared__ __attribute__((aligned(16))) float v_lds[T::V_FLOATS];
+    static_assert(T::K_FLOATS * 4 >= BS * (D * 4 + 16), "the K tile's memory doubles as the output slabs");
 
     const RowWork w = decode_row_work(p);
     if (!w.valid) return;
@@ -584,7 +622,7 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_ke
         __syncthreads();
     }
 
-    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t);
+    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, (uint8_t*)k_lds);
 }
 
 template <int BS, int D>
