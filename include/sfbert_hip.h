@@ -320,6 +320,12 @@ int sfb_layernorm(sfb_stream_t stream, void* out, int out_dtype, float* mean, fl
 /* tensor_add_matrix (ewops.h:276-282; cuda_kernels.h:526-535): out[b][i] = a[b][i] + m[i]. */
 int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, const float* m, uint32_t dim0,
                    uint64_t inner);
+/* transpose_0123to0213 (ewops.h:314-331): dst[a][c][b][:] = src[a][b][c][:], the [B, L, H, d] <-> [B, H, L, d]
+ * exchange the reference's CPU attention makes around its products (transformer.cpp:533-545).  The attention
+ * entry points of this library take [B, L, H, d] directly and need no such copy; it is provided for callers that
+ * keep tensors in the other order.  fp32, d3 % 4 == 0, dst != src. */
+int sfb_transpose_0213(sfb_stream_t stream, float* dst, const float* src, uint32_t d0, uint32_t d1, uint32_t d2,
+                       uint32_t d3);
 /* MI355X addition: bias + tensor_add_tensor + layernorm (ewops.h:10-17, 296-301, layernorm.h:13-38) in one
  * pass over memory: out = LayerNorm((in + bias[col]) + residual), same arithmetic and order as
  * sfb_bias_act followed by sfb_layernorm.  bias, residual may be NULL; out_bf16 [dev] optional second copy

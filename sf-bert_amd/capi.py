@@ -63,7 +63,7 @@ EXPORTED = [
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
-    "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
+    "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_transpose_0213", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm", "sfb_gemm_bias", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
     "sfb_model_forward",
@@ -549,6 +549,16 @@ def bias_residual_layernorm(x, bias, residual, gain, beta, with_bf16=False):
                                            _dev(gain), _dev(beta), C.c_uint32(rows), C.c_uint32(state)),
            "sfb_bias_residual_layernorm")
     return (out, out16) if with_bf16 else out
+
+
+def transpose_0123to0213(x):
+    """[d0, d1, d2, d3] -> [d0, d2, d1, d3] (ewops.h:314-331), fp32 on the device."""
+    import torch
+    d0, d1, d2, d3 = x.shape
+    out = torch.empty((d0, d2, d1, d3), dtype=torch.float32, device=x.device)
+    _check(lib.sfb_transpose_0213(_stream(), _dev(out), _dev(x), C.c_uint32(d0), C.c_uint32(d1), C.c_uint32(d2),
+                                  C.c_uint32(d3)), "sfb_transpose_0213")
+    return out
 
 
 def tensor_add_matrix(a, m):

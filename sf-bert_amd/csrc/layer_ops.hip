@@ -130,6 +130,21 @@ __global__ __launch_bounds__(256) void add_matrix_kernel(float* out, const float
         ((f32x4*)out)[i] = ((const f32x4*)a)[i] + ((const f32x4*)m)[i % inner4];
 }
 
+// dst[a][c][b][:] = src[a][b][c][:]  (ewops.h:314-331: [B, L, H, d] <-> [B, H, L, d]); rows of d3 floats stay whole
+__global__ __launch_bounds__(256) void transpose_0213_kernel(float* dst, const float* src, uint64_t vecs, uint32_t d1,
+                                                             uint32_t d2, uint32_t d3_4) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < vecs;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t x = (uint32_t)(i % d3_4);
+        const uint64_t row = i / d3_4;               // output row (a, c, b)
+        const uint32_t b = (uint32_t)(row % d1);
+        const uint64_t ac = row / d1;
+        const uint32_t c = (uint32_t)(ac % d2);
+        const uint64_t a = ac / d2;
+        ((f32x4*)dst)[i] = ((const f32x4*)src)[((a * d1 + b) * d2 + c) * d3_4 + x];
+    }
+}
+
 // out[t][:] = table[ids[t]][:] (+ pos[t % seq_len][:])  (embedding.h:5-12, ewops.h:276-282)
 __global__ __launch_bounds__(256) void embedding_kernel(float* out, const float* table, const int32_t* ids,
                                                         const float* pos, uint64_t tokens, uint32_t state4,
@@ -286,6 +301,18 @@ extern "C" int sfb_add_matrix(sfb_stream_t stream, float* out, const float* a, c
     const uint64_t vecs = dim0 * (inner / 4);
     clear_stale_error();
     add_matrix_kernel<<<dim3(grid_for(vecs)), 256, 0, (hipStream_t)stream>>>(out, a, m, vecs, inner / 4);
+    return launched();
+}
+
+extern "C" int sfb_transpose_0213(sfb_stream_t stream, float* dst, const float* src, uint32_t d0, uint32_t d1,
+                                  uint32_t d2, uint32_t d3) {
+    if (!dst || !src) return SFB_ERR_NULL_POINTER;
+    if (d0 == 0 || d1 == 0 || d2 == 0 || d3 == 0 || (d3 & 3u)) return SFB_ERR_SHAPE;
+    if (dst == src) return SFB_ERR_ARGUMENT;
+    if (((uintptr_t)dst | (uintptr_t)src) & 15u) return SFB_ERR_ALIGNMENT;
+    const uint64_t vecs = (uint64_t)d0 * d1 * d2 * (d3 / 4);
+    clear_stale_error();
+    transpose_0213_kernel<<<dim3(grid_for(vecs)), 256, 0, (hipStream_t)stream>>>(dst, src, vecs, d1, d2, d3 / 4);
     return launched();
 }
 

@@ -27,6 +27,12 @@ inline bool tensor_add_matrix(float* C, const float* A, const float* B, int dim_
                               CUstream stream = nullptr) {
     return sfb_host::ok(sfb_add_matrix(stream, C, A, B, (uint32_t)dim_0, (uint64_t)dim_1 * dim_2));
 }
+// ewops.h:314-331; the attention launchers take [B, L, H, d] directly, this is for callers that keep [B, H, L, d].
+inline bool transpose_0123to0213(const float* src, float* dst, int dim_0, int dim_1, int dim_2, int dim_3,
+                                 CUstream stream = nullptr) {
+    return sfb_host::ok(sfb_transpose_0213(stream, dst, src, (uint32_t)dim_0, (uint32_t)dim_1, (uint32_t)dim_2,
+                                           (uint32_t)dim_3));
+}
 // vocab bounds the ids (the reference does not check them).
 inline bool embedding_lookup(float* C, const float* A, const int* B, int batch_size, int seq_len, int head_num,
                              int size_per_head, int vocab, CUstream stream = nullptr) {
