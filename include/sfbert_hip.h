@@ -355,6 +355,24 @@ int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dt
 int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w, const float* bias,
                   int dtype, uint32_t m, uint32_t n, uint32_t k);
 
+/* The product followed by bias and GELU (transformer.cpp:562-569: cblas_sgemm, bias, gelu) in one kernel:
+ * C[m][n] = gelu(A[m][k] W[k][n] + bias[n]) with the reference's sigmoid form gelu(x) = x / (1 + exp(-1.702 x))
+ * (ewops.h:32-43), evaluated on the fp32 sums; c of out_dtype, c != a.  Runs on hipBLASLt (Swish epilogue with
+ * slope 1.702).  Where the hipBLASLt in the process has no such kernel or no slope argument (older builds, e.g. the
+ * one PyTorch loads), fp32 output falls back to sfb_gemm + sfb_bias_act in place and bf16 output returns
+ * SFB_ERR_LAUNCH.  n % 4 == 0. */
+int sfb_gemm_bias_gelu(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w, const float* bias,
+                       int dtype, uint32_t m, uint32_t n, uint32_t k);
+
+/* MI355X addition: the same in a form every hipBLASLt with a Swish epilogue can run.  C = *scale x gelu(A W + bias);
+ * *scale [host, out] is 1 where the library takes the slope, otherwise 1.702: x / (1 + exp(-s x)) = Swish_1(s x) / s,
+ * so the product and a copy of the bias (bias_scratch [dev] n floats) are scaled by s going in and the result is left
+ * s times too large -- a caller that multiplies C by a matrix next passes 1 / *scale as that product's factor (as
+ * the encoder layer does).  Returns SFB_ERR_LAUNCH if the library has no kernel for the shape.  n % 4 == 0. */
+int sfb_gemm_bias_gelu_scaled(sfb_stream_t stream, void* c, int out_dtype, float* scale, float* bias_scratch,
+                              const void* a, const void* w, const float* bias, int dtype, uint32_t m, uint32_t n,
+                              uint32_t k);
+
 /* Weights of one encoder layer, [in][out] row-major (transformer.cpp:98-136): matrices in the compute
  * dtype (fp32 or bf16), biases and LayerNorm parameters fp32.  All [dev]. */
 typedef struct {

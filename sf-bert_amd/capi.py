@@ -64,7 +64,7 @@ EXPORTED = [
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_transpose_0213", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
-    "sfb_gemm", "sfb_gemm_bias", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
+    "sfb_gemm", "sfb_gemm_bias", "sfb_gemm_bias_gelu", "sfb_gemm_bias_gelu_scaled", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
     "sfb_model_forward",
 ]
@@ -609,6 +609,33 @@ def gemm_bias(a, w, bias, out_dtype=None):
     _check(lib.sfb_gemm_bias(_stream(), _dev(c), code, _dev(a), _dev(w), _dev(bias), _dtype_code(a), C.c_uint32(m),
                              C.c_uint32(n), C.c_uint32(k)), "sfb_gemm_bias")
     return c
+
+
+def gemm_bias_gelu(a, w, bias, out_dtype=None):
+    """C[m, n] = gelu(a[m, k] @ w[k, n] + bias[n]), sigmoid-form GELU (ewops.h:32-43), in one kernel."""
+    import torch
+    m, k = a.shape
+    n = w.shape[1]
+    code = _dtype_code(a) if out_dtype is None else out_dtype
+    c = torch.empty((m, n), device=a.device, dtype=_torch_dtype(code))
+    _check(lib.sfb_gemm_bias_gelu(_stream(), _dev(c), code, _dev(a), _dev(w), _dev(bias), _dtype_code(a),
+                                  C.c_uint32(m), C.c_uint32(n), C.c_uint32(k)), "sfb_gemm_bias_gelu")
+    return c
+
+
+def gemm_bias_gelu_scaled(a, w, bias, out_dtype=None):
+    """(C, scale) with C[m, n] = scale * gelu(a[m, k] @ w[k, n] + bias[n]); scale is 1 or 1.702 (see the header)."""
+    import torch
+    m, k = a.shape
+    n = w.shape[1]
+    code = _dtype_code(a) if out_dtype is None else out_dtype
+    c = torch.empty((m, n), device=a.device, dtype=_torch_dtype(code))
+    scratch = torch.empty((n,), device=a.device, dtype=torch.float32)
+    scale = C.c_float(0.0)
+    _check(lib.sfb_gemm_bias_gelu_scaled(_stream(), _dev(c), code, C.byref(scale), _dev(scratch), _dev(a), _dev(w),
+                                         _dev(bias), _dtype_code(a), C.c_uint32(m), C.c_uint32(n), C.c_uint32(k)),
+           "sfb_gemm_bias_gelu_scaled")
+    return c, scale.value
 
 
 def gemm_nt(a, w):

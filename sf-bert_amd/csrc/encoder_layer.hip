@@ -31,20 +31,24 @@ rocblas_handle blas_handle() {
 
 inline size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 
-// GEMM with the bias add and the output conversion in its epilogue (hipBLASLt).  One plan per problem shape,
-// made on first use and kept; no workspace is requested, so nothing is allocated on the device.
+// GEMM with the bias add, optionally the activation, and the output conversion in its epilogue (hipBLASLt).  One
+// plan per problem shape, made on first use and kept; no workspace is requested, so nothing is allocated on the
+// device.  The activation is the reference's sigmoid form of GELU, x / (1 + exp(-1.702 x)) (ewops.h:32-43), which
+// is the library's Swish epilogue with its argument set to 1.702.
 struct LtPlan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
     hipblasLtMatmulAlgo_t algo;
     bool usable = false;
+    bool slope_set = false;   // activation plans: the library took the GELU slope as the Swish argument
 };
 hipblasLtHandle_t g_lt = nullptr;
-std::map<std::tuple<uint32_t, uint32_t, uint32_t, int, int>, LtPlan> g_plans;
+std::map<std::tuple<uint32_t, uint32_t, uint32_t, int, int, int>, LtPlan> g_plans;
+constexpr float kGeluSigmoidSlope = 1.702f;
 
 // row-major C[m][n] = A[m][k] W[k][n] + bias[n]  ==  column-major D[n][m] = W'[n][k] A'[k][m] + bias (per row of D)
-LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype) {
-    const auto key = std::make_tuple(m, n, k, dtype, out_dtype);
+LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, int act) {
+    const auto key = std::make_tuple(m, n, k, dtype, out_dtype, act);
     auto it = g_plans.find(key);
     if (it != g_plans.end()) return it->second;
     LtPlan& p = g_plans[key];
@@ -52,13 +56,18 @@ LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype) {
     const hipDataType in = dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
     const hipDataType out = out_dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
     const hipblasOperation_t none = HIPBLAS_OP_N;
-    const hipblasLtEpilogue_t epilogue = HIPBLASLT_EPILOGUE_BIAS;
+    const hipblasLtEpilogue_t epilogue = act ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT : HIPBLASLT_EPILOGUE_BIAS;
     const hipDataType bias_type = HIP_R_32F;
     bool ok = hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
+    // older builds of the library have the Swish epilogue but not its slope argument: there the slope stays 1 and
+    // the caller scales the operands instead (see gemm_bias_gelu_scaled)
+    if (ok && act)
+        p.slope_set = hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE_ACT_ARG0_EXT, &kGeluSigmoidSlope,
+                                                      sizeof(kGeluSigmoidSlope)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.w, in, n, k, n) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.a, in, k, m, k) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out, n, m, n) == HIPBLAS_STATUS_SUCCESS;
@@ -83,8 +92,9 @@ LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype) {
 
 }  // namespace
 
-extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
-                        uint32_t n, uint32_t k) {
+// c = alpha (a w), rocBLAS
+static int gemm_alpha(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m, uint32_t n,
+                      uint32_t k, float alpha) {
     if (!c || !a || !w) return SFB_ERR_NULL_POINTER;
     if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (!m || !n || !k) return SFB_ERR_SHAPE;
@@ -92,7 +102,7 @@ extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void
     rocblas_handle h = blas_handle();
     if (!h) return SFB_ERR_LAUNCH;
     if (rocblas_set_stream(h, (hipStream_t)stream) != rocblas_status_success) return SFB_ERR_LAUNCH;
-    const float alpha = 1.0f, beta = 0.0f;
+    const float beta = 0.0f;
     const rocblas_datatype in = dtype == SFB_BF16 ? rocblas_datatype_bf16_r : rocblas_datatype_f32_r;
     // row-major C[m][n] = A[m][k] W[k][n]  ==  column-major C^T[n][m] = W^T[n][k] A^T[k][m]
     const rocblas_status st = rocblas_gemm_ex(h, rocblas_operation_none, rocblas_operation_none, (int)n, (int)m,
@@ -102,30 +112,90 @@ extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void
     return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
 }
 
+extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
+                        uint32_t n, uint32_t k) {
+    return gemm_alpha(stream, c, a, w, dtype, m, n, k, 1.0f);
+}
+
+// C = act(alpha A W + bias) through one library GEMM; SFB_ERR_LAUNCH when the library has no kernel for it.
+// act = 1 without the slope argument (*slope_set false) computes Swish with slope 1.
+static int gemm_bias_epilogue(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
+                              const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k, int act,
+                              float alpha_unless_slope_set = 1.0f, bool* slope_set = nullptr) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, act);
+    if (!p.usable) return SFB_ERR_LAUNCH;
+    if (slope_set) *slope_set = p.slope_set;
+    const float alpha = (act && !p.slope_set) ? alpha_unless_slope_set : 1.0f, beta = 0.0f;
+    const void* bias_ptr = bias;
+    if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) ==
+            HIPBLAS_STATUS_SUCCESS &&
+        hipblasLtMatmul(g_lt, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo, nullptr, 0,
+                        (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS)
+        return SFB_OK;
+    p.usable = false;   // do not try this plan again
+    return SFB_ERR_LAUNCH;
+}
+
+// whether the activation plan of this shape exists and has its slope set (made on first use)
+static bool gelu_plan_state(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, bool* slope_set) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    const LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, 1);
+    *slope_set = p.slope_set;
+    return p.usable;
+}
+
+__global__ __launch_bounds__(256) void scale_vector_kernel(float* out, const float* in, float factor, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = in[i] * factor;
+}
+
 extern "C" int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
                              const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k) {
     if (!c || !a || !w || !bias) return SFB_ERR_NULL_POINTER;
     if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
     if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
-    {
-        std::lock_guard<std::mutex> lock(g_mutex);
-        LtPlan& p = lt_plan(m, n, k, dtype, out_dtype);
-        if (p.usable) {
-            const float alpha = 1.0f, beta = 0.0f;
-            const void* bias_ptr = bias;
-            if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) ==
-                    HIPBLAS_STATUS_SUCCESS &&
-                hipblasLtMatmul(g_lt, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo, nullptr, 0,
-                                (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS)
-                return SFB_OK;
-            p.usable = false;   // do not try this plan again
-        }
-    }
+    if (gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 0) == SFB_OK) return SFB_OK;
     // no fused kernel for this shape: plain GEMM, then the bias pass.  The fp32 product needs room: in place for
     // fp32 output, otherwise there is none here
     if (out_dtype != SFB_F32) return SFB_ERR_LAUNCH;
     const int rc = sfb_gemm(stream, (float*)c, a, w, dtype, m, n, k);
     return rc != SFB_OK ? rc : sfb_bias_act(stream, c, SFB_F32, (const float*)c, bias, nullptr, 0, m, n);
+}
+
+extern "C" int sfb_gemm_bias_gelu(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
+                                  const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k) {
+    if (!c || !a || !w || !bias) return SFB_ERR_NULL_POINTER;
+    if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
+    if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
+    if (c == a) return SFB_ERR_ARGUMENT;
+    bool slope_set = false;
+    if (gelu_plan_state(m, n, k, dtype, out_dtype, &slope_set) && slope_set &&
+        gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1) == SFB_OK)
+        return SFB_OK;
+    if (out_dtype != SFB_F32) return SFB_ERR_LAUNCH;
+    const int rc = sfb_gemm(stream, (float*)c, a, w, dtype, m, n, k);
+    return rc != SFB_OK ? rc : sfb_bias_act(stream, c, SFB_F32, (const float*)c, bias, nullptr, 1, m, n);
+}
+
+extern "C" int sfb_gemm_bias_gelu_scaled(sfb_stream_t stream, void* c, int out_dtype, float* scale,
+                                         float* bias_scratch, const void* a, const void* w, const float* bias,
+                                         int dtype, uint32_t m, uint32_t n, uint32_t k) {
+    if (!c || !a || !w || !bias || !scale || !bias_scratch) return SFB_ERR_NULL_POINTER;
+    if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
+    if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
+    if (c == a) return SFB_ERR_ARGUMENT;
+    bool slope_set = false;
+    if (!gelu_plan_state(m, n, k, dtype, out_dtype, &slope_set)) return SFB_ERR_LAUNCH;
+    *scale = 1.0f;
+    if (slope_set) return gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1);
+    // x / (1 + exp(-s x)) = Swish_1(s x) / s: the product and the bias are scaled by s going in, and the result is
+    // left s times too large for the caller to fold into what it does next
+    (void)hipGetLastError();   // only this launch is reported
+    scale_vector_kernel<<<dim3((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(bias_scratch, bias, kGeluSigmoidSlope, n);
+    if (hipGetLastError() != hipSuccess) return SFB_ERR_LAUNCH;
+    *scale = kGeluSigmoidSlope;
+    return gemm_bias_epilogue(stream, c, out_dtype, a, w, bias_scratch, dtype, m, n, k, 1, kGeluSigmoidSlope);
 }
 
 extern "C" int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
@@ -152,10 +222,10 @@ extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t
     const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
     const size_t f32 = sizeof(float), act = dtype == SFB_BF16 ? 2 : 4;
     // t (fp32 GEMM output, m x max(n, ffn)); q, k, v (compute dtype); attn (fp32); x1 (fp32);
-    // bf16 path only: xa (activation in compute dtype, m x max(n, ffn))
+    // bf16 path only: xa (activation in compute dtype, m x max(n, ffn)); ffn floats of bias scratch
     size_t bytes = align256(m * (ffn > n ? ffn : n) * f32) + 3 * align256(m * n * act) + 2 * align256(m * n * f32);
     if (dtype == SFB_BF16) bytes += align256(m * (ffn > n ? ffn : n) * act);
-    return bytes;
+    return bytes + align256(ffn * f32);   // scaled copy of the first FFN bias (sfb_gemm_bias_gelu_scaled)
 }
 
 // Everything a layer needs besides its input, output and weights
@@ -236,6 +306,8 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     float* attn = (float*)p;         p += align256(m * n * sizeof(float));
     float* x1 = (float*)p;           p += align256(m * n * sizeof(float));
     void* xa = bf ? (void*)p : nullptr;
+    if (bf) p += align256(m * wide * act);
+    float* bias_scratch = (float*)p;
     int rc;
 #define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
     // LN1 straight into the compute dtype; the fp32 path borrows the attention output buffer, which is free
@@ -252,11 +324,18 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     // LN2 into the compute dtype (fp32: the attention output buffer again, consumed by the GEMM above)
     void* a2 = bf ? xa : (void*)attn;
     SFB_TRY(sfb_layernorm(stream, a2, dtype, nullptr, nullptr, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m, (uint32_t)n));
-    SFB_TRY(sfb_gemm(stream, t, a2, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
-    void* gl = bf ? xa : (void*)t;
-    SFB_TRY(sfb_bias_act(stream, gl, dtype, t, wt->b1, nullptr, 1, m, ffn));
-    float* t2 = bf ? t : attn;
-    SFB_TRY(sfb_gemm(stream, t2, gl, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn));
+    void* gl = t;
+    float* t2 = attn;
+    float g_scale = 1.0f;
+    if (sfb_gemm_bias_gelu_scaled(stream, t, dtype, &g_scale, bias_scratch, a2, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
+                                  (uint32_t)n) != SFB_OK) {
+        SFB_TRY(sfb_gemm(stream, t, a2, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+        gl = bf ? xa : (void*)t;
+        SFB_TRY(sfb_bias_act(stream, gl, dtype, t, wt->b1, nullptr, 1, m, ffn));
+        t2 = bf ? t : attn;
+        g_scale = 1.0f;
+    }
+    SFB_TRY(gemm_alpha(stream, t2, gl, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale));
     SFB_TRY(sfb_bias_act(stream, y, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
 #undef SFB_TRY
     return SFB_OK;
@@ -317,6 +396,8 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     float* attn = (float*)p;         p += align256(m * n * sizeof(float));
     float* x1 = (float*)p;           p += align256(m * n * sizeof(float));
     void* xa = bf ? (void*)p : nullptr;
+    if (bf) p += align256(m * wide * act);
+    float* bias_scratch = (float*)p;
     const float scale = 1.0f / sqrtf((float)state_dim);
     int rc;
 #define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
@@ -354,12 +435,20 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
         if (!fused_ln) SFB_TRY(sfb_cast_f32_bf16(stream, xa, x1, m * n));
         fin = xa;
     }
-    SFB_TRY(sfb_gemm(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
-    void* g = bf ? xa : (void*)t;   // activation after GELU, in the compute dtype (in place for fp32)
-    SFB_TRY(sfb_bias_act(stream, g, dtype, t, wt->b1, nullptr, 1, m, ffn));
-    // the second FFN GEMM reads g and must not write over it: fp32 writes into attn's buffer
-    float* t2 = bf ? t : attn;
-    SFB_TRY(sfb_gemm(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn));
+    // bias and GELU ride in the first GEMM's epilogue where the library has such a kernel (its result goes into t,
+    // which nothing else uses at this point); otherwise GEMM into t, then one bias + GELU pass
+    void* g = t;                    // activation after GELU (times g_scale), in the compute dtype
+    float* t2 = attn;               // the second FFN GEMM reads g and must not write over it
+    float g_scale = 1.0f;
+    if (sfb_gemm_bias_gelu_scaled(stream, t, dtype, &g_scale, bias_scratch, fin, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
+                                  (uint32_t)n) != SFB_OK) {
+        SFB_TRY(sfb_gemm(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+        g = bf ? xa : (void*)t;     // in place for fp32
+        SFB_TRY(sfb_bias_act(stream, g, dtype, t, wt->b1, nullptr, 1, m, ffn));
+        t2 = bf ? t : attn;
+        g_scale = 1.0f;
+    }
+    SFB_TRY(gemm_alpha(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale));
     if (fused_ln) {
         SFB_TRY(sfb_bias_residual_layernorm(stream, y, nullptr, t2, wt->b2, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m,
                                             (uint32_t)n));

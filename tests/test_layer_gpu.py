@@ -124,6 +124,44 @@ def test_gemm_bias_one_kernel(bf16, out_bf16):
         assert rel_err(got, want) <= 1e-5
 
 
+@pytest.mark.parametrize("bf16,out_bf16", [(False, False), (True, False), (True, True)])
+def test_gemm_bias_gelu_one_kernel(bf16, out_bf16):
+    """GEMM with bias and the sigmoid-form GELU in the epilogue equals sgemm -> bias -> gelu of the oracle (values
+    chosen so that the activation's curved part, |x| < 1, and both tails are covered)."""
+    m, k, n = 520, 768, 3072
+    A = orc.fill_normal((m, k), 23)
+    W = orc.fill_normal((k, n), 24, 0.08)
+    b = orc.fill_normal((n,), 25)
+    if bf16:
+        A, W = orc.round_bf16(A), orc.round_bf16(W)
+    pre = orc.bias(orc.sgemm(A, W, nthreads=16), b)
+    assert (np.abs(pre) < 1).mean() > 0.2 and (pre > 3).mean() > 0.01 and (pre < -3).mean() > 0.01
+    want = orc.gelu(pre)
+    a, w = T(A), T(W)
+    if bf16:
+        a, w = a.to(torch.bfloat16), w.to(torch.bfloat16)
+    code = sfb.BF16 if out_bf16 else sfb.F32
+
+    def check(got, scale):
+        assert got.dtype == (torch.bfloat16 if out_bf16 else torch.float32)
+        got = got.float().cpu().numpy()
+        if out_bf16:
+            assert np.array_equal(got, orc.round_bf16(got))
+            assert np.abs(got / scale - want).max() <= 2.0 ** -8 * np.abs(want).max()
+        else:
+            assert rel_err(got / scale, want) <= 1e-5
+
+    # the scaled form runs wherever the GEMM library has a Swish epilogue; its factor is 1 or the slope
+    got, scale = sfb.gemm_bias_gelu_scaled(a, w, T(b), out_dtype=code)
+    assert scale in (1.0, np.float32(1.702))
+    check(got, np.float32(scale))
+    # the exact form needs the library's slope argument for bf16 output and says so when it is missing
+    try:
+        check(sfb.gemm_bias_gelu(a, w, T(b), out_dtype=code), np.float32(1.0))
+    except sfb.SfbError as e:
+        assert out_bf16 and scale != 1.0 and e.status == 7, e
+
+
 def layer_weights(n, ffn, seed):
     shapes = [("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)), ("w2", (ffn, n)),
               ("bq", (n,)), ("bk", (n,)), ("bv", (n,)), ("bo", (n,)), ("b1", (ffn,)), ("b2", (n,)),
