@@ -6,8 +6,10 @@ One step = one fused attention call over the whole batch of the workload (defaul
 configuration B4 H12 L4096 d64 block 64, bf16 inputs, fp32 accumulation and output).  Inputs are
 synthetic N(0,1) tensors already resident in HBM when the timed region starts.  Prints ONE JSON line:
 metric/value = effective TFLOP/s over the nonzero blocks (nnz*B*H*4*bs^2*d flops per call), plus
-`roofline` (MFMA bound, measured with HIP events on the launch stream) and `cpu_baseline` (the CPU
-oracle timed on this host's cores on a bounded sample of the same workload).
+`roofline` (MFMA bound, measured with HIP events on the launch stream), `cpu_baseline` (the CPU
+oracle timed on this host's cores on a bounded sample of the same workload) and
+`cpu_reference_single_thread` (the reference's own CPU attention functions, one thread as the reference is
+built, at the smallest configuration's shape).
 """
 import argparse
 import importlib
@@ -40,6 +42,36 @@ def make_layout(sfb, pattern, nb):
     if pattern == "strided":
         return sfb.layout_strided(nb, 4, 4)
     return sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234))
+
+
+def cpu_reference_single_thread():
+    """The reference's CPU attention as it is built (one thread, dense L x L buffers, causal: transformer.cpp:533-545)
+    at the shape of the smallest configuration, B1 H12 L512 d64: the reference's own functions compiled into
+    oracle/_ref where that library exists, otherwise the oracle's block loops on one thread over the same causal
+    layout."""
+    import numpy as np
+    import oracle_lib as orc
+    B, H, L, d, bs = 1, 12, 512, 64, 32
+    Q, K, V = (orc.fill_normal((B, L, H, d), 910 + i) for i in range(3))
+    scale = 1.0 / np.sqrt(d)
+    flops = 4.0 * B * H * (L * (L + 1) / 2) * d      # useful multiply-adds of the causal triangle
+    if orc.ref is not None:
+        from test_oracle_attention import ref_dense_causal
+        run, kind = (lambda: ref_dense_causal(Q, K, V, scale)), "reference"
+    else:
+        from test_oracle_attention import causal_case
+        _, _, _, luts, words = causal_case(B, H, L, d, bs, seed=910)
+        run, kind = (lambda: orc.attention(Q, K, V, luts["nn_lut"], bs, scale, mask=words, nthreads=1)), "port"
+    run()
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 10 and time.perf_counter() - t_begin < 5.0:
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    dt = sum(times) / len(times)
+    return {"ms_per_call": dt * 1e3, "value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": "dense causal attention B1 H12 L512 d64 fp32, %d calls" % len(times)}
 
 
 def cpu_baseline(luts, B, H, L, d, bs, bf16, flops):
@@ -358,6 +390,7 @@ def main():
             result["model_forward"] = time_model(sfb, torch, luts, bs, H, d, args.max_blocks)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops)
+        result["cpu_reference_single_thread"] = cpu_reference_single_thread()
     print(json.dumps(result))
 
 
