@@ -289,8 +289,9 @@ def main():
                     help="only the fused-attention line: no unfused comparison, no encoder-layer timing")
     ap.add_argument("--heavy", type=int, default=-1,
                     help="override the schedule's number of leading items launched for all heads first")
-    ap.add_argument("--max-blocks", type=int, default=16,
-                    help="split block-rows longer than this many key blocks (0 = one work-group per row)")
+    ap.add_argument("--max-blocks", type=int, default=-1,
+                    help="split block-rows longer than this many key blocks (0 = one work-group per row, "
+                         "-1 = what sfb_suggest_max_blocks gives for the launch's batch x heads)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path shards over (batch, head) with no exchange and "
@@ -322,6 +323,9 @@ def main():
     order = sfb.to_device(luts["row_order"])
     scale = 1.0 / (d ** 0.5)
 
+    auto_blocks = args.max_blocks < 0
+    if auto_blocks:
+        args.max_blocks = sfb.suggest_max_blocks(luts["nn_lut"], nb, B * H)
     if args.max_blocks > 0:
         sched = sfb.build_schedule(luts["nn_lut"], nb, args.max_blocks)
         if args.heavy >= 0:
@@ -369,7 +373,8 @@ def main():
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": "%s: %s block-sparse attention B%d H%d L%d d%d block %d, %d nonzero "
                                "blocks, %s inputs, fp32 accumulate/output" %
-                               (args.workload, pattern, B, H, L, d, bs, blocks, dtype)},
+                               (args.workload, pattern, B, H, L, d, bs, blocks, dtype),
+                   "max_blocks": args.max_blocks},
         "ms_per_attention_call": kernel_ms,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": traffic,
@@ -386,8 +391,10 @@ def main():
             result["backward_fused"] = time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale,
                                                            args.max_blocks, flops)
         if args.workload == "c4":
-            result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, args.max_blocks)
-            result["model_forward"] = time_model(sfb, torch, luts, bs, H, d, args.max_blocks)
+            # the layer and the model run eight sequences: their own chunk length
+            layer_blocks = sfb.suggest_max_blocks(luts["nn_lut"], nb, 8 * H) if auto_blocks else args.max_blocks
+            result["encoder_layer"] = time_layer(sfb, torch, luts, bs, H, d, layer_blocks)
+            result["model_forward"] = time_model(sfb, torch, luts, bs, H, d, layer_blocks)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(luts, B, H, L, d, bs, bf16, flops)
         result["cpu_reference_single_thread"] = cpu_reference_single_thread()

@@ -123,6 +123,11 @@ typedef struct {
  * query call.  n_slots = number of split rows, n_parts = total chunks of split rows, n_heavy = number
  * of leading items with at least twice the median number of key blocks (launched for all heads
  * before the rest; always < n_items). */
+/* MI355X addition: a max_blocks for sfb_build_schedule that suits a launch over batch_heads = batch x heads
+ * (batch, head) pairs: 1.25 x the key blocks one of the device's 1024 resident work-group slots gets to process in
+ * the whole launch, at least 16.  (BigBird L = 4096, 12 heads: 16 for one sequence, 19 for two, 37 -- global rows cut in
+ * two -- for four, no cut from eight on.) */
+uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_heads);
 int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
                        uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
 /* Bytes of the [dev] workspace a scheduled launch needs: arrival counters + partial records.  The

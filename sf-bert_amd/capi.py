@@ -47,6 +47,7 @@ lib.sfb_count_blocks.restype = C.c_uint32
 lib.sfb_magicu64.restype = None
 lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
+lib.sfb_suggest_max_blocks.restype = C.c_uint32
 lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
@@ -58,7 +59,7 @@ EXPORTED = [
     "sfb_layout_strided", "sfb_layout_bigbird", "sfb_bigbird_draw", "sfb_count_blocks",
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
-    "sfb_build_schedule", "sfb_schedule_workspace_bytes",
+    "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
@@ -188,6 +189,12 @@ def transpose_mask(words, blocks, bs):
 
 WORK_ITEM_DTYPE = np.dtype([(n, np.uint32) for n in
                             ("row", "first", "count", "nchunks", "chunk", "slot", "part", "lut_first")])
+
+
+def suggest_max_blocks(nn_lut, nb, batch_heads):
+    """Chunk length for build_schedule that suits a launch over batch_heads (batch, head) pairs."""
+    nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
+    return int(lib.sfb_suggest_max_blocks(_np(nn_lut), nb, C.c_uint32(batch_heads)))
 
 
 def build_schedule(nn_lut, nb, max_blocks=16):

@@ -310,6 +310,20 @@ int sfb_build_row_order(uint32_t* row_order, const sfb_uint2* nn_lut, int nb) {
     return SFB_OK;
 }
 
+uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_heads) {
+    if (!nn_lut || nb <= 0 || batch_heads == 0) return 16;
+    // The device keeps 256 x 4 work-groups of the fused kernel resident.  A work item should not be longer than
+    // what one of those slots gets to do in the whole launch (else it alone decides when the launch ends), and
+    // every cut costs a partial record, a device-wide counter update and a share of a merge, so rows are cut into
+    // as few chunks as that allows; with few (batch, head) pairs the chunks stay at 16 key blocks so that the
+    // long rows spread over the idle slots.
+    constexpr uint64_t kResidentWorkGroups = 1024;
+    uint64_t total = 0;
+    for (int r = 0; r < nb; ++r) total += nn_lut[r].y;
+    const uint64_t per_slot = (5 * total * batch_heads + 4 * kResidentWorkGroups - 1) / (4 * kResidentWorkGroups);
+    return (uint32_t)(per_slot > 16 ? (per_slot < 0xffffffffull ? per_slot : 0xffffffffull) : 16);
+}
+
 int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
                        uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
     if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;

@@ -213,6 +213,11 @@ __device__ __forceinline__ void coherent_store4(float* p, f32x4 v) {
 __device__ __forceinline__ float coherent_load(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// two consecutive floats (8-byte aligned) in one access
+__device__ __forceinline__ f32x2 coherent_load2(const float* p) {
+    const uint64_t bits = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(f32x2, bits);
+}
 // Partial-record offset (floats) of output vector (mt, ig) of a lane: vectors of one (mt, ig, half)
 // are contiguous over the block's queries, so every store instruction writes whole lines.
 template <int BS>
@@ -299,8 +304,11 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchun
         sum += coherent_load(stats + 2) * wgt;
         for_each_out_vec<NO>([&](int mt, int ig) {
             const float* src = part + partial_offset<BS>(mt, ig, half, q_in_block);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[mt][ig * 4 + e] += coherent_load(src + e) * wgt;
+            const f32x2 lo = coherent_load2(src), hi = coherent_load2(src + 2);
+            acc[mt][ig * 4 + 0] += lo.x * wgt;
+            acc[mt][ig * 4 + 1] += lo.y * wgt;
+            acc[mt][ig * 4 + 2] += hi.x * wgt;
+            acc[mt][ig * 4 + 3] += hi.y * wgt;
         });
     }
     store_output<NO>(o_row, o_row_bytes, as_bf16, lse_row, acc, m_used, m_true, sum, c, lane, slab);

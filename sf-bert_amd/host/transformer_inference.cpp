@@ -80,11 +80,12 @@ int main(int argc, char** argv) {
     HIP_OK(hipMemcpy(d_nn, nn.data(), nn.size() * sizeof(sfb_uint2), hipMemcpyHostToDevice));
     HIP_OK(hipMalloc((void**)&d_mask, mask.size() * 8));
     HIP_OK(hipMemcpy(d_mask, mask.data(), mask.size() * 8, hipMemcpyHostToDevice));
-    // rows longer than 16 key blocks are split into chunks so that the launch is balanced
+    // rows much longer than a work-group's share of the launch are split into chunks so that the launch is balanced
+    const uint32_t max_blocks = sfb_suggest_max_blocks(nn.data(), nb, (uint32_t)(batch_size * head_num));
     uint32_t n_items = 0, n_heavy = 0, n_slots = 0, n_parts = 0;
-    sfb_build_schedule(nullptr, &n_items, &n_heavy, &n_slots, &n_parts, nn.data(), nb, 16);
+    sfb_build_schedule(nullptr, &n_items, &n_heavy, &n_slots, &n_parts, nn.data(), nb, max_blocks);
     std::vector<sfb_work_item> items(n_items);
-    sfb_build_schedule(items.data(), &n_items, &n_heavy, &n_slots, &n_parts, nn.data(), nb, 16);
+    sfb_build_schedule(items.data(), &n_items, &n_heavy, &n_slots, &n_parts, nn.data(), nb, max_blocks);
     sfb_work_item* d_items = nullptr;
     HIP_OK(hipMalloc((void**)&d_items, items.size() * sizeof(sfb_work_item)));
     HIP_OK(hipMemcpy(d_items, items.data(), items.size() * sizeof(sfb_work_item), hipMemcpyHostToDevice));

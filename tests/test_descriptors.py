@@ -114,6 +114,22 @@ def test_error_codes():
         sfb.layout_local(4, -1)
 
 
+def test_suggested_chunk_length():
+    """1.25 x (key blocks of one head x batch x heads / 1024 resident work-groups), rounded up, at least 16."""
+    lay = orc.layout_bigbird(64, 1, 2, True, orc.bigbird_draw(64, 1, 2, True, 3, 1234))
+    luts = sfb.build_luts(lay)
+    total = int(lay.sum())
+    assert total == 622
+    got = [sfb.suggest_max_blocks(luts["nn_lut"], 64, bh) for bh in (1, 12, 24, 48, 96, 192)]
+    want = [max(16, -(-5 * total * bh // 4096)) for bh in (1, 12, 24, 48, 96, 192)]
+    assert got == want == [16, 16, 19, 37, 73, 146]
+    # what it means for the two global rows of 64 key blocks: four chunks, four, two, none
+    for mb, chunks in ((16, 4), (19, 4), (37, 2), (73, 1)):
+        sched = sfb.build_schedule(luts["nn_lut"], 64, mb)
+        assert int((sched["items"]["row"] == 0).sum()) == chunks
+    assert sfb.suggest_max_blocks(luts["nn_lut"], 64, 0) == 16
+
+
 @pytest.mark.parametrize("max_blocks", [1, 3, 8, 100])
 def test_schedule_covers_every_block_once(max_blocks):
     lay = orc.layout_bigbird(64, 1, 2, True, orc.bigbird_draw(64, 1, 2, True, 3, 1234))
