@@ -47,8 +47,8 @@ struct LineWork {
     int32_t slot;   // -1: write the output directly
     bool valid;
 };
-__device__ __forceinline__ LineWork decode_line_work(const BackwardParams& p, const sfb_uint2* lut) {
-    const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.ranks, p.heavy);
+__device__ __forceinline__ LineWork decode_line_work(const BackwardParams& p, const sfb_uint2* lut, uint32_t wg) {
+    const WorkId id = decode_work(wg, p.batch * p.heads, p.ranks, p.heavy);
     LineWork w;
     w.valid = id.valid;
     w.bh = id.bh;
@@ -91,13 +91,13 @@ __device__ __forceinline__ void store_rows_f32(float* row, const f32x16 (&acc)[N
 // ------------------------------------------------------------------------------------------------
 // dQ: row owner
 // ------------------------------------------------------------------------------------------------
+// wg: index of the work-group among those of this part of the launch; smem: 4 tiles (K0 K1 V0 V1)
 template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void attention_dq_kernel(BackwardParams p) {
+__device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t wg, uint8_t* smem) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
 
-    const LineWork work = decode_line_work(p, p.nn_lut);
+    const LineWork work = decode_line_work(p, p.nn_lut, wg);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
     const uint32_t r = work.line;
@@ -194,13 +194,13 @@ __global__ __launch_bounds__(BS * 2, 2) void attention_dq_kernel(BackwardParams 
 // ------------------------------------------------------------------------------------------------
 // dK, dV: column owner
 // ------------------------------------------------------------------------------------------------
+// wg: index of the work-group among those of this part of the launch; smem: 4 tiles (Q0 Q1 dO0 dO1)
 template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void attention_dkdv_kernel(BackwardParams p) {
+__device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t wg, uint8_t* smem) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // Q0 Q1 dO0 dO1
 
-    const LineWork work = decode_line_work(p, p.tn_lut);
+    const LineWork work = decode_line_work(p, p.tn_lut, wg);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
     const uint32_t col = work.line;
@@ -321,6 +321,18 @@ __global__ __launch_bounds__(BS * 2, 2) void attention_dkdv_kernel(BackwardParam
 // Sum of the partial records of split block-rows (TENSORS = 1: dQ) or block-columns (TENSORS = 2: dK, dV), in chunk
 // order, by the work-group of the line's first chunk; all other work-groups leave at once.  A separate launch: the
 // partials are complete when it starts, nobody has to wait for anybody.
+// One launch for both halves of the backward pass: the first col_wgs work-groups own key columns (dK, dV: the longer
+// items, so they go first), the others own query rows (dQ).  As two launches, the second waits until the last
+// work-group of the first is done; as one, its work-groups fill the slots as the first's drain.  col_wgs is a
+// multiple of 8, so both halves see the same work-group -> XCD assignment as a launch of their own.
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 2) void attention_backward_kernel(BackwardParams cols, BackwardParams rows,
+                                                                       uint32_t col_wgs) {
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * Bf16DirectTiles<BS, D>::TILE_BYTES];
+    if (blockIdx.x < col_wgs) attention_dkdv<BS, D, MASKED>(cols, blockIdx.x, smem);
+    else attention_dq<BS, D, MASKED>(rows, blockIdx.x - col_wgs, smem);
+}
+
 template <int BS, int D, int TENSORS>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(float* out0, float* out1, const float* partials,
                                                               const sfb_work_item* items, uint32_t n_parts,
@@ -354,13 +366,11 @@ static int launch_backward(hipStream_t stream, const BackwardParams& p, const sf
     cols.items = col_items; cols.ranks = col_items ? n_col_items : p.nb; cols.heavy = col_items ? n_col_heavy : 0;
     cols.n_parts = n_col_parts; cols.partials = col_partials;
     clear_stale_error();
-    if (masked) {
-        attention_dkdv_kernel<BS, 64, true><<<dim3(groups * 8u * cols.ranks), dim3(BS * 2), 0, stream>>>(cols);
-        attention_dq_kernel<BS, 64, true><<<dim3(groups * 8u * rows.ranks), dim3(BS * 2), 0, stream>>>(rows);
-    } else {
-        attention_dkdv_kernel<BS, 64, false><<<dim3(groups * 8u * cols.ranks), dim3(BS * 2), 0, stream>>>(cols);
-        attention_dq_kernel<BS, 64, false><<<dim3(groups * 8u * rows.ranks), dim3(BS * 2), 0, stream>>>(rows);
-    }
+    const uint32_t col_wgs = groups * 8u * cols.ranks, row_wgs = groups * 8u * rows.ranks;
+    if (masked)
+        attention_backward_kernel<BS, 64, true><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
+    else
+        attention_backward_kernel<BS, 64, false><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
     if (col_items && n_col_parts)
         reduce_partials_kernel<BS, 64, 2><<<dim3(n_col_items, p.batch * p.heads), dim3(256), 0, stream>>>(
             p.dk, p.dv, col_partials, col_items, n_col_parts, p.heads, p.nb * BS);
