@@ -333,13 +333,12 @@ __global__ __launch_bounds__(BS * 2, 2) void attention_backward_kernel(BackwardP
     else attention_dq<BS, D, MASKED>(rows, blockIdx.x - col_wgs, smem);
 }
 
+// Sum of the partial records of one split line, in chunk order (so the result does not depend on which chunk
+// finished when), written to the line's rows of the output tensors.
 template <int BS, int D, int TENSORS>
-__global__ __launch_bounds__(256) void reduce_partials_kernel(float* out0, float* out1, const float* partials,
-                                                              const sfb_work_item* items, uint32_t n_parts,
-                                                              uint32_t heads, uint32_t ctx) {
-    const sfb_work_item it = items[blockIdx.x];
-    if (it.nchunks <= 1 || it.chunk != 0) return;
-    const uint32_t bh = blockIdx.y, b = bh / heads, h = bh % heads;
+__device__ __forceinline__ void reduce_line(float* out0, float* out1, const float* partials, const sfb_work_item& it,
+                                            uint32_t n_parts, uint32_t bh, uint32_t heads, uint32_t ctx) {
+    const uint32_t b = bh / heads, h = bh % heads;
     constexpr int VECS = BS * D / 4;
     for (int tensor = 0; tensor < TENSORS; ++tensor) {
         float* out = tensor == 0 ? out0 : out1;
@@ -351,6 +350,21 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(float* out0, float
             *(f32x4*)(out + token_offset(b, it.row * BS + row, h, ctx, heads, D) + c4 * 4) = sum;
         }
     }
+}
+
+// grid (n_col_items + n_row_items, batch*heads): the work-groups of the first chunk of a split column (dK, dV) or
+// row (dQ) do the sums, all others leave at once
+template <int BS, int D>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(float* dk, float* dv, float* dq, const float* col_partials,
+                                                              const float* row_partials, const sfb_work_item* col_items,
+                                                              const sfb_work_item* row_items, uint32_t n_col_items,
+                                                              uint32_t n_col_parts, uint32_t n_row_parts, uint32_t heads,
+                                                              uint32_t ctx) {
+    const bool column = blockIdx.x < n_col_items;
+    const sfb_work_item it = column ? col_items[blockIdx.x] : row_items[blockIdx.x - n_col_items];
+    if (it.nchunks <= 1 || it.chunk != 0) return;
+    if (column) reduce_line<BS, D, 2>(dk, dv, col_partials, it, n_col_parts, blockIdx.y, heads, ctx);
+    else reduce_line<BS, D, 1>(dq, nullptr, row_partials, it, n_row_parts, blockIdx.y, heads, ctx);
 }
 
 template <int BS>
@@ -371,12 +385,12 @@ static int launch_backward(hipStream_t stream, const BackwardParams& p, const sf
         attention_backward_kernel<BS, 64, true><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
     else
         attention_backward_kernel<BS, 64, false><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
-    if (col_items && n_col_parts)
-        reduce_partials_kernel<BS, 64, 2><<<dim3(n_col_items, p.batch * p.heads), dim3(256), 0, stream>>>(
-            p.dk, p.dv, col_partials, col_items, n_col_parts, p.heads, p.nb * BS);
-    if (row_items && n_row_parts)
-        reduce_partials_kernel<BS, 64, 1><<<dim3(n_row_items, p.batch * p.heads), dim3(256), 0, stream>>>(
-            p.dq, nullptr, row_partials, row_items, n_row_parts, p.heads, p.nb * BS);
+    const uint32_t reduce_cols = (col_items && n_col_parts) ? n_col_items : 0u;
+    const uint32_t reduce_rows = (row_items && n_row_parts) ? n_row_items : 0u;
+    if (reduce_cols + reduce_rows)
+        reduce_partials_kernel<BS, 64><<<dim3(reduce_cols + reduce_rows, p.batch * p.heads), dim3(256), 0, stream>>>(
+            p.dk, p.dv, p.dq, col_partials, row_partials, col_items, row_items, reduce_cols, n_col_parts, n_row_parts,
+            p.heads, p.nb * BS);
     return launch_status();
 }
 
