@@ -88,6 +88,31 @@ __device__ __forceinline__ void store_rows_f32(float* row, const f32x16 (&acc)[N
         }
 }
 
+// The same rows to an output tensor through a wave-private LDS slab (32 rows of D floats + 16 bytes each), so that
+// memory sees whole 256-byte rows as streaming stores instead of 32-byte pieces of 32 rows per instruction: the
+// gradients are written once and read by nobody in this launch.  my_row: this lane's row; row_floats: distance
+// between the rows of consecutive tokens.
+template <int NO>
+__device__ __forceinline__ void store_rows_slab(float* my_row, uint32_t row_floats, const f32x16 (&acc)[NO],
+                                                uint32_t lane, uint8_t* slab) {
+    constexpr int D = NO * 32, PITCH = D * 4 + 16, CHUNKS = D / 4;
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    store_rows_f32<NO>((float*)(slab + qn * PITCH), acc, half);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float* const wave_rows = my_row - (size_t)qn * row_floats;
+#pragma unroll
+    for (int pass = 0; pass < CHUNKS / 2; ++pass) {
+        const uint32_t idx = pass * 64 + lane, row = idx / CHUNKS, ch = idx % CHUNKS;
+        __builtin_nontemporal_store(*(const f32x4*)(slab + row * PITCH + ch * 16),
+                                    (f32x4*)(wave_rows + (size_t)row * row_floats + ch * 4));
+    }
+    // the slab is reused by the next tensor of the same wave
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 // ------------------------------------------------------------------------------------------------
 // dQ: row owner
 // ------------------------------------------------------------------------------------------------
@@ -187,8 +212,13 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
             e = e_next;
         }
     }
-    if (work.slot < 0) store_rows_f32<NO>(p.dq + my_row, dq_acc, half);
-    else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
+    if (work.slot < 0) {
+        // the last iteration's look-ahead tile loads have landed and every wave is done with the tiles: their
+        // memory carries the output slabs now
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        store_rows_slab<NO>(p.dq + my_row, p.heads * D, dq_acc, lane, smem + wave * (32 * (D * 4 + 16)));
+    } else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -309,8 +339,13 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
         }
     }
     if (work.slot < 0) {
-        store_rows_f32<NO>(p.dk + my_row, dk_acc, half);
-        store_rows_f32<NO>(p.dv + my_row, dv_acc, half);
+        // the last iteration's look-ahead tile loads have landed and every wave is done with the tiles: their
+        // memory carries the output slabs now
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        uint8_t* const slab = smem + wave * (32 * (D * 4 + 16));
+        store_rows_slab<NO>(p.dk + my_row, p.heads * D, dk_acc, lane, slab);
+        store_rows_slab<NO>(p.dv + my_row, p.heads * D, dv_acc, lane, slab);
     } else {   // partial record of a split column: dK rows, then dV rows
         float* part = p.partials + (((size_t)work.bh * p.n_parts + work.slot) * 2 * BS + key_in_block) * D;
         store_rows_f32<NO>(part, dk_acc, half);
