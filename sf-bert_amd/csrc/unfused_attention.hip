@@ -157,7 +157,7 @@ struct RowSlab {
         for (int pass = 0; pass < PASSES; ++pass) {
             const uint32_t row = pass * ROWS_PER_PASS + lane / CHUNKS, c = lane % CHUNKS;
             const u32x4 v = *(const u32x4*)(slab + row * PITCH + c * 16);
-            *(u32x4*)((uint8_t*)rows + row * ROW_BYTES + c * 16) = v;
+            __builtin_nontemporal_store(v, (u32x4*)((uint8_t*)rows + row * ROW_BYTES + c * 16));
         }
     }
     // memory -> registers in the same layout
@@ -326,11 +326,12 @@ __device__ __forceinline__ float wave_sum(float l) {
     return l;
 }
 
-// 8 consecutive elements of a lane: one 16-byte access for bf16, two for fp32
+// 8 consecutive elements of a lane: one 16-byte access for bf16, two for fp32.  S and P are streamed -- read once,
+// written once, far larger than the L2 -- so the bf16 accesses carry the non-temporal hint.
 template <typename T>
 __device__ __forceinline__ void load8(const T* src, float (&v)[8]) {
     if constexpr (sizeof(T) == 2) {
-        const u32x4 r = *(const u32x4*)src;
+        const u32x4 r = __builtin_nontemporal_load((const u32x4*)src);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             v[2 * i] = bf16_bits_to_f32(r[i] & 0xffffu);
@@ -345,7 +346,7 @@ template <typename T>
 __device__ __forceinline__ void store8(T* dst, const float (&v)[8]) {
     if constexpr (sizeof(T) == 2) {
         const u32x4 r = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
-        *(u32x4*)dst = r;
+        __builtin_nontemporal_store(r, (u32x4*)dst);
     } else {
         const f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
         *(f32x4*)dst = lo;
@@ -363,7 +364,7 @@ template <> struct Packed8<float> {
 };
 template <> struct Packed8<__bf16> {
     u32x4 r;
-    __device__ __forceinline__ void load(const __bf16* src) { r = *(const u32x4*)src; }
+    __device__ __forceinline__ void load(const __bf16* src) { r = __builtin_nontemporal_load((const u32x4*)src); }
     __device__ __forceinline__ float get(int i) const {
         return (i & 1) ? __builtin_bit_cast(float, r[i >> 1] & 0xffff0000u) : bf16_bits_to_f32(r[i >> 1] & 0xffffu);
     }
