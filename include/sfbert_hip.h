@@ -123,13 +123,13 @@ typedef struct {
  * query call.  n_slots = number of split rows, n_parts = total chunks of split rows, n_heavy = number
  * of leading items with at least twice the median number of key blocks (launched for all heads
  * before the rest; always < n_items). */
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
 /* MI355X addition: a max_blocks for sfb_build_schedule that suits a launch over batch_heads = batch x heads
  * (batch, head) pairs: 1.25 x the key blocks one of the device's 1024 resident work-group slots gets to process in
  * the whole launch, at least 16.  (BigBird L = 4096, 12 heads: 16 for one sequence, 19 for two, 37 -- global rows cut in
  * two -- for four, no cut from eight on.) */
 uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_heads);
-int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
-                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
 /* Bytes of the [dev] workspace a scheduled launch needs: arrival counters + partial records.  The
  * workspace must be zero-filled once before its first use; launches leave the counters at zero. */
 size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
@@ -194,7 +194,7 @@ int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const 
                                       uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                       uint32_t mask_heads, float scale);
 
-/* MI355X addition: the whole backward of the attention in two kernels, with P, dP and dS kept on chip.  Same
+/* MI355X addition: the whole backward of the attention in one pass over the blocks, with P, dP and dS kept on chip.  Same
  * arithmetic as the reference's sequence TN, NT, softmax gradient, TN, NN (transformer_attention_optimize.cu:
  * 924-965; ewops.h:101-124; matmul.h:81-99): P = exp2(S scale log2e - lse), dV = P^T dO, dS = P (dO V^T - delta)
  * scale, dK = dS^T Q, dQ = dS K, where delta = rowsum(dO * O) (computed here into the caller's buffer) stands for
