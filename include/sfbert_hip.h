@@ -135,6 +135,34 @@ uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_
 size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
                                     uint32_t head_dim, uint32_t block_size, uint32_t state_dim);
 
+/* MI355X addition (no reference counterpart): plan of a launch whose work-groups stay resident.  Instead of one
+ * work-group per work item, wg_slots work-groups (sfb_resident_work_groups(): as many as the device runs at once)
+ * each walk a list of items chosen here so that all lists cost about the same (key blocks plus a fixed charge per
+ * item): no dispatch gaps between items, and an item's descriptors are fetched while its predecessors are computed.
+ * Long items come first in every list; the lists of one die (slot index mod 8) only hold (batch, head) pairs of
+ * the same residue mod 8, so that a head's K and V stay in one L2. */
+typedef struct {
+    uint32_t batch, head;  /* which sequence and head */
+    uint32_t row;          /* the fields of sfb_work_item */
+    uint32_t first;
+    uint32_t count;        /* 0xffffffff: end of the list */
+    uint32_t nchunks;
+    uint32_t chunk;
+    uint32_t slot;
+    uint32_t part;
+    uint32_t lut_first;
+    uint32_t reserved[2];  /* entries are 48 bytes */
+} sfb_plan_entry;
+/*   nn_lut [host] lut_heads tables of lut_dim entries (lut_heads = 1: one layout for all heads; = head_dim:
+ *   per-head layouts as fixed_fusion_test.cu:38-39 builds them, every head with the same number of blocks).
+ *   plan [host] receives wg_slots lists of *plan_stride entries each (the last entries of a list are end marks);
+ *   NULL: only the sizes are returned.  *n_slots / *n_parts size the workspace (sfb_schedule_workspace_bytes). */
+int sfb_build_plan(sfb_plan_entry* plan, uint32_t* plan_stride, uint32_t* n_slots, uint32_t* n_parts,
+                   const sfb_uint2* nn_lut, int nb, uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim,
+                   uint32_t head_dim, uint32_t wg_slots, uint32_t max_blocks);
+/* Work-groups of the fused kernels the current device keeps resident (4 per compute unit); 0 without a device. */
+uint32_t sfb_resident_work_groups(void);
+
 /* ================================================================================================
  * Device entry points
  * ============================================================================================== */
@@ -193,6 +221,17 @@ int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const 
                                       void* workspace, size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
                                       uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                       uint32_t mask_heads, float scale);
+
+/* The same operation launched over sfb_build_plan's lists: wg_slots resident work-groups, each walking its list.
+ * Takes per-head look-up tables (lut_heads = head_dim) as well as a shared one.  plan [dev] wg_slots * plan_stride
+ * entries; lse may be NULL; out_dtype SFB_F32 or SFB_BF16; workspace as for sfb_fused_attention_scheduled. */
+int sfb_fused_attention_planned(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                                int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                const int32_t* valid_len, const sfb_plan_entry* plan, uint32_t wg_slots,
+                                uint32_t plan_stride, uint32_t n_slots, uint32_t n_parts, void* workspace,
+                                size_t workspace_bytes, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
+                                uint32_t lut_dim, uint32_t mask_heads, float scale);
 
 /* MI355X addition: the whole backward of the attention in one pass over the blocks, with P, dP and dS kept on chip.  Same
  * arithmetic as the reference's sequence TN, NT, softmax gradient, TN, NN (transformer_attention_optimize.cu:

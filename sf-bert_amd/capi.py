@@ -51,6 +51,7 @@ lib.sfb_suggest_max_blocks.restype = C.c_uint32
 lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
+lib.sfb_resident_work_groups.restype = C.c_uint32
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -60,6 +61,7 @@ EXPORTED = [
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
+    "sfb_build_plan", "sfb_resident_work_groups", "sfb_fused_attention_planned",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
@@ -210,6 +212,38 @@ def build_schedule(nn_lut, nb, max_blocks=16):
                 n_slots=int(n_slots.value), n_parts=int(n_parts.value))
 
 
+def resident_work_groups():
+    return int(lib.sfb_resident_work_groups())
+
+
+PLAN_ENTRY_DTYPE = np.dtype([(n, np.uint32) for n in
+                             ("batch", "head", "row", "first", "count", "nchunks", "chunk", "slot", "part",
+                              "lut_first", "reserved0", "reserved1")])
+PLAN_END = 0xffffffff
+
+
+def build_plan(nn_lut, nb, batch, heads, max_blocks=None, lut_heads=1, wg_slots=None):
+    """Lists of work items for the resident work-groups of a planned launch (sfb_build_plan): dict(plan
+    [wg_slots, stride] of PLAN_ENTRY_DTYPE, n_slots, n_parts, wg_slots, plan_stride, ...).  nn_lut: one table, or
+    lut_heads tables of equal length concatenated.  max_blocks None: what sfb_suggest_max_blocks gives for the
+    first table; wg_slots None: what the device keeps resident (sfb_resident_work_groups)."""
+    nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
+    lut_dim = nn_lut.shape[0] // lut_heads
+    if wg_slots is None:
+        wg_slots = resident_work_groups() or 1024
+    if max_blocks is None:
+        max_blocks = suggest_max_blocks(nn_lut[:lut_dim], nb, batch * heads)
+    stride, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    args = (_np(nn_lut), nb, C.c_uint32(lut_heads), C.c_uint32(lut_dim), C.c_uint32(batch), C.c_uint32(heads),
+            C.c_uint32(wg_slots), C.c_uint32(max_blocks))
+    _check(lib.sfb_build_plan(None, C.byref(stride), C.byref(n_slots), C.byref(n_parts), *args), "sfb_build_plan")
+    plan = np.zeros((wg_slots, stride.value), PLAN_ENTRY_DTYPE)
+    _check(lib.sfb_build_plan(_np(plan), C.byref(stride), C.byref(n_slots), C.byref(n_parts), *args), "sfb_build_plan")
+    return Luts(plan=plan, n_slots=int(n_slots.value), n_parts=int(n_parts.value), wg_slots=int(wg_slots),
+                plan_stride=int(stride.value), max_blocks=int(max_blocks), lut_heads=int(lut_heads),
+                lut_dim=int(lut_dim))
+
+
 def schedule_workspace_bytes(sched, batch, heads, block_size, d):
     return int(lib.sfb_schedule_workspace_bytes(C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]),
                                                 C.c_uint32(batch), C.c_uint32(heads),
@@ -349,6 +383,25 @@ def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_si
 
 
 # ------------------------------------------------------------------------------------ unfused trio
+def fused_attention_planned(q, k, v, nn_lut, plan_dev, plan, workspace, block_size, blocks, scale, mask=None,
+                            valid_len=None, mask_heads=1, out=None, lse=None):
+    """sfb_fused_attention_planned: resident work-groups walking build_plan()'s lists.  plan_dev: device copy of
+    plan["plan"]; workspace: zero-filled uint8 tensor of schedule_workspace_bytes(plan, ...) bytes (or None
+    without split rows)."""
+    import torch
+    B, L, H, d = q.shape
+    if out is None:
+        out = torch.empty((B, L, H, d), device=q.device, dtype=torch.float32)
+    _check(lib.sfb_fused_attention_planned(
+        _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dev(lse), _dtype_code(q), _dtype_code(out), _dev(nn_lut),
+        _dev(mask), _dev(valid_len), _dev(plan_dev), C.c_uint32(plan["wg_slots"]), C.c_uint32(plan["plan_stride"]),
+        C.c_uint32(plan["n_slots"]), C.c_uint32(plan["n_parts"]), _dev(workspace),
+        C.c_size_t(workspace.numel() if workspace is not None else 0), C.c_uint32(block_size), C.c_uint32(blocks),
+        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(plan["lut_heads"]),
+        C.c_uint32(plan["lut_dim"]), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_planned")
+    return out
+
+
 def _torch_dtype(code):
     import torch
     return torch.bfloat16 if code == BF16 else torch.float32

@@ -324,6 +324,117 @@ uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_
     return (uint32_t)(per_slot > 16 ? (per_slot < 0xffffffffull ? per_slot : 0xffffffffull) : 16);
 }
 
+}  // extern "C"
+
+// Work items of one head's NN look-up table, longest first; *slots / *parts count the split rows and their chunks.
+static std::vector<sfb_work_item> work_items_of(const sfb_uint2* nn_lut, int nb, uint32_t max_blocks,
+                                                uint32_t* slots_out, uint32_t* parts_out) {
+    std::vector<sfb_work_item> all;
+    uint32_t slots = 0, parts = 0;
+    for (int r = 0; r < nb; ++r) {
+        const uint32_t count = nn_lut[r].y;
+        const uint32_t chunks = count > max_blocks ? (count + max_blocks - 1) / max_blocks : 1;
+        if (chunks == 1) {
+            all.push_back(sfb_work_item{(uint32_t)r, 0u, count, 1u, 0u, 0u, 0u, nn_lut[r].x});
+            continue;
+        }
+        const uint32_t base = count / chunks, extra = count % chunks;
+        uint32_t first = 0;
+        for (uint32_t c = 0; c < chunks; ++c) {
+            const uint32_t len = base + (c < extra ? 1u : 0u);
+            all.push_back(sfb_work_item{(uint32_t)r, first, len, chunks, c, slots, parts, nn_lut[r].x + first});
+            first += len;
+        }
+        ++slots;
+        parts += chunks;
+    }
+    std::stable_sort(all.begin(), all.end(),
+                     [](const sfb_work_item& a, const sfb_work_item& b) { return a.count > b.count; });
+    *slots_out = slots;
+    *parts_out = parts;
+    return all;
+}
+
+extern "C" {
+
+int sfb_build_plan(sfb_plan_entry* plan, uint32_t* plan_stride, uint32_t* n_slots, uint32_t* n_parts,
+                   const sfb_uint2* nn_lut, int nb, uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim,
+                   uint32_t head_dim, uint32_t wg_slots, uint32_t max_blocks) {
+    if (!plan_stride || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
+    if (nb <= 0 || batch_dim == 0 || head_dim == 0 || wg_slots == 0 || lut_heads == 0) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && lut_heads != head_dim) return SFB_ERR_SHAPE;
+    if (max_blocks == 0) return SFB_ERR_ARGUMENT;
+    const uint64_t num_bh64 = (uint64_t)batch_dim * head_dim;
+    if (num_bh64 > 0x7fffffffull) return SFB_ERR_SHAPE;
+    const uint32_t num_bh = (uint32_t)num_bh64;
+
+    // item tables: one per look-up table (shared by all heads, or one per head)
+    std::vector<std::vector<sfb_work_item>> tables(lut_heads);
+    uint32_t slots = 0, parts = 0;
+    for (uint32_t h = 0; h < lut_heads; ++h) {
+        uint32_t s = 0, q = 0;
+        tables[h] = work_items_of(nn_lut + (size_t)h * lut_dim, nb, max_blocks, &s, &q);
+        slots = std::max(slots, s);
+        parts = std::max(parts, q);
+    }
+
+    // A work item costs its key blocks plus a fixed charge (start-up, write-out) of about two key blocks' time.
+    constexpr uint64_t kItemCharge = 2;
+    // Slots are dealt to the 8 dies like consecutive work-group ids; a (batch, head) whose index has residue x
+    // mod 8 is worked on by the slots of die x only, so its K and V stay in one L2.  The last batch*heads % 8
+    // pairs have no die of their own and go wherever the load is smallest.
+    const uint32_t dies = (wg_slots % 8 == 0 && num_bh >= 8) ? 8 : 1;
+    const uint32_t bound_bh = dies == 8 ? num_bh - num_bh % 8 : num_bh;
+    std::vector<std::vector<sfb_plan_entry>> lists(wg_slots);
+    std::vector<uint64_t> load(wg_slots, 0);
+    auto place = [&](uint32_t bh, const sfb_work_item& it) {
+        uint32_t best = 0xffffffffu;
+        const bool bound = dies == 8 && bh < bound_bh;
+        for (uint32_t s = bound ? bh % 8 : 0; s < wg_slots; s += bound ? 8 : 1)
+            if (best == 0xffffffffu || load[s] < load[best]) best = s;
+        lists[best].push_back(sfb_plan_entry{bh / head_dim, bh % head_dim, it.row, it.first, it.count, it.nchunks,
+                                             it.chunk, it.slot, it.part, it.lut_first, {0u, 0u}});
+        load[best] += it.count + kItemCharge;
+    };
+    auto table_of = [&](uint32_t bh) { return lut_heads > 1 ? bh % head_dim : 0u; };
+    // long items (at least twice the median) of every (batch, head) first, longest first; then the rest, one
+    // (batch, head) after the other, so that the slots of a die work on the same few heads at any time
+    std::vector<uint32_t> heavy(lut_heads, 0);
+    uint32_t longest = 0;
+    for (uint32_t h = 0; h < lut_heads; ++h) {
+        const auto& tb = tables[h];
+        if (tb.empty()) continue;
+        const uint32_t median = tb[tb.size() / 2].count;
+        while (heavy[h] < tb.size() && tb[heavy[h]].count >= 2 * median && tb[heavy[h]].count > median) ++heavy[h];
+        longest = std::max(longest, tb[0].count);
+    }
+    for (uint32_t len = longest; len > 0; --len)
+        for (uint32_t bh = 0; bh < num_bh; ++bh) {
+            const uint32_t h = table_of(bh);
+            for (uint32_t i = 0; i < heavy[h]; ++i)
+                if (tables[h][i].count == len) place(bh, tables[h][i]);
+        }
+    for (uint32_t bh = 0; bh < num_bh; ++bh) {
+        const uint32_t h = table_of(bh);
+        for (uint32_t i = heavy[h]; i < tables[h].size(); ++i) place(bh, tables[h][i]);
+    }
+    uint32_t stride = 0;
+    for (const auto& l : lists) stride = std::max(stride, (uint32_t)l.size());
+    stride += 2;   // two end marks: a work-group reads two entries ahead
+
+    if (plan) {
+        if (*plan_stride < stride) return SFB_ERR_ARGUMENT;
+        const sfb_plan_entry end = {0u, 0u, 0u, 0u, 0xffffffffu, 0u, 0u, 0u, 0u, 0u, {0u, 0u}};
+        for (uint32_t s = 0; s < wg_slots; ++s)
+            for (uint32_t i = 0; i < stride; ++i)
+                plan[(size_t)s * stride + i] = i < lists[s].size() ? lists[s][i] : end;
+    }
+    *plan_stride = stride;
+    *n_slots = slots;
+    *n_parts = parts;
+    return SFB_OK;
+}
+
 int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
                        uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
     if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;

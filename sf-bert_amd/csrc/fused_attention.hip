@@ -30,6 +30,8 @@ struct FusedParams {
     const int32_t* valid_len;       // per batch, or nullptr
     const uint32_t* row_order;      // rank -> block-row (unscheduled launches), or nullptr
     const sfb_work_item* items;     // rank -> work item (scheduled launches), or nullptr
+    const sfb_plan_entry* plan;     // planned launches: one list of work items per resident work-group
+    uint32_t plan_stride;           // entries between the lists of consecutive work-groups
     uint32_t* counters;             // [batch*heads][n_slots] arrival counters of split rows
     float* partials;                // [batch*heads][n_parts][BS*D + 4*BS]
     uint32_t n_slots, n_parts;
@@ -51,16 +53,16 @@ struct RowWork {
     uint32_t nchunks, slot, part;   // split rows: number of chunks, counter index, first partial index
     uint32_t chunk;
     uint32_t lut_first;             // index of the item's first entry in the head's NN LUT
-    bool valid;
+    uint32_t valid;
 };
 
 __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
     RowWork w;
     const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.ranks, p.heavy);
     w.valid = id.valid;
-    w.bh = id.bh;
-    w.b = id.bh / p.heads;
-    w.h = id.bh % p.heads;
+    w.bh = __builtin_amdgcn_readfirstlane(id.bh);
+    w.b = __builtin_amdgcn_readfirstlane(id.bh / p.heads);
+    w.h = __builtin_amdgcn_readfirstlane(id.bh % p.heads);
     if (p.items) {
         const sfb_work_item it = p.items[id.rank];
         w.row = it.row; w.first = it.first; w.count = it.count;
@@ -75,6 +77,45 @@ __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
         w.nchunks = 1; w.slot = 0; w.part = 0; w.chunk = 0;
     }
     return w;
+}
+
+// Work of one entry of a planned launch.
+__device__ __forceinline__ RowWork plan_row_work(const FusedParams& p, const sfb_plan_entry& e) {
+    RowWork w;
+    w.valid = 1;
+    w.b = e.batch;
+    w.h = e.head;
+    w.bh = e.batch * p.heads + e.head;
+    w.row = e.row; w.first = e.first; w.count = e.count;
+    w.nchunks = e.nchunks; w.slot = e.slot; w.part = e.part; w.chunk = e.chunk;
+    w.lut_first = e.lut_first;
+    return w;
+}
+constexpr uint32_t kPlanEnd = 0xffffffffu;
+// Plan entries are read through the constant address space: nothing writes them during a launch, and the
+// loads then go through the scalar unit, so an entry waits in scalar registers while an item is computed.
+typedef const uint32_t __attribute__((address_space(4)))* plan_words;
+struct PlanList {
+    plan_words words;
+    __device__ __forceinline__ sfb_plan_entry operator[](uint32_t i) const {
+        const plan_words w = words + (size_t)i * (sizeof(sfb_plan_entry) / 4);
+        sfb_plan_entry e;
+        e.batch = w[0]; e.head = w[1]; e.row = w[2]; e.first = w[3]; e.count = w[4]; e.nchunks = w[5];
+        e.chunk = w[6]; e.slot = w[7]; e.part = w[8]; e.lut_first = w[9];
+        e.reserved[0] = 0; e.reserved[1] = 0;
+        return e;
+    }
+};
+__device__ __forceinline__ PlanList plan_list_of(const FusedParams& p) {
+    return PlanList{(plan_words)(uintptr_t)(p.plan + (size_t)blockIdx.x * p.plan_stride)};
+}
+
+// LUT entries of key blocks [first, first + 64) of an item, one per lane (clamped to the item's last one).
+__device__ __forceinline__ sfb_uint2 lut_window(const FusedParams& p, const RowWork& w, uint32_t first, uint32_t lane) {
+    sfb_uint2 none = {0u, 0u};
+    if (w.count == 0) return none;
+    const uint32_t idx = first + lane;
+    return p.nn_lut[(size_t)w.h * p.lut_stride + w.lut_first + (idx < w.count ? idx : w.count - 1)];
 }
 
 // The probabilities of a row are kept relative to a reference maximum m_used that is only moved
@@ -356,34 +397,30 @@ __device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[
 //   * finds the row maximum of S(j), then, chunk by chunk, exponentiates S(j), feeds V(j)^T . P^T and
 //     computes a slice of S(j+1) = K(j+1) . Q^T;
 //   * waits for its own loads and meets the other waves at the one barrier of the iteration.
-template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
+// SLIM (launches without element mask and key padding): the probabilities of the whole item are taken relative to
+// one fixed offset, the row maximum of the item's first key block, so the loop needs no per-block maximum and never
+// rescales its accumulators.  The offset is a real score of the row, hence the row sum is at least about 1 and cannot
+// vanish; a later block whose scores exceed the offset by more than 2^100 in probability makes the sum overflow,
+// which the end of the item detects, and the item is then redone by the general loop (returns false).  The 1e-6 of
+// the reference's denominator is applied relative to the offset instead of the true row maximum, a relative
+// difference of at most 1e-6.
+template <int BS, int D, bool MASKED, bool SLIM>
+__device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const RowWork& w, uint8_t* smem, uint32_t* retry_flag,
+                                                 sfb_uint2 first_window) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
     constexpr int TILE = T::TILE_BYTES;
     constexpr int SC = PU >= 2 ? PU / 2 : 1;   // chunks that carry a slice of the next block's scores
+    static_assert(!(MASKED && SLIM), "masked launches take the general loop");
 
-    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
-    static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
-
-    const RowWork w = decode_row_work(p);
-    if (!w.valid) return;
     const uint32_t L = p.nb * BS;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
     const uint32_t row_bytes = p.heads * D * 2;
 
-    const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
-    const uint32_t lut_off = __builtin_amdgcn_readfirstlane(w.lut_first);
     const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
     float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
-
-    if (count == 0) {
-        store_zero_row<D>(o_row, p.o_bf16, half);
-        if (p.lse && half == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
-        return;
-    }
 
     const __bf16* Q = (const __bf16*)p.q;
     const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)w.h * p.mask_stride * (BS / 8) : nullptr;
@@ -397,13 +434,11 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     const uint32_t lds0 = T::lds_address(smem);
     // LUT entries of key blocks [win, win + 64) of this item, one per lane (clamped to the last one)
     uint32_t win = 0;
-    sfb_uint2 entries;
+    sfb_uint2 entries = first_window;
     auto refill = [&](uint32_t first) {
         win = first;
-        const uint32_t idx = first + lane;
-        entries = lut[lut_off + (idx < count ? idx : count - 1)];
+        entries = lut_window(p, w, first, lane);
     };
-    refill(0);
     auto column_of = [&](uint32_t j) -> uint32_t {
         const uint32_t jj = j < count ? j : count - 1;
         return __builtin_amdgcn_readlane(entries.y, jj - win);
@@ -422,7 +457,9 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     load_k(0, 0);
     load_v(0, 0);
     load_k(1, 1);
+    if (SLIM && t == 0) *retry_flag = 0;
 
+    const float c = p.scale_log2e, slack = p.slack;
     bf16x8 qf[KS];
     T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
     const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
@@ -433,7 +470,6 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
     RowState st = {kMaxSeed, kMaxSeed, 0.f};
-    const float c = p.scale_log2e, slack = p.slack;
 
     f32x16 s_even[KT], s_odd[KT];
     loads_landed();
@@ -445,6 +481,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         for (int ks = 0; ks < KS; ++ks)
             s_even[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(smem, k_lane, kt, ks), qf[ks], s_even[kt], 0, 0, 0);
     }
+    if constexpr (SLIM) st.m_used = st.m_true = block_row_max<KT>(s_even);
     __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
 
     auto iteration = [&](uint32_t j, f32x16 (&s)[KT], f32x16 (&s_next)[KT]) {
@@ -472,15 +509,17 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
                 if (__builtin_amdgcn_ballot_w64((keep & kAll) != kAll) != 0) apply_keep<KT>(s, keep, half);
             }
         }
-        const float mloc = block_row_max<KT>(s);
-        st.m_true = fmaxf(st.m_true, mloc);
-        if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
-            const float m_new = fmaxf(st.m_used, mloc);
-            const float alpha = exp2_fast((st.m_used - m_new) * c);
-            st.m_used = m_new;
-            st.l *= alpha;
+        if constexpr (!SLIM) {
+            const float mloc = block_row_max<KT>(s);
+            st.m_true = fmaxf(st.m_true, mloc);
+            if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
+                const float m_new = fmaxf(st.m_used, mloc);
+                const float alpha = exp2_fast((st.m_used - m_new) * c);
+                st.m_used = m_new;
+                st.l *= alpha;
 #pragma unroll
-            for (int n = 0; n < NO; ++n) o_acc[n] *= alpha;
+                for (int n = 0; n < NO; ++n) o_acc[n] *= alpha;
+            }
         }
         const float mc = st.m_used * c;
         float sum0 = 0.f, sum1 = 0.f;
@@ -522,7 +561,67 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
         if (j + 1 < count) iteration(j + 1, s_odd, s_even);
     }
 
+    if constexpr (SLIM) {
+        const float total = st.l + __shfl_xor(st.l, 32);
+        if (__builtin_amdgcn_ballot_w64(!(total < 0x1p100f)) != 0 && lane == 0) *retry_flag = 1;   // overflow, or NaN
+        __syncthreads();
+        if (*retry_flag != 0) return false;
+    }
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, smem);
+    return true;
+}
+
+template <int BS, int D, bool MASKED, bool PLANNED>
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int TILE = T::TILE_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+    __shared__ uint32_t retry_flag;
+    static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
+
+    const uint32_t lane = threadIdx.x & 63;
+    auto run = [&](const RowWork& w, sfb_uint2 window) {
+        if (w.count == 0) {
+            const uint32_t L = p.nb * BS, q_in_block = (threadIdx.x >> 6) * 32 + (lane & 31);
+            float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
+            store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
+            if (p.lse && (lane >> 5) == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
+            return;
+        }
+        if constexpr (!MASKED) {
+            if (attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window)) return;
+        }
+        attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window);
+    };
+    if constexpr (!PLANNED) {
+        const RowWork w = decode_row_work(p);
+        if (!w.valid) return;
+        run(w, lut_window(p, w, 0, lane));
+        return;
+    }
+    // Planned launch: this work-group stays resident and walks its own list of work items.  The list entry two
+    // items ahead and the first LUT window of the next item are requested before the current item starts and
+    // arrive while it is computed, so an item's first tile loads wait for nothing but themselves.  (Every list
+    // ends with two end marks.)
+    const PlanList mine = plan_list_of(p);
+    sfb_plan_entry e = mine[0];
+    if (e.count == kPlanEnd) return;
+    sfb_plan_entry e_next = mine[1];
+    RowWork w = plan_row_work(p, e);
+    sfb_uint2 window = lut_window(p, w, 0, lane);
+    for (uint32_t i = 2;; ++i) {
+        const bool more = e_next.count != kPlanEnd;
+        const RowWork w_next = plan_row_work(p, e_next);     // an end mark decodes to an item without key blocks
+        const sfb_uint2 window_next = more ? lut_window(p, w_next, 0, lane) : window;
+        e_next = mine[i];
+        run(w, window);
+        if (!more) break;
+        // the output rows left through the tiles' memory, which the next item's loads overwrite: every wave must
+        // have read its slab (LDS reads complete) before any wave goes on; the stores to memory may still be in flight
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        w = w_next;
+        window = window_next;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -530,18 +629,11 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
 // ------------------------------------------------------------------------------------------------
 // One LDS buffer (K tile and V tile); the next block waits in registers.
 template <int BS, int D>
-__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_kernel(FusedParams p) {
+__device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowWork& w, float* k_lds, float* v_lds) {
     using T = F32Tiles<BS, D>;
     constexpr int KT = BS / 32;
     constexpr int NO = D / 32;
     constexpr int QG = D / 8;        // float4 groups of Q per lane
-
-    __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
-    __shared__ __attribute__((aligned(16))) float v_lds[T::V_FLOATS];
-    static_assert(T::K_FLOATS * 4 >= BS * (D * 4 + 16), "the K tile's memory doubles as the output slabs");
-
-    const RowWork w = decode_row_work(p);
-    if (!w.valid) return;
     const uint32_t L = p.nb * BS;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint32_t qn = lane & 31, half = lane >> 5;
@@ -633,22 +725,48 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_ke
     finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, (uint8_t*)k_lds);
 }
 
+template <int BS, int D, bool PLANNED>
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_kernel(FusedParams p) {
+    using T = F32Tiles<BS, D>;
+    __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
+    __shared__ __attribute__((aligned(16))) float v_lds[T::V_FLOATS];
+    static_assert(T::K_FLOATS * 4 >= BS * (D * 4 + 16), "the K tile's memory doubles as the output slabs");
+    if constexpr (!PLANNED) {
+        const RowWork w = decode_row_work(p);
+        if (w.valid) attend_item_f32<BS, D>(p, w, k_lds, v_lds);
+        return;
+    }
+    // planned launch: a resident work-group walks its list of work items
+    const PlanList mine = plan_list_of(p);
+    sfb_plan_entry e = mine[0];
+    for (uint32_t i = 1; e.count != kPlanEnd; ++i) {
+        const sfb_plan_entry e_next = mine[i];
+        attend_item_f32<BS, D>(p, plan_row_work(p, e), k_lds, v_lds);
+        __syncthreads();   // the output rows left through the K tile's memory
+        e = e_next;
+    }
+}
+
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
-    const uint32_t grid = p.groups * 8u * ranks;
+    const uint32_t grid = p.plan ? ranks : p.groups * 8u * ranks;   // planned launches: ranks = resident work-groups
     clear_stale_error();
+    const bool masked = p.mask || p.valid_len, planned = p.plan != nullptr;
+    const dim3 g(grid), b(BS * 2);
     if (in_dtype == SFB_BF16) {
         if constexpr (D == 64) {
-            if (p.mask || p.valid_len)
-                fused_attention_bf16_kernel<BS, D, true><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
-            else
-                fused_attention_bf16_kernel<BS, D, false><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+            if (masked && planned) fused_attention_bf16_kernel<BS, D, true, true><<<g, b, 0, stream>>>(p);
+            else if (masked) fused_attention_bf16_kernel<BS, D, true, false><<<g, b, 0, stream>>>(p);
+            else if (planned) fused_attention_bf16_kernel<BS, D, false, true><<<g, b, 0, stream>>>(p);
+            else fused_attention_bf16_kernel<BS, D, false, false><<<g, b, 0, stream>>>(p);
         } else {
             return SFB_ERR_HEAD_STATE;   // the bf16 kernel is built for head size 64 only
         }
-    } else
-        fused_attention_f32_kernel<BS, D><<<dim3(grid), dim3(BS * 2), 0, stream>>>(p);
+    } else if (planned)
+        fused_attention_f32_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+    else
+        fused_attention_f32_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
     return launch_status();
 }
 
@@ -693,6 +811,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.lse = nullptr;
     p.nn_lut = nn_lut; p.mask = mask; p.valid_len = valid_len;
     p.row_order = nullptr; p.items = nullptr; p.counters = nullptr; p.partials = nullptr;
+    p.plan = nullptr; p.plan_stride = 0;
     p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
@@ -809,4 +928,39 @@ extern "C" int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void
     return fused_attention_scheduled(stream, q, k, v, o, lse, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
                                      n_items, n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
+}
+
+extern "C" int sfb_fused_attention_planned(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                           float* lse, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
+                                           const void* mask, const int32_t* valid_len, const sfb_plan_entry* plan,
+                                           uint32_t wg_slots, uint32_t plan_stride, uint32_t n_slots,
+                                           uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                           uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                           uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                           uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale) {
+    using namespace sfb;
+    const int rc = check_common(q, k, v, o, in_dtype, nn_lut, block_size, blocks, batch_dim, ctx_blks, head_dim,
+                                state_dim, lut_heads, lut_dim, mask_heads, scale);
+    if (rc != SFB_OK) return rc;
+    if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (!plan) return SFB_ERR_NULL_POINTER;
+    if (wg_slots == 0 || plan_stride < 3) return SFB_ERR_SHAPE;
+    if ((uintptr_t)plan & 15u) return SFB_ERR_ALIGNMENT;
+    const size_t need = sfb_schedule_workspace_bytes(n_slots, n_parts, batch_dim, head_dim, block_size, state_dim);
+    if (n_parts > 0 && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
+        return SFB_ERR_WORKSPACE;
+    FusedParams p;
+    fill_common(p, q, k, v, o, out_dtype, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
+                lut_heads, lut_dim, mask_heads, scale);
+    p.plan = plan;
+    p.plan_stride = plan_stride;
+    p.lse = lse;
+    p.n_slots = n_slots; p.n_parts = n_parts;
+    const size_t bh = (size_t)batch_dim * head_dim;
+    const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
+    p.counters = (uint32_t*)workspace;
+    p.partials = (float*)((uint8_t*)workspace + counters);
+    hipStream_t s = (hipStream_t)stream;
+    if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, wg_slots, state_dim);
+    return launch_fused_any<32>(s, p, in_dtype, wg_slots, state_dim);
 }

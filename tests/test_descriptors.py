@@ -165,3 +165,49 @@ def test_schedule_covers_every_block_once(max_blocks):
     assert not parts or (parts[0][0] == 0 and parts[-1][0] + parts[-1][1] == sched["n_parts"])
     nbytes = sfb.schedule_workspace_bytes(sched, 4, 12, 64, 64)
     assert nbytes == (4 * 12 * sched["n_slots"] * 4 + 255) // 256 * 256 + 4 * 12 * sched["n_parts"] * (64 * 64 + 256) * 4
+
+
+def test_plan_lists_cover_every_item_once():
+    nb, B, H = 64, 4, 12
+    luts = sfb.build_luts(sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234)))
+    plan = sfb.build_plan(luts["nn_lut"], nb, B, H, max_blocks=37, wg_slots=1024)
+    sched = sfb.build_schedule(luts["nn_lut"], nb, 37)
+    entries = plan["plan"]
+    assert entries.shape == (1024, plan["plan_stride"])
+    live = entries["count"] != sfb.PLAN_END
+    assert live.sum() == B * H * sched["n_items"]
+    assert (plan["n_slots"], plan["n_parts"]) == (sched["n_slots"], sched["n_parts"])
+    # every (batch, head) gets every work item of the schedule exactly once
+    fields = ("row", "first", "count", "nchunks", "chunk", "slot", "part", "lut_first")
+    want = sorted(tuple(int(it[f]) for f in fields) for it in sched["items"])
+    for b in range(B):
+        for h in range(H):
+            sel = live & (entries["batch"] == b) & (entries["head"] == h)
+            assert sorted(tuple(int(e[f]) for f in fields) for e in entries[sel]) == want
+    # live entries lead every list, followed by at least two end marks
+    assert (np.diff(live.astype(int), axis=1) <= 0).all() and not live[:, -2:].any()
+    # a (batch, head) only appears in the lists of slots of the same residue mod 8
+    slot = np.broadcast_to(np.arange(1024)[:, None], live.shape)
+    bh = entries["batch"] * H + entries["head"]
+    assert np.array_equal(slot[live] % 8, bh[live] % 8)
+    # the lists are balanced (key blocks + 2 per item) and the cut global rows lead their lists
+    loads = np.where(live, entries["count"].astype(np.int64) + 2, 0).sum(axis=1)
+    assert loads.max() <= loads.mean() + 10, (loads.max(), loads.mean())
+    assert (entries["count"][:, 1:][live[:, 1:]] <= 8).all()
+
+
+def test_plan_per_head_tables_and_odd_sizes():
+    nb, B, H = 16, 3, 4
+    lay = sfb.layout_fixed(H, nb, 4, causal=True)
+    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
+    nn = np.concatenate([p["nn_lut"] for p in per_head])
+    for wg_slots in (1, 7, 40):
+        plan = sfb.build_plan(nn, nb, B, H, max_blocks=2, lut_heads=H, wg_slots=wg_slots)
+        entries = plan["plan"]
+        live = entries["count"] != sfb.PLAN_END
+        for h in range(H):
+            sched = sfb.build_schedule(per_head[h]["nn_lut"], nb, 2)
+            sel = live & (entries["head"] == h)
+            assert sel.sum() == B * sched["n_items"]
+            assert sorted(entries["lut_first"][sel & (entries["batch"] == 0)]) == sorted(sched["items"]["lut_first"])
+        assert not live[:, -2:].any()
