@@ -36,7 +36,8 @@ typedef enum {
     SFB_ERR_ALIGNMENT = 6,      /* a tensor pointer is not 16-byte aligned */
     SFB_ERR_LAUNCH = 7,         /* hipGetLastError() reported a failure after the launch */
     SFB_ERR_ARGUMENT = 8,       /* other invalid argument (op code, pattern parameter ...) */
-    SFB_ERR_WORKSPACE = 9       /* workspace missing or too small */
+    SFB_ERR_WORKSPACE = 9,      /* workspace missing or too small */
+    SFB_ERR_SCRATCH_LIMIT = 10  /* the launch needs more scratch than the library's static device array holds */
 } sfb_status;
 
 typedef enum { SFB_F32 = 0, SFB_BF16 = 1 } sfb_dtype;
@@ -211,6 +212,24 @@ int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const v
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
+/* No counterpart in the reference.  For callers that cannot allocate device memory or pass a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The same launch as
+ * sfb_fused_attention_scheduled_to, with the arrival counters and partial records of split rows kept in a static
+ * device array of SFB_STATIC_SCRATCH_BYTES inside the library (each device the library runs on holds one until the
+ * process ends) instead of a caller's workspace; the call allocates nothing.  A launch whose
+ * sfb_schedule_workspace_bytes() exceeds SFB_STATIC_SCRATCH_BYTES returns SFB_ERR_SCRATCH_LIMIT (BigBird L = 4096,
+ * 12 heads, head size 64 needs 0.8 MiB per sequence while its global rows are cut, nothing from 8 sequences on).
+ * All calls on one device share the array: calls that overlap in time on one device (two streams, two threads)
+ * race and must be ordered by the caller. */
+#define SFB_STATIC_SCRATCH_BYTES (8u << 20)
+size_t sfb_static_scratch_bytes(void);
+int sfb_fused_attention_scheduled_noalloc(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                          int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                          const int32_t* valid_len, const sfb_work_item* items, uint32_t n_items,
+                                          uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts, uint32_t block_size,
+                                          uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                          uint32_t state_dim, uint32_t mask_heads, float scale);
+
 /* The same launch for a training step: additionally writes lse [dev] fp32 [batch][heads][ctx], the base-2
  * logarithm of each query row's softmax denominator in units where the normalised probability of a key with raw
  * score s is exp2(s * scale * log2(e) - lse).  sfb_fused_attention_backward rebuilds P from it. */

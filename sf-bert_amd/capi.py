@@ -52,6 +52,7 @@ lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
 lib.sfb_resident_work_groups.restype = C.c_uint32
+lib.sfb_static_scratch_bytes.restype = C.c_size_t
 
 #: every symbol include/sfbert_hip.h declares (checked by the CPU test-suite)
 EXPORTED = [
@@ -62,6 +63,7 @@ EXPORTED = [
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
     "sfb_build_plan", "sfb_resident_work_groups", "sfb_fused_attention_planned",
+    "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",

@@ -59,6 +59,7 @@ const char* sfb_status_string(int status) {
         case SFB_ERR_LAUNCH: return "kernel launch failed";
         case SFB_ERR_ARGUMENT: return "invalid argument";
         case SFB_ERR_WORKSPACE: return "workspace missing or too small";
+        case SFB_ERR_SCRATCH_LIMIT: return "the launch needs more scratch than the library's static device array holds";
         default: return "unknown status";
     }
 }

@@ -17,6 +17,8 @@
 // by sum + 1e-6 (ewops.h:93), and O = P.V (matmul.h:6-20).
 #include "tiles.hip.h"
 
+#include <mutex>
+
 namespace sfb {
 
 struct FusedParams {
@@ -963,4 +965,80 @@ extern "C" int sfb_fused_attention_planned(sfb_stream_t stream, const void* q, c
     hipStream_t s = (hipStream_t)stream;
     if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, wg_slots, state_dim);
     return launch_fused_any<32>(s, p, in_dtype, wg_slots, state_dim);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Scheduled launch that allocates nothing: the arrival counters and partial records of split rows live in a
+// static device array instead of a caller's workspace.
+// ------------------------------------------------------------------------------------------------
+namespace sfb {
+
+constexpr size_t kStaticScratchBytes = SFB_STATIC_SCRATCH_BYTES;
+// Every device the library runs on holds its own copy of this array until the process ends.  In host code the
+// name is only a handle for hipGetSymbolAddress; kernels and fills get the device address kept in scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* scratch_ptr[kMaxDevices];   // device address of `scratch` on each device, looked up on first use
+static std::mutex scratch_mutex;
+
+// Device address of the current device's copy of `scratch`.
+static int static_scratch(void** out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) {
+        (void)hipGetLastError();
+        return SFB_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[device] == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            return SFB_ERR_LAUNCH;
+        }
+        scratch_ptr[device] = ptr;
+    }
+    *out = scratch_ptr[device];
+    return SFB_OK;
+}
+
+// Fill kernel (a captured graph must not hold a memset node): words[0 .. n) = 0.
+__global__ void clear_words_kernel(uint32_t* words, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0u;
+}
+
+}  // namespace sfb
+
+extern "C" size_t sfb_static_scratch_bytes(void) { return sfb::kStaticScratchBytes; }
+
+extern "C" int sfb_fused_attention_scheduled_noalloc(sfb_stream_t stream, const void* q, const void* k, const void* v,
+                                                     void* o, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
+                                                     const void* mask, const int32_t* valid_len,
+                                                     const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                                                     uint32_t n_slots, uint32_t n_parts, uint32_t block_size,
+                                                     uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
+                                                     uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
+                                                     float scale) {
+    using namespace sfb;
+    // the largest launch this entry point takes: its counters and partial records must fit the static array
+    const size_t need = sfb_schedule_workspace_bytes(n_slots, n_parts, batch_dim, head_dim, block_size, state_dim);
+    if (need > kStaticScratchBytes) return SFB_ERR_SCRATCH_LIMIT;
+    void* ptr = nullptr;
+    const int rc = static_scratch(&ptr);
+    if (rc != SFB_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    // The array keeps what the previous call on this device left in it.  Partial records are written before they
+    // are read; the arrival counters must start at zero, so they are cleared here (a launch that ran to its end
+    // leaves them at zero, one that was cut short need not).
+    const size_t counter_words = (size_t)batch_dim * head_dim * n_slots;
+    if (n_parts > 0 && counter_words > 0) {
+        clear_stale_error();
+        clear_words_kernel<<<dim3((unsigned)((counter_words + 255) / 256)), dim3(256), 0, s>>>((uint32_t*)ptr,
+                                                                                             (uint32_t)counter_words);
+        if (launch_status() != SFB_OK) return SFB_ERR_LAUNCH;
+    }
+    return fused_attention_scheduled(stream, q, k, v, o, nullptr, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
+                                     n_items, n_heavy, n_slots, n_parts, ptr, kStaticScratchBytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
 }
