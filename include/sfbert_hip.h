@@ -2,8 +2,13 @@
  * libsfbert_hip -- C ABI of the MI355X (gfx950) block-sparse attention path.
  *
  * Plain pointers and sizes only.  Device pointers are marked [dev], host pointers [host].  Every
- * device entry point enqueues work on the given HIP stream and returns without synchronising; it
- * allocates nothing and keeps no state.  Tensors Q/K/V/O are [batch, ctx, heads, head_state]
+ * device entry point enqueues work on the given HIP stream and returns without synchronising.  The
+ * attention and layer-op entry points allocate nothing and keep no state.  The GEMM entry points
+ * (sfb_gemm*, sfb_encoder_layer_forward*, sfb_model_forward) go through rocBLAS / hipBLASLt: the
+ * library keeps one handle of each per process and one plan per GEMM problem, made on first use
+ * behind one mutex and kept until sfb_gemm_release(); making a plan times the library's candidate
+ * kernels on the caller's operands, which synchronises with the stream once (skipped when the
+ * stream is being captured into a graph).  Tensors Q/K/V/O are [batch, ctx, heads, head_state]
  * contiguous (element offset b*ctx*H*d + token*H*d + h*d + k), sparse S/P tensors are
  * [batch][heads][blocks][bs][bs], exactly as the reference lays them out
  * (openai_blocksparse.h:40-41,148).  Each declaration cites the reference interface it replaces.
@@ -403,6 +408,10 @@ int sfb_embedding_lookup(sfb_stream_t stream, float* out, const float* table, co
 /* fp32 -> bf16, round to nearest even (the reference's to_bhalf, ew_op_gpu.h:241-254, rounds half
  * away from zero; inputs of the bf16 configurations are defined as RNE-rounded); n % 4 == 0. */
 int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in, uint64_t n);
+
+/* Destroys the GEMM plans and the rocBLAS / hipBLASLt handles the GEMM entry points made (they are made again on
+ * the next use).  Call it when no GEMM of this library is in flight. */
+void sfb_gemm_release(void);
 
 /* cblas_sgemm(RowMajor, NoTrans, NoTrans, m, n, k, 1, A, k, W, n, 0, C, n) (transformer.cpp:516-522, 547,
  * 562, 571; cublasSgemm twins transformer_attention_optimize.cu:693-716): C[m][n] = A[m][k] W[k][n],

@@ -30,39 +30,77 @@ rocblas_handle blas_handle() {
 }
 
 inline size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+constexpr size_t kGemmWorkspaceBytes = 32u << 20;
 
-// GEMM with the bias add, optionally the activation, and the output conversion in its epilogue (hipBLASLt).  One
-// plan per problem shape, made on first use and kept; no workspace is requested, so nothing is allocated on the
-// device.  The activation is the reference's sigmoid form of GELU, x / (1 + exp(-1.702 x)) (ewops.h:32-43), which
-// is the library's Swish epilogue with its argument set to 1.702.
+// GEMM with, optionally, the bias add, the activation and the output conversion in its epilogue (hipBLASLt).  One
+// plan per problem (shape, element types, epilogue, whether a workspace is on offer), made on first use and kept
+// until sfb_gemm_release().  Making a plan asks the library for up to kCandidates kernels that fit the offered
+// workspace and -- unless the stream is being captured into a graph -- times each of them once on the caller's own
+// operands (the products all write the same result) and keeps the fastest; under capture the library's first
+// choice is taken.  The activation is the reference's sigmoid form of GELU, x / (1 + exp(-1.702 x))
+// (ewops.h:32-43), which is the library's Swish epilogue with its argument set to 1.702.
 struct LtPlan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
     hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;     // bytes the chosen kernel wants
     bool usable = false;
     bool slope_set = false;   // activation plans: the library took the GELU slope as the Swish argument
+    bool tuned = false;       // candidates were timed (false: first choice taken under graph capture)
 };
 hipblasLtHandle_t g_lt = nullptr;
-std::map<std::tuple<uint32_t, uint32_t, uint32_t, int, int, int>, LtPlan> g_plans;
+typedef std::tuple<uint32_t, uint32_t, uint32_t, int, int, int, int, int> PlanKey;
+std::map<PlanKey, LtPlan> g_plans;
 constexpr float kGeluSigmoidSlope = 1.702f;
+constexpr int kCandidates = 16;
 
-// row-major C[m][n] = A[m][k] W[k][n] + bias[n]  ==  column-major D[n][m] = W'[n][k] A'[k][m] + bias (per row of D)
-LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, int act) {
-    const auto key = std::make_tuple(m, n, k, dtype, out_dtype, act);
+void destroy_plan(LtPlan& p) {
+    if (p.w) hipblasLtMatrixLayoutDestroy(p.w);
+    if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    p = LtPlan();
+}
+
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) { (void)hipGetLastError(); return true; }
+    return status != hipStreamCaptureStatusNone;
+}
+
+// Operands of the call that makes a plan: the candidates are timed on them.
+struct LtOperands {
+    hipStream_t stream;
+    void* c;
+    const void* a;
+    const void* w;
+    const float* bias;
+    void* workspace;
+    size_t workspace_bytes;
+};
+
+// row-major C[m][n] = A[m][k] W[k][n] (+ bias[n])  ==  column-major D[n][m] = W'[n][k] A'[k][m] (+ bias per row of D)
+// act: 0 none, 1 sigmoid-GELU (needs a bias); epilogue without bias when ops.bias is null
+LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, int act, const LtOperands& ops) {
+    const int with_bias = ops.bias != nullptr, with_ws = ops.workspace != nullptr && ops.workspace_bytes > 0;
+    const PlanKey key = std::make_tuple(m, n, k, dtype, out_dtype, act, with_bias, with_ws);
     auto it = g_plans.find(key);
     if (it != g_plans.end()) return it->second;
     LtPlan& p = g_plans[key];
     if (!g_lt && hipblasLtCreate(&g_lt) != HIPBLAS_STATUS_SUCCESS) { g_lt = nullptr; return p; }
+    if (act && !with_bias) return p;
     const hipDataType in = dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
     const hipDataType out = out_dtype == SFB_BF16 ? HIP_R_16BF : HIP_R_32F;
     const hipblasOperation_t none = HIPBLAS_OP_N;
-    const hipblasLtEpilogue_t epilogue = act ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT : HIPBLASLT_EPILOGUE_BIAS;
+    const hipblasLtEpilogue_t epilogue = act ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT
+                                             : (with_bias ? HIPBLASLT_EPILOGUE_BIAS : HIPBLASLT_EPILOGUE_DEFAULT);
     const hipDataType bias_type = HIP_R_32F;
     bool ok = hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &none, sizeof(none)) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epilogue, sizeof(epilogue)) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
+    if (with_bias)
+        ok = ok && hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
     // older builds of the library have the Swish epilogue but not its slope argument: there the slope stays 1 and
     // the caller scales the operands instead (see gemm_bias_gelu_scaled)
     if (ok && act)
@@ -72,21 +110,55 @@ LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, in
     ok = ok && hipblasLtMatrixLayoutCreate(&p.a, in, k, m, k) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && hipblasLtMatrixLayoutCreate(&p.c, out, n, m, n) == HIPBLAS_STATUS_SUCCESS;
     if (!ok) return p;
-    // the heuristic needs a bias pointer to be present in the descriptor; the real one is set per call
-    const void* placeholder = &p;
-    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &placeholder, sizeof(placeholder));
+    // the heuristic needs the bias pointer to be present in the descriptor; it is set again on every call
+    if (with_bias) {
+        const void* bias_ptr = ops.bias;
+        hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr));
+    }
     hipblasLtMatmulPreference_t pref = nullptr;
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
-    const uint64_t no_workspace = 0;
-    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &no_workspace, sizeof(no_workspace));
-    hipblasLtMatmulHeuristicResult_t result;
+    const uint64_t max_ws = with_ws ? ops.workspace_bytes : 0;
+    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+    hipblasLtMatmulHeuristicResult_t results[kCandidates];
     int found = 0;
-    if (hipblasLtMatmulAlgoGetHeuristic(g_lt, p.desc, p.w, p.a, p.c, p.c, pref, 1, &result, &found) == HIPBLAS_STATUS_SUCCESS &&
-        found > 0 && result.workspaceSize == 0) {
-        p.algo = result.algo;
-        p.usable = true;
-    }
+    const bool got = hipblasLtMatmulAlgoGetHeuristic(g_lt, p.desc, p.w, p.a, p.c, p.c, pref, kCandidates, results, &found) ==
+                     HIPBLAS_STATUS_SUCCESS;
     hipblasLtMatmulPreferenceDestroy(pref);
+    if (!got || found <= 0) return p;
+    int best = -1;
+    if (!stream_is_capturing(ops.stream) && ops.c && ops.a && ops.w) {
+        // time every candidate on the caller's operands: 1 untimed + 3 timed launches each
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+            const float alpha = 1.0f, beta = 0.0f;
+            float best_ms = 0.f;
+            for (int i = 0; i < found; ++i) {
+                if (results[i].state != HIPBLAS_STATUS_SUCCESS || results[i].workspaceSize > max_ws) continue;
+                bool ran = true;
+                for (int rep = 0; rep < 4 && ran; ++rep) {
+                    if (rep == 1) ran = hipEventRecord(e0, ops.stream) == hipSuccess;
+                    ran = ran && hipblasLtMatmul(g_lt, p.desc, &alpha, ops.w, p.w, ops.a, p.a, &beta, ops.c, p.c, ops.c, p.c,
+                                                 &results[i].algo, ops.workspace, results[i].workspaceSize,
+                                                 ops.stream) == HIPBLAS_STATUS_SUCCESS;
+                }
+                float ms = 0.f;
+                ran = ran && hipEventRecord(e1, ops.stream) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+                      hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+                if (!ran) { (void)hipGetLastError(); continue; }
+                if (best < 0 || ms < best_ms) { best = i; best_ms = ms; }
+            }
+            p.tuned = best >= 0;
+        }
+        if (e0) hipEventDestroy(e0);
+        if (e1) hipEventDestroy(e1);
+    }
+    if (best < 0)
+        for (int i = 0; i < found && best < 0; ++i)
+            if (results[i].state == HIPBLAS_STATUS_SUCCESS && results[i].workspaceSize <= max_ws) best = i;
+    if (best < 0) return p;
+    p.algo = results[best].algo;
+    p.workspace = results[best].workspaceSize;
+    p.usable = true;
     return p;
 }
 
@@ -112,35 +184,45 @@ static int gemm_alpha(sfb_stream_t stream, float* c, const void* a, const void* 
     return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
 }
 
-extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
-                        uint32_t n, uint32_t k) {
-    return gemm_alpha(stream, c, a, w, dtype, m, n, k, 1.0f);
-}
-
-// C = act(alpha A W + bias) through one library GEMM; SFB_ERR_LAUNCH when the library has no kernel for it.
-// act = 1 without the slope argument (*slope_set false) computes Swish with slope 1.
-static int gemm_bias_epilogue(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
-                              const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k, int act,
-                              float alpha_unless_slope_set = 1.0f, bool* slope_set = nullptr) {
+// C = act(alpha A W (+ bias)) through one library GEMM; SFB_ERR_LAUNCH when the library has no kernel for it.
+// act = 1 without the slope argument (*slope_set false) computes Swish with slope 1.  workspace (may be null):
+// device memory the library's kernels may use.
+static int lt_gemm(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w, const float* bias,
+                   int dtype, uint32_t m, uint32_t n, uint32_t k, int act, float alpha, void* workspace,
+                   size_t workspace_bytes, bool* slope_set = nullptr, bool scale_unless_slope_set = false) {
     std::lock_guard<std::mutex> lock(g_mutex);
-    LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, act);
+    const LtOperands ops = {(hipStream_t)stream, c, a, w, bias, workspace, workspace_bytes};
+    LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, act, ops);
     if (!p.usable) return SFB_ERR_LAUNCH;
     if (slope_set) *slope_set = p.slope_set;
-    const float alpha = (act && !p.slope_set) ? alpha_unless_slope_set : 1.0f, beta = 0.0f;
+    if (scale_unless_slope_set && p.slope_set) alpha = 1.0f;
+    const float beta = 0.0f;
     const void* bias_ptr = bias;
-    if (hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) ==
-            HIPBLAS_STATUS_SUCCESS &&
-        hipblasLtMatmul(g_lt, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo, nullptr, 0,
+    if ((bias == nullptr ||
+         hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias_ptr, sizeof(bias_ptr)) ==
+             HIPBLAS_STATUS_SUCCESS) &&
+        hipblasLtMatmul(g_lt, p.desc, &alpha, w, p.w, a, p.a, &beta, c, p.c, c, p.c, &p.algo, workspace, p.workspace,
                         (hipStream_t)stream) == HIPBLAS_STATUS_SUCCESS)
         return SFB_OK;
     p.usable = false;   // do not try this plan again
     return SFB_ERR_LAUNCH;
 }
 
-// whether the activation plan of this shape exists and has its slope set (made on first use)
-static bool gelu_plan_state(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, bool* slope_set) {
+extern "C" void sfb_gemm_release(void) {
     std::lock_guard<std::mutex> lock(g_mutex);
-    const LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, 1);
+    for (auto& kv : g_plans) destroy_plan(kv.second);
+    g_plans.clear();
+    if (g_lt) { hipblasLtDestroy(g_lt); g_lt = nullptr; }
+    if (g_handle) { rocblas_destroy_handle(g_handle); g_handle = nullptr; }
+}
+
+// whether the activation plan of this shape exists and has its slope set (made on first use, on these operands)
+static bool gelu_plan_state(sfb_stream_t stream, void* c, const void* a, const void* w, const float* bias, uint32_t m,
+                            uint32_t n, uint32_t k, int dtype, int out_dtype, void* workspace, size_t workspace_bytes,
+                            bool* slope_set) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    const LtOperands ops = {(hipStream_t)stream, c, a, w, bias, workspace, workspace_bytes};
+    const LtPlan& p = lt_plan(m, n, k, dtype, out_dtype, 1, ops);
     *slope_set = p.slope_set;
     return p.usable;
 }
@@ -150,17 +232,37 @@ __global__ __launch_bounds__(256) void scale_vector_kernel(float* out, const flo
     if (i < n) out[i] = in[i] * factor;
 }
 
-extern "C" int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
-                             const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k) {
+// c = alpha (a w): the tuned library kernel where there is one, else rocBLAS
+static int gemm_ws(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m, uint32_t n,
+                   uint32_t k, float alpha, void* ws, size_t ws_bytes) {
+    if (!c || !a || !w) return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (!m || !n || !k) return SFB_ERR_SHAPE;
+    if (lt_gemm(stream, c, SFB_F32, a, w, nullptr, dtype, m, n, k, 0, alpha, ws, ws_bytes) == SFB_OK) return SFB_OK;
+    return gemm_alpha(stream, c, a, w, dtype, m, n, k, alpha);
+}
+
+extern "C" int sfb_gemm(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
+                        uint32_t n, uint32_t k) {
+    return gemm_ws(stream, c, a, w, dtype, m, n, k, 1.0f, nullptr, 0);
+}
+
+static int gemm_bias_ws(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w, const float* bias,
+                        int dtype, uint32_t m, uint32_t n, uint32_t k, void* ws, size_t ws_bytes) {
     if (!c || !a || !w || !bias) return SFB_ERR_NULL_POINTER;
     if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
     if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
-    if (gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 0) == SFB_OK) return SFB_OK;
+    if (lt_gemm(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 0, 1.0f, ws, ws_bytes) == SFB_OK) return SFB_OK;
     // no fused kernel for this shape: plain GEMM, then the bias pass.  The fp32 product needs room: in place for
     // fp32 output, otherwise there is none here
     if (out_dtype != SFB_F32) return SFB_ERR_LAUNCH;
-    const int rc = sfb_gemm(stream, (float*)c, a, w, dtype, m, n, k);
+    const int rc = gemm_ws(stream, (float*)c, a, w, dtype, m, n, k, 1.0f, ws, ws_bytes);
     return rc != SFB_OK ? rc : sfb_bias_act(stream, c, SFB_F32, (const float*)c, bias, nullptr, 0, m, n);
+}
+
+extern "C" int sfb_gemm_bias(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
+                             const float* bias, int dtype, uint32_t m, uint32_t n, uint32_t k) {
+    return gemm_bias_ws(stream, c, out_dtype, a, w, bias, dtype, m, n, k, nullptr, 0);
 }
 
 extern "C" int sfb_gemm_bias_gelu(sfb_stream_t stream, void* c, int out_dtype, const void* a, const void* w,
@@ -170,32 +272,38 @@ extern "C" int sfb_gemm_bias_gelu(sfb_stream_t stream, void* c, int out_dtype, c
     if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
     if (c == a) return SFB_ERR_ARGUMENT;
     bool slope_set = false;
-    if (gelu_plan_state(m, n, k, dtype, out_dtype, &slope_set) && slope_set &&
-        gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1) == SFB_OK)
+    if (gelu_plan_state(stream, c, a, w, bias, m, n, k, dtype, out_dtype, nullptr, 0, &slope_set) && slope_set &&
+        lt_gemm(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1, 1.0f, nullptr, 0) == SFB_OK)
         return SFB_OK;
     if (out_dtype != SFB_F32) return SFB_ERR_LAUNCH;
     const int rc = sfb_gemm(stream, (float*)c, a, w, dtype, m, n, k);
     return rc != SFB_OK ? rc : sfb_bias_act(stream, c, SFB_F32, (const float*)c, bias, nullptr, 1, m, n);
 }
 
-extern "C" int sfb_gemm_bias_gelu_scaled(sfb_stream_t stream, void* c, int out_dtype, float* scale,
-                                         float* bias_scratch, const void* a, const void* w, const float* bias,
-                                         int dtype, uint32_t m, uint32_t n, uint32_t k) {
+static int gemm_bias_gelu_scaled_ws(sfb_stream_t stream, void* c, int out_dtype, float* scale, float* bias_scratch,
+                                    const void* a, const void* w, const float* bias, int dtype, uint32_t m, uint32_t n,
+                                    uint32_t k, void* ws, size_t ws_bytes) {
     if (!c || !a || !w || !bias || !scale || !bias_scratch) return SFB_ERR_NULL_POINTER;
     if ((dtype != SFB_F32 && dtype != SFB_BF16) || (out_dtype != SFB_F32 && out_dtype != SFB_BF16)) return SFB_ERR_DTYPE;
     if (!m || !n || !k || (n & 3u)) return SFB_ERR_SHAPE;
     if (c == a) return SFB_ERR_ARGUMENT;
     bool slope_set = false;
-    if (!gelu_plan_state(m, n, k, dtype, out_dtype, &slope_set)) return SFB_ERR_LAUNCH;
+    if (!gelu_plan_state(stream, c, a, w, bias, m, n, k, dtype, out_dtype, ws, ws_bytes, &slope_set)) return SFB_ERR_LAUNCH;
     *scale = 1.0f;
-    if (slope_set) return gemm_bias_epilogue(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1);
+    if (slope_set) return lt_gemm(stream, c, out_dtype, a, w, bias, dtype, m, n, k, 1, 1.0f, ws, ws_bytes);
     // x / (1 + exp(-s x)) = Swish_1(s x) / s: the product and the bias are scaled by s going in, and the result is
     // left s times too large for the caller to fold into what it does next
     (void)hipGetLastError();   // only this launch is reported
     scale_vector_kernel<<<dim3((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(bias_scratch, bias, kGeluSigmoidSlope, n);
     if (hipGetLastError() != hipSuccess) return SFB_ERR_LAUNCH;
     *scale = kGeluSigmoidSlope;
-    return gemm_bias_epilogue(stream, c, out_dtype, a, w, bias_scratch, dtype, m, n, k, 1, kGeluSigmoidSlope);
+    return lt_gemm(stream, c, out_dtype, a, w, bias_scratch, dtype, m, n, k, 1, kGeluSigmoidSlope, ws, ws_bytes);
+}
+
+extern "C" int sfb_gemm_bias_gelu_scaled(sfb_stream_t stream, void* c, int out_dtype, float* scale,
+                                         float* bias_scratch, const void* a, const void* w, const float* bias,
+                                         int dtype, uint32_t m, uint32_t n, uint32_t k) {
+    return gemm_bias_gelu_scaled_ws(stream, c, out_dtype, scale, bias_scratch, a, w, bias, dtype, m, n, k, nullptr, 0);
 }
 
 extern "C" int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const void* w, int dtype, uint32_t m,
@@ -225,7 +333,13 @@ extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t
     // bf16 path only: xa (activation in compute dtype, m x max(n, ffn)); ffn floats of bias scratch
     size_t bytes = align256(m * (ffn > n ? ffn : n) * f32) + 3 * align256(m * n * act) + 2 * align256(m * n * f32);
     if (dtype == SFB_BF16) bytes += align256(m * (ffn > n ? ffn : n) * act);
-    return bytes + align256(ffn * f32);   // scaled copy of the first FFN bias (sfb_gemm_bias_gelu_scaled)
+    bytes += align256(ffn * f32);   // scaled copy of the first FFN bias (sfb_gemm_bias_gelu_scaled)
+    return bytes + kGemmWorkspaceBytes;   // scratch for the GEMM library's kernels
+}
+
+// Scratch offered to the GEMM library's kernels at the end of a layer's workspace
+static void* gemm_scratch(const float* bias_scratch, uint32_t ffn) {
+    return (uint8_t*)bias_scratch + align256((size_t)ffn * sizeof(float));
 }
 
 // Everything a layer needs besides its input, output and weights
@@ -246,9 +360,10 @@ struct LayerArgs {
 // out = a W + bias in the compute dtype: one GEMM with the bias in its epilogue, or, where that is not available,
 // GEMM into the fp32 scratch t followed by the bias pass
 static int project(sfb_stream_t stream, void* out, int out_dtype, float* t, const void* a, const void* w,
-                   const float* bias, int dtype, size_t m, uint32_t n, uint32_t k) {
-    if (sfb_gemm_bias(stream, out, out_dtype, a, w, bias, dtype, (uint32_t)m, n, k) == SFB_OK) return SFB_OK;
-    const int rc = sfb_gemm(stream, t, a, w, dtype, (uint32_t)m, n, k);
+                   const float* bias, int dtype, size_t m, uint32_t n, uint32_t k, void* ws) {
+    if (gemm_bias_ws(stream, out, out_dtype, a, w, bias, dtype, (uint32_t)m, n, k, ws, kGemmWorkspaceBytes) == SFB_OK)
+        return SFB_OK;
+    const int rc = gemm_ws(stream, t, a, w, dtype, (uint32_t)m, n, k, 1.0f, ws, kGemmWorkspaceBytes);
     return rc != SFB_OK ? rc : sfb_bias_act(stream, out, out_dtype, t, bias, nullptr, 0, m, n);
 }
 
@@ -308,18 +423,19 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     void* xa = bf ? (void*)p : nullptr;
     if (bf) p += align256(m * wide * act);
     float* bias_scratch = (float*)p;
+    void* const gws = gemm_scratch(bias_scratch, ffn);
     int rc;
 #define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
     // LN1 straight into the compute dtype; the fp32 path borrows the attention output buffer, which is free
     // until the attention runs
     void* a = bf ? xa : (void*)attn;
     SFB_TRY(sfb_layernorm(stream, a, dtype, nullptr, nullptr, x, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
-    SFB_TRY(project(stream, q, dtype, t, a, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(project(stream, k, dtype, t, a, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(project(stream, v, dtype, t, a, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, q, dtype, t, a, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+    SFB_TRY(project(stream, k, dtype, t, a, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+    SFB_TRY(project(stream, v, dtype, t, a, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
     const void* ain = nullptr;
     SFB_TRY(attention_operand(stream, g, q, k, v, attn, xa, m * n, &ain));
-    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n, gws));
     SFB_TRY(sfb_bias_act(stream, x1, SFB_F32, t, nullptr, x, 0, m, (uint32_t)n));
     // LN2 into the compute dtype (fp32: the attention output buffer again, consumed by the GEMM above)
     void* a2 = bf ? xa : (void*)attn;
@@ -327,15 +443,15 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     void* gl = t;
     float* t2 = attn;
     float g_scale = 1.0f;
-    if (sfb_gemm_bias_gelu_scaled(stream, t, dtype, &g_scale, bias_scratch, a2, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
-                                  (uint32_t)n) != SFB_OK) {
-        SFB_TRY(sfb_gemm(stream, t, a2, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+    if (gemm_bias_gelu_scaled_ws(stream, t, dtype, &g_scale, bias_scratch, a2, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
+                                 (uint32_t)n, gws, kGemmWorkspaceBytes) != SFB_OK) {
+        SFB_TRY(gemm_ws(stream, t, a2, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n, 1.0f, gws, kGemmWorkspaceBytes));
         gl = bf ? xa : (void*)t;
         SFB_TRY(sfb_bias_act(stream, gl, dtype, t, wt->b1, nullptr, 1, m, ffn));
         t2 = bf ? t : attn;
         g_scale = 1.0f;
     }
-    SFB_TRY(gemm_alpha(stream, t2, gl, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale));
+    SFB_TRY(gemm_ws(stream, t2, gl, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale, gws, kGemmWorkspaceBytes));
     SFB_TRY(sfb_bias_act(stream, y, SFB_F32, t2, wt->b2, x1, 0, m, (uint32_t)n));
 #undef SFB_TRY
     return SFB_OK;
@@ -398,6 +514,7 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     void* xa = bf ? (void*)p : nullptr;
     if (bf) p += align256(m * wide * act);
     float* bias_scratch = (float*)p;
+    void* const gws = gemm_scratch(bias_scratch, ffn);
     const float scale = 1.0f / sqrtf((float)state_dim);
     int rc;
 #define SFB_TRY(call) do { rc = (call); if (rc != SFB_OK) return rc; } while (0)
@@ -405,9 +522,9 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     // Q, K, V projections (+ bias), stored in the compute dtype for the attention kernel
     const void* xin = x;
     if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x, m * n)); xin = xa; }
-    SFB_TRY(project(stream, q, dtype, t, xin, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(project(stream, k, dtype, t, xin, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n));
-    SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, q, dtype, t, xin, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+    SFB_TRY(project(stream, k, dtype, t, xin, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+    SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
 
     // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
     const LayerArgs args = {dtype, nn_lut, mask, valid_len, items, n_items, n_heavy, n_slots, n_parts, attn_workspace,
@@ -417,7 +534,7 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     SFB_TRY(attention_operand(stream, args, q, k, v, attn, xa, m * n, &ain));
 
     // output projection + bias, residual, LayerNorm 1
-    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n));
+    SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n, gws));
     // residual + LayerNorm 1 in one pass when the row fits in registers; the bf16 path gets its copy of x1
     // for the next GEMM from the same kernel
     const bool fused_ln = n <= 2048;
@@ -440,15 +557,15 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     void* g = t;                    // activation after GELU (times g_scale), in the compute dtype
     float* t2 = attn;               // the second FFN GEMM reads g and must not write over it
     float g_scale = 1.0f;
-    if (sfb_gemm_bias_gelu_scaled(stream, t, dtype, &g_scale, bias_scratch, fin, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
-                                  (uint32_t)n) != SFB_OK) {
-        SFB_TRY(sfb_gemm(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n));
+    if (gemm_bias_gelu_scaled_ws(stream, t, dtype, &g_scale, bias_scratch, fin, wt->w1, wt->b1, dtype, (uint32_t)m, ffn,
+                                 (uint32_t)n, gws, kGemmWorkspaceBytes) != SFB_OK) {
+        SFB_TRY(gemm_ws(stream, t, fin, wt->w1, dtype, (uint32_t)m, ffn, (uint32_t)n, 1.0f, gws, kGemmWorkspaceBytes));
         g = bf ? xa : (void*)t;     // in place for fp32
         SFB_TRY(sfb_bias_act(stream, g, dtype, t, wt->b1, nullptr, 1, m, ffn));
         t2 = bf ? t : attn;
         g_scale = 1.0f;
     }
-    SFB_TRY(gemm_alpha(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale));
+    SFB_TRY(gemm_ws(stream, t2, g, wt->w2, dtype, (uint32_t)m, (uint32_t)n, ffn, 1.0f / g_scale, gws, kGemmWorkspaceBytes));
     if (fused_ln) {
         SFB_TRY(sfb_bias_residual_layernorm(stream, y, nullptr, t2, wt->b2, x1, wt->ln2_g, wt->ln2_b, (uint32_t)m,
                                             (uint32_t)n));

@@ -392,6 +392,33 @@ __device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[
     sum1 = dot2_bf16_ones(e, sum1);
 }
 
+// The same for scores that already are base-2 exponents (scale and offset folded into the score product): one
+// exponential per element and nothing else; the row sum is taken over the fp32 values with plain additions, which --
+// unlike v_dot2c -- run while the matrix pipe is busy.
+template <int KT>
+__device__ __forceinline__ void exp_chunk_slim(const f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], int u, float& sum0,
+                                               float& sum1) {
+    const int kt = u / 2, i0 = (u % 2) * 8;
+    const float p0 = exp2_fast(s[kt][i0 + 0]), p1 = exp2_fast(s[kt][i0 + 1]);
+    const float p2 = exp2_fast(s[kt][i0 + 2]), p3 = exp2_fast(s[kt][i0 + 3]);
+    const float p4 = exp2_fast(s[kt][i0 + 4]), p5 = exp2_fast(s[kt][i0 + 5]);
+    const float p6 = exp2_fast(s[kt][i0 + 6]), p7 = exp2_fast(s[kt][i0 + 7]);
+    pk[u * 4 + 0] = pack_bf16(p0, p1); pk[u * 4 + 1] = pack_bf16(p2, p3);
+    pk[u * 4 + 2] = pack_bf16(p4, p5); pk[u * 4 + 3] = pack_bf16(p6, p7);
+    sum0 += (p0 + p2) + (p4 + p6);
+    sum1 += (p1 + p3) + (p5 + p7);
+}
+
+// q * c, rounded to bf16 again (round to nearest even).
+__device__ __forceinline__ bf16x8 scale_bf16x8(bf16x8 q, float c) {
+    const u32x4 bits = __builtin_bit_cast(u32x4, q);
+    u32x4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        out[i] = pack_bf16(bf16_bits_to_f32(bits[i] & 0xffffu) * c, __builtin_bit_cast(float, bits[i] & 0xffff0000u) * c);
+    return __builtin_bit_cast(bf16x8, out);
+}
+
 // K and V tiles of a key block are fetched with LDS-direct loads into swizzled row-major buffers (see
 // Bf16DirectTiles; no staging registers, no LDS writes by the waves), V^T fragments come from transposing
 // LDS reads.  Software pipeline over the key blocks of the item; in iteration j a wave
@@ -460,10 +487,16 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     load_v(0, 0);
     load_k(1, 1);
     if (SLIM && t == 0) *retry_flag = 0;
-
     const float c = p.scale_log2e, slack = p.slack;
+
     bf16x8 qf[KS];
     T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
+    if constexpr (SLIM) {
+        // the score product then delivers base-2 exponents; the second rounding of Q moves them by less than the
+        // rounding of the probabilities does
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = scale_bf16x8(qf[ks], c);
+    }
     const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
 
     f32x16 o_acc[NO];
@@ -483,7 +516,16 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         for (int ks = 0; ks < KS; ++ks)
             s_even[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(smem, k_lane, kt, ks), qf[ks], s_even[kt], 0, 0, 0);
     }
-    if constexpr (SLIM) st.m_used = st.m_true = block_row_max<KT>(s_even);
+    // SLIM: -offset in every element, the accumulator input of each later block's first product step
+    f32x16 off_vec;
+    if constexpr (SLIM) {
+        const float m_scaled = block_row_max<KT>(s_even);
+        st.m_used = st.m_true = m_scaled / c;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) off_vec[i] = -m_scaled;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) s_even[kt] += off_vec;
+    }
     __syncthreads();   // every wave has read K(0) before iteration 0 overwrites its buffer
 
     auto iteration = [&](uint32_t j, f32x16 (&s)[KT], f32x16 (&s_next)[KT]) {
@@ -526,35 +568,77 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         const float mc = st.m_used * c;
         float sum0 = 0.f, sum1 = 0.f;
         uint32_t pk[KT * 8];
-        exp_chunk<KT, NO>(s, pk, 0, c, mc, sum0, sum1);
+        auto exps = [&](int u) {
+            if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, sum0, sum1);
+            else exp_chunk<KT, NO>(s, pk, u, c, mc, sum0, sum1);
+        };
+        // Every chunk carries the same work: the exponentials of the next chunk, one slice (KS / PU product steps) of
+        // the next block's scores and one step of the output product.  The fragments of a chunk are requested from
+        // LDS one chunk ahead of the matrix instructions that consume them.
+        constexpr int KPC = KS / PU;   // score product steps per chunk
+        static_assert(KS % PU == 0, "the score product is spread evenly over the chunks");
+        bf16x8 kfr[PU][KPC][KT], vfr[PU][NO];
+        auto fragments = [&](int u) {
+#pragma unroll
+            for (int kk = 0; kk < KPC; ++kk)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) kfr[u][kk][kt] = T::k_frag(k_read, k_lane, kt, u * KPC + kk);
+#pragma unroll
+            for (int mt = 0; mt < NO; ++mt) vfr[u][mt] = T::v_frag(v_read, v_lane, mt, u);
+        };
+        fragments(0);
+        exps(0);
+#pragma unroll
+        for (int i = 0; i < T::LOADS; ++i) {
+            T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
+            T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
+        }
+        if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the tile loads are issued here, not later
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
-            if (u + 1 < PU) exp_chunk<KT, NO>(s, pk, u + 1, c, mc, sum0, sum1);
-#pragma unroll
-            for (int i = 0; i < (u == 0 ? T::LOADS : 0); ++i) {
-                T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
-                T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
+            if (u + 1 < PU) {
+                fragments(u + 1);
+                exps(u + 1);
             }
-            // the next block's scores are finished in the first half of the chunks: the maximum at the
-            // top of the next iteration then finds them complete instead of waiting for the MFMA pipe
 #pragma unroll
-            for (int ks = u * (KS / SC); ks < (u + 1) * (KS / SC) && ks < KS; ++ks)
+            for (int kk = 0; kk < KPC; ++kk)
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) {
+                    const int ks = u * KPC + kk;
                     if (ks == 0) {
                         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, k_lane, kt, ks), qf[ks], zero, 0, 0, 0);
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u][kk][kt], qf[ks], SLIM ? off_vec : zero, 0, 0, 0);
                     } else {
-                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k_read, k_lane, kt, ks), qf[ks], s_next[kt], 0, 0, 0);
+                        s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u][kk][kt], qf[ks], s_next[kt], 0, 0, 0);
                     }
                 }
             const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
             const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
             for (int mt = 0; mt < NO; ++mt)
-                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::v_frag(v_read, v_lane, mt, u), bfrag, o_acc[mt], 0, 0, 0);
+                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[u][mt], bfrag, o_acc[mt], 0, 0, 0);
+        }
+        if constexpr (SLIM) {
+            // the order the instructions are to be issued in: the LDS reads of chunk u + 1 before the matrix
+            // instructions of chunk u, and between two matrix instructions an equal share of the vector work
+            constexpr int MF = KPC * KT + NO;                    // matrix instructions per chunk
+            constexpr int DS = KPC * KT + 2 * NO;                // LDS reads per chunk
+            constexpr int VA = (BS / 2 + BS / 4 + BS / 2) / PU;  // exp + pack + add per chunk (BS/2 elements per lane)
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                if (u + 1 < PU) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
+#pragma unroll
+                for (int m = 0; m < MF; ++m) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (u + 1 < PU) {
+                        __builtin_amdgcn_sched_group_barrier(0x400, BS / 2 / PU / MF, 0);        // exponentials
+                        __builtin_amdgcn_sched_group_barrier(0x002, (BS / 4 + BS / 2) / PU / MF, 0);   // pack, add
+                    }
+                }
+            }
         }
         st.l += sum0 + sum1;
+        if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the wait for the tiles comes last
         loads_landed();
     };
 
