@@ -141,31 +141,68 @@ uint32_t sfb_suggest_max_blocks(const sfb_uint2* nn_lut, int nb, uint32_t batch_
 size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_parts, uint32_t batch_dim,
                                     uint32_t head_dim, uint32_t block_size, uint32_t state_dim);
 
-/* MI355X addition (no reference counterpart): plan of a launch whose work-groups stay resident.  Instead of one
- * work-group per work item, wg_slots work-groups (sfb_resident_work_groups(): as many as the device runs at once)
- * each walk a list of items chosen here so that all lists cost about the same (key blocks plus a fixed charge per
- * item): no dispatch gaps between items, and an item's descriptors are fetched while its predecessors are computed.
- * Long items come first in every list; the lists of one die (slot index mod 8) only hold (batch, head) pairs of
- * the same residue mod 8, so that a head's K and V stay in one L2. */
+/* MI355X addition (no reference counterpart): streams of a launch whose work-groups stay resident.  Instead of
+ * one work-group per work item, wg_slots work-groups (sfb_resident_work_groups(): as many as the device runs at once)
+ * each walk one stream of key blocks that strings its work items together, so that the tiles, the queries and the
+ * descriptors of an item are fetched while its predecessor is still being computed and no work-group is dispatched
+ * in the middle of the launch.  The streams are made to cost the same (key blocks plus charges per item, partial
+ * record and merge): block-rows are placed whole, longest first, on the least loaded stream; rows too long for that
+ * (BigBird's global rows) are cut and poured into the streams up to the common level.  The chunks of a cut row
+ * stand first in their streams and leave partial records (unnormalised output, maxima, sum) in a workspace, each
+ * followed by a flag; one stream ends with the row's merge task, which finds the flags set, adds the records and
+ * writes the row.  Streams of one die (slot index mod 8) only hold (batch, head) pairs of the same residue mod 8,
+ * so that a head's K and V stay in one L2.  All of it is one blob, built on the host and copied to the device. */
 typedef struct {
-    uint32_t batch, head;  /* which sequence and head */
-    uint32_t row;          /* the fields of sfb_work_item */
-    uint32_t first;
-    uint32_t count;        /* 0xffffffff: end of the list */
-    uint32_t nchunks;
-    uint32_t chunk;
-    uint32_t slot;
+    uint32_t kv_off;   /* ((batch * ctx + key column * block_size) * heads + head): first key row of the block, in rows of head_state elements */
+    uint32_t info;     /* SFB_STREAM_BLOCK_INDEX: index of the block in the layout (mask words); SFB_STREAM_FIRST / _LAST: first / last block of its item */
+    uint32_t col;      /* key block column */
+    uint32_t q_off;    /* first block of an item: the item's q_off (its queries are requested two blocks ahead); else 0 */
+} sfb_stream_block;
+#define SFB_STREAM_BLOCK_INDEX 0x0fffffffu
+#define SFB_STREAM_FIRST 0x40000000u
+#define SFB_STREAM_LAST 0x80000000u
+typedef struct {
+    uint32_t q_off;      /* ((batch * ctx + row * block_size) * heads + head): first query row, same unit as kv_off */
+    uint32_t batch, head, row;
+    uint32_t kind;       /* 0: the whole block-row, written to O; 1: chunk of a cut row, leaves partial record `part` */
     uint32_t part;
-    uint32_t lut_first;
-    uint32_t reserved[2];  /* entries are 48 bytes */
-} sfb_plan_entry;
+    uint32_t lse_off;    /* (batch * heads + head) * ctx + row * block_size: the row's first query in the lse output */
+    uint32_t lut_first;  /* index of the item's first entry in the head's NN LUT */
+    uint32_t count;      /* key blocks */
+    uint32_t first;      /* first key block, relative to the row's LUT segment */
+    uint32_t nchunks, chunk;
+    uint32_t reserved[4];   /* items are 64 bytes */
+} sfb_stream_item;
+typedef struct {
+    uint32_t q_off, batch, head, row;
+    uint32_t part;       /* first partial record of the row */
+    uint32_t nparts;     /* number of records to add; 0: the row has no key blocks and is written as zeros */
+    uint32_t reserved[2];
+} sfb_stream_merge;
+typedef struct {
+    uint32_t block_begin, n_blocks;   /* this work-group's run of sfb_stream_block entries */
+    uint32_t item_begin, n_items;     /* ... of sfb_stream_item entries, in the order their blocks appear */
+    uint32_t merge_begin, n_merges;   /* ... of sfb_stream_merge entries, done after the stream */
+    uint32_t reserved[2];
+} sfb_stream_slot;
+typedef struct {
+    uint32_t wg_slots, n_blocks, n_items, n_merges;
+    uint32_t n_parts;                 /* partial records (and flags) the launch uses */
+    uint32_t block_size, batch_dim, head_dim, ctx_blks;   /* what the streams were built for */
+    float balance;                    /* mean stream cost / largest stream cost, over the resident streams */
+    uint32_t resident;                /* the first `resident` streams are the long ones (one per resident work-group) */
+    uint64_t slots_offset, blocks_offset, items_offset, merges_offset;   /* byte offsets of the four arrays in the blob */
+    uint64_t total_bytes;             /* size of the blob */
+} sfb_stream_plan;
 /*   nn_lut [host] lut_heads tables of lut_dim entries (lut_heads = 1: one layout for all heads; = head_dim:
- *   per-head layouts as fixed_fusion_test.cu:38-39 builds them, every head with the same number of blocks).
- *   plan [host] receives wg_slots lists of *plan_stride entries each (the last entries of a list are end marks);
- *   NULL: only the sizes are returned.  *n_slots / *n_parts size the workspace (sfb_schedule_workspace_bytes). */
-int sfb_build_plan(sfb_plan_entry* plan, uint32_t* plan_stride, uint32_t* n_slots, uint32_t* n_parts,
-                   const sfb_uint2* nn_lut, int nb, uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim,
-                   uint32_t head_dim, uint32_t wg_slots, uint32_t max_blocks);
+ *   per-head layouts as fixed_fusion_test.cu:38-39 builds them).  blob [host] NULL: only *plan (sizes) is filled;
+ *   otherwise blob_bytes >= plan->total_bytes as returned by such a call. */
+int sfb_build_stream(sfb_stream_plan* plan, void* blob, size_t blob_bytes, const sfb_uint2* nn_lut, int nb,
+                     uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim, uint32_t head_dim, uint32_t block_size,
+                     uint32_t wg_slots, int level, uint32_t tail_percent);
+/* Bytes of the [dev] workspace a streamed launch needs: one flag per partial record, the records, a status word.
+ * The workspace must be zero-filled once before its first use; launches leave the flags at zero. */
+size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim);
 /* Work-groups of the fused kernels the current device keeps resident (4 per compute unit); 0 without a device. */
 uint32_t sfb_resident_work_groups(void);
 
@@ -246,16 +283,23 @@ int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const 
                                       uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
                                       uint32_t mask_heads, float scale);
 
-/* The same operation launched over sfb_build_plan's lists: wg_slots resident work-groups, each walking its list.
- * Takes per-head look-up tables (lut_heads = head_dim) as well as a shared one.  plan [dev] wg_slots * plan_stride
- * entries; lse may be NULL; out_dtype SFB_F32 or SFB_BF16; workspace as for sfb_fused_attention_scheduled. */
-int sfb_fused_attention_planned(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
-                                int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
-                                const int32_t* valid_len, const sfb_plan_entry* plan, uint32_t wg_slots,
-                                uint32_t plan_stride, uint32_t n_slots, uint32_t n_parts, void* workspace,
-                                size_t workspace_bytes, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
-                                uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
-                                uint32_t lut_dim, uint32_t mask_heads, float scale);
+/* The same operation launched over sfb_build_stream's streams: plan->wg_slots resident work-groups, each walking
+ * its stream (bf16 tensors with head size 64: tiles, queries and descriptors of the next item in flight while an
+ * item is computed; other cases: item after item).  Takes per-head look-up tables and masks (lut_heads, mask_heads
+ * = head_dim) as well as shared ones.  plan [host] as sfb_build_stream filled it, blob [dev] a copy of the blob;
+ * lse may be NULL; out_dtype SFB_F32 or SFB_BF16; workspace [dev] sfb_stream_workspace_bytes() bytes, 256-byte
+ * aligned.  A merge task waits for the flags of its records with a bounded number of polls (their producers stand
+ * first in their streams, so they are set long before); if the launch has more work-groups than the device keeps
+ * resident and a wait runs out, the row is left unwritten and the workspace's status word is set to 1: sfb_stream_status() reads it after the stream has been synchronised. */
+int sfb_fused_attention_streamed(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o, float* lse,
+                                 int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                 const int32_t* valid_len, const sfb_stream_plan* plan, const void* blob,
+                                 void* workspace, size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                 uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                 uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale);
+/* Status word of a streamed launch's workspace (synchronous copy from the device): 0 = every merge found its
+ * records, 1 = a wait ran out, negative = the copy failed. */
+int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const void* workspace);
 
 /* MI355X addition: the whole backward of the attention in one pass over the blocks, with P, dP and dS kept on chip.  Same
  * arithmetic as the reference's sequence TN, NT, softmax gradient, TN, NN (transformer_attention_optimize.cu:
@@ -478,6 +522,18 @@ int sfb_encoder_layer_forward_pre_ln(sfb_stream_t stream, float* y, const float*
                                      uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                      uint32_t head_dim, uint32_t state_dim, uint32_t ffn, void* workspace,
                                      size_t workspace_bytes);
+
+/* Either layer (pre_ln = 0: sfb_encoder_layer_forward's wiring, 1: sfb_encoder_layer_forward_pre_ln's) with its
+ * attention launched over sfb_build_stream's streams: per-head look-up tables and masks (lut_heads, mask_heads =
+ * head_dim; the reference's `fixed` pattern, fixed_fusion_test.cu:38-39) as well as shared ones.  plan / blob /
+ * attn_workspace as for sfb_fused_attention_streamed; the other arguments as for sfb_encoder_layer_forward. */
+int sfb_encoder_layer_forward_streamed(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
+                                       int dtype, int pre_ln, const sfb_uint2* nn_lut, const void* mask,
+                                       const int32_t* valid_len, const sfb_stream_plan* plan, const void* blob,
+                                       void* attn_workspace, size_t attn_workspace_bytes, uint32_t block_size,
+                                       uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                       uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads,
+                                       uint32_t ffn, void* workspace, size_t workspace_bytes);
 
 /* cblas_sgemm(RowMajor, NoTrans, Trans, m, n, k, 1, A, k, W, k, 0, C, n) (transformer_inference_part.cpp:236, the
  * tied-embedding logits): C[m][n] = A[m][k] W[n][k]^T, a and w of dtype, c fp32.  Runs on rocBLAS. */

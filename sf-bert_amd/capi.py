@@ -52,6 +52,7 @@ lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
 lib.sfb_resident_work_groups.restype = C.c_uint32
+lib.sfb_stream_workspace_bytes.restype = C.c_size_t
 lib.sfb_static_scratch_bytes.restype = C.c_size_t
 lib.sfb_gemm_release.restype = None
 
@@ -63,7 +64,8 @@ EXPORTED = [
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
-    "sfb_build_plan", "sfb_resident_work_groups", "sfb_fused_attention_planned",
+    "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_resident_work_groups",
+    "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
@@ -71,6 +73,7 @@ EXPORTED = [
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_transpose_0213", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_gemm_release", "sfb_gemm", "sfb_gemm_bias", "sfb_gemm_bias_gelu", "sfb_gemm_bias_gelu_scaled", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
+    "sfb_encoder_layer_forward_streamed",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
     "sfb_model_forward",
 ]
@@ -219,32 +222,55 @@ def resident_work_groups():
     return int(lib.sfb_resident_work_groups())
 
 
-PLAN_ENTRY_DTYPE = np.dtype([(n, np.uint32) for n in
-                             ("batch", "head", "row", "first", "count", "nchunks", "chunk", "slot", "part",
-                              "lut_first", "reserved0", "reserved1")])
-PLAN_END = 0xffffffff
+class StreamPlan(C.Structure):
+    """sfb_stream_plan"""
+    _fields_ = [(n, C.c_uint32) for n in ("wg_slots", "n_blocks", "n_items", "n_merges", "n_parts", "block_size",
+                                          "batch_dim", "head_dim", "ctx_blks")] + [("balance", C.c_float), ("resident", C.c_uint32)] + \
+               [(n, C.c_uint64) for n in ("slots_offset", "blocks_offset", "items_offset", "merges_offset",
+                                          "total_bytes")]
 
 
-def build_plan(nn_lut, nb, batch, heads, max_blocks=None, lut_heads=1, wg_slots=None):
-    """Lists of work items for the resident work-groups of a planned launch (sfb_build_plan): dict(plan
-    [wg_slots, stride] of PLAN_ENTRY_DTYPE, n_slots, n_parts, wg_slots, plan_stride, ...).  nn_lut: one table, or
-    lut_heads tables of equal length concatenated.  max_blocks None: what sfb_suggest_max_blocks gives for the
-    first table; wg_slots None: what the device keeps resident (sfb_resident_work_groups)."""
+STREAM_SLOT_DTYPE = np.dtype([(n, np.uint32) for n in ("block_begin", "n_blocks", "item_begin", "n_items",
+                                                       "merge_begin", "n_merges", "reserved0", "reserved1")])
+STREAM_BLOCK_DTYPE = np.dtype([(n, np.uint32) for n in ("kv_off", "info", "col", "q_off")])
+STREAM_ITEM_DTYPE = np.dtype([(n, np.uint32) for n in ("q_off", "batch", "head", "row", "kind", "part", "lse_off",
+                                                       "lut_first", "count", "first", "nchunks", "chunk", "r0", "r1",
+                                                       "r2", "r3")])
+STREAM_MERGE_DTYPE = np.dtype([(n, np.uint32) for n in ("q_off", "batch", "head", "row", "part", "nparts", "r0", "r1")])
+STREAM_BLOCK_INDEX, STREAM_FIRST, STREAM_LAST = 0x0fffffff, 0x40000000, 0x80000000
+
+
+def build_stream(nn_lut, nb, batch, heads, block_size, lut_heads=1, wg_slots=None, level=True, tail_percent=0):
+    """Streams of key blocks for the resident work-groups of a streamed launch (sfb_build_stream): dict(plan
+    (StreamPlan), blob (uint8 array to copy to the device), slots / blocks / items / merges (views of the blob),
+    lut_heads, lut_dim).  nn_lut: one table, or lut_heads tables of equal length concatenated.  wg_slots None: what
+    the device keeps resident (sfb_resident_work_groups)."""
     nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
     lut_dim = nn_lut.shape[0] // lut_heads
     if wg_slots is None:
         wg_slots = resident_work_groups() or 1024
-    if max_blocks is None:
-        max_blocks = suggest_max_blocks(nn_lut[:lut_dim], nb, batch * heads)
-    stride, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    plan = StreamPlan()
     args = (_np(nn_lut), nb, C.c_uint32(lut_heads), C.c_uint32(lut_dim), C.c_uint32(batch), C.c_uint32(heads),
-            C.c_uint32(wg_slots), C.c_uint32(max_blocks))
-    _check(lib.sfb_build_plan(None, C.byref(stride), C.byref(n_slots), C.byref(n_parts), *args), "sfb_build_plan")
-    plan = np.zeros((wg_slots, stride.value), PLAN_ENTRY_DTYPE)
-    _check(lib.sfb_build_plan(_np(plan), C.byref(stride), C.byref(n_slots), C.byref(n_parts), *args), "sfb_build_plan")
-    return Luts(plan=plan, n_slots=int(n_slots.value), n_parts=int(n_parts.value), wg_slots=int(wg_slots),
-                plan_stride=int(stride.value), max_blocks=int(max_blocks), lut_heads=int(lut_heads),
-                lut_dim=int(lut_dim))
+            C.c_uint32(block_size), C.c_uint32(wg_slots), C.c_int(1 if level else 0), C.c_uint32(tail_percent))
+    _check(lib.sfb_build_stream(C.byref(plan), None, C.c_size_t(0), *args), "sfb_build_stream")
+    blob = np.zeros(plan.total_bytes, np.uint8)
+    _check(lib.sfb_build_stream(C.byref(plan), _np(blob), C.c_size_t(blob.nbytes), *args), "sfb_build_stream")
+
+    def view(offset, count, dtype):
+        return blob[offset:offset + count * dtype.itemsize].view(dtype)
+    return Luts(plan=plan, blob=blob, lut_heads=int(lut_heads), lut_dim=int(lut_dim),
+                slots=view(plan.slots_offset, plan.wg_slots, STREAM_SLOT_DTYPE),
+                blocks=view(plan.blocks_offset, plan.n_blocks, STREAM_BLOCK_DTYPE),
+                items=view(plan.items_offset, plan.n_items, STREAM_ITEM_DTYPE),
+                merges=view(plan.merges_offset, plan.n_merges, STREAM_MERGE_DTYPE))
+
+
+def stream_workspace_bytes(stream, d):
+    return int(lib.sfb_stream_workspace_bytes(C.byref(stream["plan"]), C.c_uint32(d)))
+
+
+def stream_status(stream, d, workspace):
+    return int(lib.sfb_stream_status(C.byref(stream["plan"]), C.c_uint32(d), _dev(workspace)))
 
 
 def schedule_workspace_bytes(sched, batch, heads, block_size, d):
@@ -386,22 +412,20 @@ def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_si
 
 
 # ------------------------------------------------------------------------------------ unfused trio
-def fused_attention_planned(q, k, v, nn_lut, plan_dev, plan, workspace, block_size, blocks, scale, mask=None,
-                            valid_len=None, mask_heads=1, out=None, lse=None):
-    """sfb_fused_attention_planned: resident work-groups walking build_plan()'s lists.  plan_dev: device copy of
-    plan["plan"]; workspace: zero-filled uint8 tensor of schedule_workspace_bytes(plan, ...) bytes (or None
-    without split rows)."""
+def fused_attention_streamed(q, k, v, nn_lut, blob_dev, stream, workspace, block_size, blocks, scale, mask=None,
+                             valid_len=None, mask_heads=1, out=None, lse=None):
+    """sfb_fused_attention_streamed: resident work-groups walking build_stream()'s streams.  blob_dev: device copy
+    of stream["blob"]; workspace: zero-filled uint8 tensor of stream_workspace_bytes(stream, d) bytes."""
     import torch
     B, L, H, d = q.shape
     if out is None:
         out = torch.empty((B, L, H, d), device=q.device, dtype=torch.float32)
-    _check(lib.sfb_fused_attention_planned(
+    _check(lib.sfb_fused_attention_streamed(
         _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dev(lse), _dtype_code(q), _dtype_code(out), _dev(nn_lut),
-        _dev(mask), _dev(valid_len), _dev(plan_dev), C.c_uint32(plan["wg_slots"]), C.c_uint32(plan["plan_stride"]),
-        C.c_uint32(plan["n_slots"]), C.c_uint32(plan["n_parts"]), _dev(workspace),
-        C.c_size_t(workspace.numel() if workspace is not None else 0), C.c_uint32(block_size), C.c_uint32(blocks),
-        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(plan["lut_heads"]),
-        C.c_uint32(plan["lut_dim"]), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_planned")
+        _dev(mask), _dev(valid_len), C.byref(stream["plan"]), _dev(blob_dev), _dev(workspace),
+        C.c_size_t(workspace.numel()), C.c_uint32(block_size), C.c_uint32(blocks),
+        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(stream["lut_heads"]),
+        C.c_uint32(stream["lut_dim"]), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_streamed")
     return out
 
 
@@ -735,11 +759,16 @@ class EncoderLayer:
     weights: dict of fp32 CUDA tensors (wq..w2 [in, out], bq..b2, ln1_g, ln1_b, ln2_g, ln2_b);
     dtype BF16 casts the six matrices to bf16 once."""
 
-    def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16, pre_ln=False):
+    def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16, pre_ln=False,
+                 streamed=False, lut_heads=1, mask_heads=1):
+        """streamed: the attention runs over build_stream()'s streams (sfb_encoder_layer_forward_streamed); then
+        luts["nn_lut"] may hold lut_heads tables (one per head) and the mask passed to forward() mask_heads masks."""
         import torch
         self.dtype, self.bs, self.heads, self.d, self.ffn = dtype, block_size, heads, head_state, ffn
         self.luts = luts
         self.pre_ln = pre_ln   # True: the reference's own wiring (sfb_encoder_layer_forward_pre_ln)
+        self.streamed, self.lut_heads, self.mask_heads = streamed, lut_heads, mask_heads
+        self._streams = {}
         self.tensors = {}
         for name, t in weights.items():
             t = t.contiguous()
@@ -748,7 +777,7 @@ class EncoderLayer:
             self.tensors[name] = t
         self.c_weights = LayerWeights(**{n: t.data_ptr() for n, t in self.tensors.items()})
         self.nn_lut = to_device(luts["nn_lut"])
-        self.sched = build_schedule(luts["nn_lut"], luts["nb"], max_blocks) if max_blocks else None
+        self.sched = build_schedule(luts["nn_lut"], luts["nb"], max_blocks) if max_blocks and not streamed else None
         self.items = to_device(self.sched["items"]) if self.sched else None
         self._ws = {}
 
@@ -771,6 +800,22 @@ class EncoderLayer:
         if out is None:
             out = torch.empty_like(x)
         ws, aws = self._workspaces(B, L, x.device)
+        if self.streamed:
+            import torch
+            if B not in self._streams:
+                st = build_stream(self.luts["nn_lut"], L // self.bs, B, self.heads, self.bs, lut_heads=self.lut_heads,
+                                  level=False)
+                self._streams[B] = (st, to_device(st["blob"]),
+                                    torch.zeros(stream_workspace_bytes(st, self.d), dtype=torch.uint8, device=x.device))
+            st, blob, sws = self._streams[B]
+            _check(lib.sfb_encoder_layer_forward_streamed(
+                _stream(), _dev(out), _dev(x), C.byref(self.c_weights), self.dtype, C.c_int(1 if self.pre_ln else 0),
+                _dev(self.nn_lut), _dev(mask), _dev(valid_len), C.byref(st["plan"]), _dev(blob), _dev(sws),
+                C.c_size_t(sws.numel()), C.c_uint32(self.bs), C.c_uint32(self.luts["blocks"]), C.c_uint32(B),
+                C.c_uint32(L // self.bs), C.c_uint32(self.heads), C.c_uint32(self.d), C.c_uint32(st["lut_heads"]),
+                C.c_uint32(st["lut_dim"]), C.c_uint32(self.mask_heads), C.c_uint32(self.ffn), _dev(ws),
+                C.c_size_t(ws.numel())), "sfb_encoder_layer_forward_streamed")
+            return out
         s = self.sched
         entry = lib.sfb_encoder_layer_forward_pre_ln if self.pre_ln else lib.sfb_encoder_layer_forward
         _check(entry(

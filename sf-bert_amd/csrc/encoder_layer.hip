@@ -355,6 +355,10 @@ struct LayerArgs {
     uint32_t block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn;
     void* workspace;
     size_t workspace_bytes;
+    // streamed attention launch instead of a scheduled one (takes per-head look-up tables and masks)
+    const sfb_stream_plan* st_plan = nullptr;
+    const void* st_blob = nullptr;
+    uint32_t lut_heads = 1, lut_dim = 0, mask_heads = 1;
 };
 
 // out = a W + bias in the compute dtype: one GEMM with the bias in its epilogue, or, where that is not available,
@@ -374,6 +378,15 @@ static int attention_call(sfb_stream_t stream, const LayerArgs& g, const void* q
 static int attention_operand(sfb_stream_t stream, const LayerArgs& g, const void* q, const void* k, const void* v,
                              float* attn, void* lp, size_t elements, const void** ain) {
     const float scale = 1.0f / sqrtf((float)g.state_dim);
+    if (g.st_plan) {
+        // bf16 activations: bf16 straight into lp; fp32: into attn
+        void* const out = g.dtype == SFB_BF16 ? lp : (void*)attn;
+        *ain = out;
+        return sfb_fused_attention_streamed(stream, q, k, v, out, nullptr, g.dtype, g.dtype, g.nn_lut, g.mask, g.valid_len,
+                                            g.st_plan, g.st_blob, g.attn_workspace, g.attn_workspace_bytes, g.block_size,
+                                            g.blocks, g.batch_dim, g.ctx_blks, g.head_dim, g.state_dim, g.lut_heads,
+                                            g.lut_dim, g.mask_heads, scale);
+    }
     if (g.dtype == SFB_BF16 && g.items) {
         *ain = lp;
         return sfb_fused_attention_scheduled_to(stream, q, k, v, lp, g.dtype, SFB_BF16, g.nn_lut, g.mask, g.valid_len,
@@ -486,14 +499,15 @@ extern "C" int sfb_encoder_layer_forward_pre_ln(sfb_stream_t stream, float* y, c
     return rc != SFB_OK ? rc : layer_forward_pre_ln(stream, y, x, wt, g);
 }
 
-extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x,
-                                         const sfb_layer_weights* wt, int dtype, const sfb_uint2* nn_lut,
-                                         const void* mask, const int32_t* valid_len,
-                                         const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
-                                         uint32_t n_slots, uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
-                                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
-                                         uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t ffn,
-                                         void* workspace, size_t workspace_bytes) {
+// Post-LN layer: x1 = LN1(x + Attn(xWq+bq, xWk+bk, xWv+bv) Wo + bo), y = LN2(x1 + gelu(x1 W1 + b1) W2 + b2)
+static int layer_forward_post_ln(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
+                                 const LayerArgs& la) {
+    const int dtype = la.dtype;
+    const sfb_uint2* const nn_lut = la.nn_lut;
+    void* const workspace = la.workspace;
+    const size_t workspace_bytes = la.workspace_bytes;
+    const uint32_t block_size = la.block_size, batch_dim = la.batch_dim, ctx_blks = la.ctx_blks, head_dim = la.head_dim,
+                   state_dim = la.state_dim, ffn = la.ffn;
     if (!y || !x || !wt || !nn_lut || !workspace) return SFB_ERR_NULL_POINTER;
     if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
     const uint32_t ctx = ctx_blks * block_size;
@@ -527,11 +541,8 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
 
     // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
-    const LayerArgs args = {dtype, nn_lut, mask, valid_len, items, n_items, n_heavy, n_slots, n_parts, attn_workspace,
-                         attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
-                         workspace, workspace_bytes};
     const void* ain = nullptr;
-    SFB_TRY(attention_operand(stream, args, q, k, v, attn, xa, m * n, &ain));
+    SFB_TRY(attention_operand(stream, la, q, k, v, attn, xa, m * n, &ain));
 
     // output projection + bias, residual, LayerNorm 1
     SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n, gws));
@@ -575,6 +586,45 @@ extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const fl
     }
 #undef SFB_TRY
     return SFB_OK;
+}
+
+extern "C" int sfb_encoder_layer_forward(sfb_stream_t stream, float* y, const float* x,
+                                         const sfb_layer_weights* wt, int dtype, const sfb_uint2* nn_lut,
+                                         const void* mask, const int32_t* valid_len,
+                                         const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                                         uint32_t n_slots, uint32_t n_parts, void* attn_workspace, size_t attn_workspace_bytes,
+                                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                         uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t ffn,
+                                         void* workspace, size_t workspace_bytes) {
+    const LayerArgs g = {dtype, nn_lut, mask, valid_len, items, n_items, n_heavy, n_slots, n_parts, attn_workspace,
+                         attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
+                         workspace, workspace_bytes};
+    return layer_forward_post_ln(stream, y, x, wt, g);
+}
+
+extern "C" int sfb_encoder_layer_forward_streamed(sfb_stream_t stream, float* y, const float* x,
+                                                  const sfb_layer_weights* wt, int dtype, int pre_ln,
+                                                  const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                                                  const sfb_stream_plan* plan, const void* blob, void* attn_workspace,
+                                                  size_t attn_workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                                  uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                                  uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim,
+                                                  uint32_t mask_heads, uint32_t ffn, void* workspace,
+                                                  size_t workspace_bytes) {
+    if (!plan || !blob) return SFB_ERR_NULL_POINTER;
+    LayerArgs g = {dtype, nn_lut, mask, valid_len, nullptr, 0, 0, 0, 0, attn_workspace,
+                   attn_workspace_bytes, block_size, blocks, batch_dim, ctx_blks, head_dim, state_dim, ffn,
+                   workspace, workspace_bytes};
+    g.st_plan = plan;
+    g.st_blob = blob;
+    g.lut_heads = lut_heads;
+    g.lut_dim = lut_dim;
+    g.mask_heads = mask_heads;
+    if (pre_ln) {
+        const int rc = check_layer_args(y, x, wt, g);
+        return rc != SFB_OK ? rc : layer_forward_pre_ln(stream, y, x, wt, g);
+    }
+    return layer_forward_post_ln(stream, y, x, wt, g);
 }
 
 // ------------------------------------------------------------------------------------------------

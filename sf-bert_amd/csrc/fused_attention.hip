@@ -18,6 +18,7 @@
 #include "tiles.hip.h"
 
 #include <mutex>
+#include <type_traits>
 
 namespace sfb {
 
@@ -32,8 +33,12 @@ struct FusedParams {
     const int32_t* valid_len;       // per batch, or nullptr
     const uint32_t* row_order;      // rank -> block-row (unscheduled launches), or nullptr
     const sfb_work_item* items;     // rank -> work item (scheduled launches), or nullptr
-    const sfb_plan_entry* plan;     // planned launches: one list of work items per resident work-group
-    uint32_t plan_stride;           // entries between the lists of consecutive work-groups
+    const void* st_slots;           // streamed launches: sfb_stream_slot per resident work-group,
+    const void* st_blocks;          //   sfb_stream_block, sfb_stream_item and sfb_stream_merge arrays
+    const void* st_items;
+    const void* st_merges;
+    uint32_t* st_flags;             // one flag per partial record of a streamed launch
+    uint32_t* st_status;            // set to 1 when a merge task's wait ran out
     uint32_t* counters;             // [batch*heads][n_slots] arrival counters of split rows
     float* partials;                // [batch*heads][n_parts][BS*D + 4*BS]
     uint32_t n_slots, n_parts;
@@ -79,37 +84,6 @@ __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
         w.nchunks = 1; w.slot = 0; w.part = 0; w.chunk = 0;
     }
     return w;
-}
-
-// Work of one entry of a planned launch.
-__device__ __forceinline__ RowWork plan_row_work(const FusedParams& p, const sfb_plan_entry& e) {
-    RowWork w;
-    w.valid = 1;
-    w.b = e.batch;
-    w.h = e.head;
-    w.bh = e.batch * p.heads + e.head;
-    w.row = e.row; w.first = e.first; w.count = e.count;
-    w.nchunks = e.nchunks; w.slot = e.slot; w.part = e.part; w.chunk = e.chunk;
-    w.lut_first = e.lut_first;
-    return w;
-}
-constexpr uint32_t kPlanEnd = 0xffffffffu;
-// Plan entries are read through the constant address space: nothing writes them during a launch, and the
-// loads then go through the scalar unit, so an entry waits in scalar registers while an item is computed.
-typedef const uint32_t __attribute__((address_space(4)))* plan_words;
-struct PlanList {
-    plan_words words;
-    __device__ __forceinline__ sfb_plan_entry operator[](uint32_t i) const {
-        const plan_words w = words + (size_t)i * (sizeof(sfb_plan_entry) / 4);
-        sfb_plan_entry e;
-        e.batch = w[0]; e.head = w[1]; e.row = w[2]; e.first = w[3]; e.count = w[4]; e.nchunks = w[5];
-        e.chunk = w[6]; e.slot = w[7]; e.part = w[8]; e.lut_first = w[9];
-        e.reserved[0] = 0; e.reserved[1] = 0;
-        return e;
-    }
-};
-__device__ __forceinline__ PlanList plan_list_of(const FusedParams& p) {
-    return PlanList{(plan_words)(uintptr_t)(p.plan + (size_t)blockIdx.x * p.plan_stride)};
 }
 
 // LUT entries of key blocks [first, first + 64) of an item, one per lane (clamped to the item's last one).
@@ -419,6 +393,31 @@ __device__ __forceinline__ bf16x8 scale_bf16x8(bf16x8 q, float c) {
     return __builtin_bit_cast(bf16x8, out);
 }
 
+// The order in which the instructions of the chunks of one key block are to be issued (slim loop): the LDS reads of
+// chunk u + 1 ahead of the matrix instructions of chunk u, and behind every matrix instruction an equal share of the
+// vector work -- first the packing and adding of exponentials that were issued a slot earlier (their results are
+// ready by then), then the next exponentials.
+template <int BS, int D>
+__device__ __forceinline__ void schedule_chunks() {
+    constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, KPC = KS / PU;
+    constexpr int MF = KPC * KT + NO;                    // matrix instructions per chunk
+    constexpr int DS = KPC * KT + 2 * NO;                // LDS reads per chunk
+    constexpr int EXP = BS / 2 / PU / MF;                // exponentials per slot (BS/2 elements per lane and key block)
+    constexpr int REST = (BS / 4 + BS / 2) / PU / MF;    // pack + add per slot
+#pragma unroll
+    for (int u = 0; u < PU; ++u) {
+        if (u + 1 < PU) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
+#pragma unroll
+        for (int m = 0; m < MF; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (u > 0 || m > 0) {
+                if (u + 1 < PU || m == 0) __builtin_amdgcn_sched_group_barrier(0x002, REST, 0);
+            }
+            if (u + 1 < PU) __builtin_amdgcn_sched_group_barrier(0x400, EXP, 0);
+        }
+    }
+}
+
 // K and V tiles of a key block are fetched with LDS-direct loads into swizzled row-major buffers (see
 // Bf16DirectTiles; no staging registers, no LDS writes by the waves), V^T fragments come from transposing
 // LDS reads.  Software pipeline over the key blocks of the item; in iteration j a wave
@@ -433,9 +432,12 @@ __device__ __forceinline__ bf16x8 scale_bf16x8(bf16x8 q, float c) {
 // which the end of the item detects, and the item is then redone by the general loop (returns false).  The 1e-6 of
 // the reference's denominator is applied relative to the offset instead of the true row maximum, a relative
 // difference of at most 1e-6.
-template <int BS, int D, bool MASKED, bool SLIM>
+//
+// finish(o_acc, st) ends the item: it gets the unnormalised output accumulators and the row state (maxima in raw-score
+// units, this lane's part of the sum).
+template <int BS, int D, bool MASKED, bool SLIM, typename Finish>
 __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const RowWork& w, uint8_t* smem, uint32_t* retry_flag,
-                                                 sfb_uint2 first_window) {
+                                                 sfb_uint2 first_window, Finish&& finish) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
     constexpr int TILE = T::TILE_BYTES;
@@ -619,23 +621,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
                 o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[u][mt], bfrag, o_acc[mt], 0, 0, 0);
         }
         if constexpr (SLIM) {
-            // the order the instructions are to be issued in: the LDS reads of chunk u + 1 before the matrix
-            // instructions of chunk u, and between two matrix instructions an equal share of the vector work
-            constexpr int MF = KPC * KT + NO;                    // matrix instructions per chunk
-            constexpr int DS = KPC * KT + 2 * NO;                // LDS reads per chunk
-            constexpr int VA = (BS / 2 + BS / 4 + BS / 2) / PU;  // exp + pack + add per chunk (BS/2 elements per lane)
-#pragma unroll
-            for (int u = 0; u < PU; ++u) {
-                if (u + 1 < PU) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
-#pragma unroll
-                for (int m = 0; m < MF; ++m) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    if (u + 1 < PU) {
-                        __builtin_amdgcn_sched_group_barrier(0x400, BS / 2 / PU / MF, 0);        // exponentials
-                        __builtin_amdgcn_sched_group_barrier(0x002, (BS / 4 + BS / 2) / PU / MF, 0);   // pack, add
-                    }
-                }
-            }
+            schedule_chunks<BS, D>();
         }
         st.l += sum0 + sum1;
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the wait for the tiles comes last
@@ -653,11 +639,11 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         __syncthreads();
         if (*retry_flag != 0) return false;
     }
-    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, smem);
+    finish(o_acc, st);
     return true;
 }
 
-template <int BS, int D, bool MASKED, bool PLANNED>
+template <int BS, int D, bool MASKED>
 __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int TILE = T::TILE_BYTES;
@@ -666,56 +652,32 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedPa
     static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
 
     const uint32_t lane = threadIdx.x & 63;
-    auto run = [&](const RowWork& w, sfb_uint2 window) {
-        if (w.count == 0) {
-            const uint32_t L = p.nb * BS, q_in_block = (threadIdx.x >> 6) * 32 + (lane & 31);
-            float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
-            store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
-            if (p.lse && (lane >> 5) == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
-            return;
-        }
-        if constexpr (!MASKED) {
-            if (attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window)) return;
-        }
-        attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window);
-    };
-    if constexpr (!PLANNED) {
-        const RowWork w = decode_row_work(p);
-        if (!w.valid) return;
-        run(w, lut_window(p, w, 0, lane));
+    const RowWork w = decode_row_work(p);
+    if (!w.valid) return;
+    const uint32_t L = p.nb * BS, q_in_block = (threadIdx.x >> 6) * 32 + (lane & 31);
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
+    if (w.count == 0) {
+        store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
+        if (p.lse && (lane >> 5) == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
         return;
     }
-    // Planned launch: this work-group stays resident and walks its own list of work items.  The list entry two
-    // items ahead and the first LUT window of the next item are requested before the current item starts and
-    // arrive while it is computed, so an item's first tile loads wait for nothing but themselves.  (Every list
-    // ends with two end marks.)
-    const PlanList mine = plan_list_of(p);
-    sfb_plan_entry e = mine[0];
-    if (e.count == kPlanEnd) return;
-    sfb_plan_entry e_next = mine[1];
-    RowWork w = plan_row_work(p, e);
-    sfb_uint2 window = lut_window(p, w, 0, lane);
-    for (uint32_t i = 2;; ++i) {
-        const bool more = e_next.count != kPlanEnd;
-        const RowWork w_next = plan_row_work(p, e_next);     // an end mark decodes to an item without key blocks
-        const sfb_uint2 window_next = more ? lut_window(p, w_next, 0, lane) : window;
-        e_next = mine[i];
-        run(w, window);
-        if (!more) break;
-        // the output rows left through the tiles' memory, which the next item's loads overwrite: every wave must
-        // have read its slab (LDS reads complete) before any wave goes on; the stores to memory may still be in flight
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        w = w_next;
-        window = window_next;
+    const sfb_uint2 window = lut_window(p, w, 0, lane);
+    auto finish = [&](f32x16 (&o_acc)[D / 32], const RowState& st) {
+        finish_row<BS, D>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, threadIdx.x, smem);
+    };
+    if constexpr (!MASKED) {
+        if (attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window, finish)) return;
     }
+    attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window, finish);
 }
 
 // ------------------------------------------------------------------------------------------------
 // fp32 inputs: v_mfma_f32_32x32x2_f32 (true fp32 products and accumulation)
 // ------------------------------------------------------------------------------------------------
 // One LDS buffer (K tile and V tile); the next block waits in registers.
-template <int BS, int D>
-__device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowWork& w, float* k_lds, float* v_lds) {
+template <int BS, int D, typename Finish>
+__device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowWork& w, float* k_lds, float* v_lds,
+                                                Finish&& finish) {
     using T = F32Tiles<BS, D>;
     constexpr int KT = BS / 32;
     constexpr int NO = D / 32;
@@ -808,51 +770,506 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
         __syncthreads();
     }
 
-    finish_row<BS, D>(p, w, o_row, o_acc, st, c, q_in_block, half, t, (uint8_t*)k_lds);
+    finish(o_acc, st);
 }
 
-template <int BS, int D, bool PLANNED>
+template <int BS, int D>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_kernel(FusedParams p) {
     using T = F32Tiles<BS, D>;
     __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
     __shared__ __attribute__((aligned(16))) float v_lds[T::V_FLOATS];
     static_assert(T::K_FLOATS * 4 >= BS * (D * 4 + 16), "the K tile's memory doubles as the output slabs");
-    if constexpr (!PLANNED) {
-        const RowWork w = decode_row_work(p);
-        if (w.valid) attend_item_f32<BS, D>(p, w, k_lds, v_lds);
-        return;
+    const RowWork w = decode_row_work(p);
+    if (!w.valid) return;
+    const uint32_t t = threadIdx.x, lane = t & 63, q_in_block = (t >> 6) * 32 + (lane & 31);
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, p.nb * BS, p.heads, D));
+    attend_item_f32<BS, D>(p, w, k_lds, v_lds, [&](f32x16 (&o_acc)[D / 32], const RowState& st) {
+        finish_row<BS, D>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, t, (uint8_t*)k_lds);
+    });
+}
+
+// ------------------------------------------------------------------------------------------------
+// Streamed launches: resident work-groups, each walking one stream of key blocks
+// ------------------------------------------------------------------------------------------------
+// The arrays of a stream are read through the constant address space: nothing writes them during a launch, and
+// the loads then go through the scalar unit, so entries wait in scalar registers while the blocks before them are
+// computed.
+typedef const uint32_t __attribute__((address_space(4)))* const_words;
+
+struct StreamBlock {
+    uint32_t kv_off, info, col;
+    uint32_t q_off;     // first block of an item: the item's first query row
+};
+// What the pipeline carries of an item: where its queries and its output are, and what becomes of the result.
+struct StreamItem {
+    uint32_t q_off;     // first query row
+    uint32_t tag;       // 0: whole row, written to O; otherwise index + 1 of the partial record the chunk leaves
+    uint32_t lse_off;   // index of the row's first query in the lse output
+    uint32_t batch, head;
+};
+// Entry i of a run of n block entries; past the end: the last entry without its flags (its tiles are loaded once
+// more and never used).
+// (Every value here is the same for all lanes; readfirstlane says so where the compiler cannot see it, which keeps
+// the entries and everything computed from them in scalar registers.)
+__device__ __forceinline__ uint32_t uni(uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ StreamBlock stream_block(const_words base, uint32_t i, uint32_t n) {
+    i = uni(i);
+    const const_words w = base + (size_t)(i < n ? i : n - 1) * (sizeof(sfb_stream_block) / 4);
+    StreamBlock e = {uni(w[0]), i < n ? uni(w[1]) : 0u, uni(w[2]), uni(w[3])};
+    return e;
+}
+template <bool MASKED = true>
+__device__ __forceinline__ StreamItem stream_item(const_words base, uint32_t i, uint32_t n) {
+    i = uni(i);
+    const const_words w = base + (size_t)(i < n ? i : n - 1) * (sizeof(sfb_stream_item) / 4);
+    // words: q_off, batch, head, row | kind, part, lse_off, lut_first | count, first, nchunks, chunk
+    return StreamItem{uni(w[0]), w[4] != 0 ? uni(w[5]) + 1u : 0u, uni(w[6]), MASKED ? uni(w[1]) : 0u, MASKED ? uni(w[2]) : 0u};
+}
+// Inside the pipeline the entries are fetched with vector loads (every lane the same 16 bytes) instead: a scalar load
+// in flight would turn every wait for an LDS fragment into a wait for all of them (the two share one counter that
+// then counts out of order), whereas these are simply waited for together with the tiles at the end of the iteration.
+__device__ __forceinline__ u32x4 entry_load(const_words base, uint32_t index, uint32_t n, uint32_t words_per_entry, uint32_t word) {
+    index = uni(index);
+    const uint64_t address = (uint64_t)(uintptr_t)(base + (size_t)(index < n ? index : n - 1) * words_per_entry + word);
+    u32x4 out;
+    const uint32_t zero = 0;
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(out) : "v"(zero), "s"(address) : "memory");
+    return out;
+}
+// To be called behind the wait for memory: makes what follows use the loaded values, not what the registers held before.
+__device__ __forceinline__ void entry_landed(u32x4& e) { asm volatile("" : "+v"(e)); }
+__device__ __forceinline__ StreamBlock uni(const StreamBlock& e) { return StreamBlock{uni(e.kv_off), uni(e.info), uni(e.col), uni(e.q_off)}; }
+__device__ __forceinline__ StreamItem uni(const StreamItem& it) {
+    return StreamItem{uni(it.q_off), uni(it.tag), uni(it.lse_off), uni(it.batch), uni(it.head)};
+}
+// The whole record, as the work of a launch that does item after item.
+__device__ __forceinline__ RowWork stream_row_work(const FusedParams& p, const_words base, uint32_t i) {
+    const const_words w = base + (size_t)uni(i) * (sizeof(sfb_stream_item) / 4);
+    RowWork r;
+    r.valid = 1;
+    r.b = w[1]; r.h = w[2]; r.bh = w[1] * p.heads + w[2];
+    r.row = w[3]; r.first = w[9]; r.count = w[8];
+    r.nchunks = w[10]; r.chunk = w[11]; r.slot = 0; r.part = w[5];
+    r.lut_first = w[7];
+    return r;
+}
+
+// End of a streamed item.  A whole row is normalised and stored straight from the accumulators; a chunk of a cut
+// row leaves its partial record and returns the record's index + 1: its flag is to be set once these stores have
+// completed (the caller does that after its next wait for memory).  Returns 0 otherwise.
+template <int BS, int D>
+__device__ __forceinline__ uint32_t stream_end_item(const FusedParams& p, const StreamItem& it, f32x16 (&o)[D / 32],
+                                                    float m_used, float m_true, float l, float c, uint32_t t) {
+    constexpr int NO = D / 32, PART = BS * D + 4 * BS;
+    const uint32_t lane = t & 63, qn = lane & 31, half = lane >> 5, q_in_block = (t >> 6) * 32 + qn;
+    const float total = l + __shfl_xor(l, 32);
+    if (it.tag == 0) {
+        float* o_row = output_row(p, ((size_t)it.q_off + (size_t)q_in_block * p.heads) * D);
+        const float f = exp2_fast((m_true - m_used) * c);
+        const float inv = 1.0f / (total + 1e-6f * f);
+        if (p.lse != nullptr && half == 0)
+            p.lse[(size_t)it.lse_off + q_in_block] = __builtin_fmaf(m_used, c, __builtin_log2f(total + 1e-6f * f));
+        for_each_out_vec<NO>([&](int mt, int ig) {
+            const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
+                               o[mt][ig * 4 + 3] * inv};
+            const uint32_t col = mt * 32 + ig * 8 + half * 4;
+            if (p.o_bf16) {
+                const u32x2 packed = {pack_bf16(out.x, out.y), pack_bf16(out.z, out.w)};
+                *(u32x2*)((uint8_t*)o_row + col * 2) = packed;
+            } else {
+                *(f32x4*)(o_row + col) = out;
+            }
+        });
+        return 0;
     }
-    // planned launch: a resident work-group walks its list of work items
-    const PlanList mine = plan_list_of(p);
-    sfb_plan_entry e = mine[0];
-    for (uint32_t i = 1; e.count != kPlanEnd; ++i) {
-        const sfb_plan_entry e_next = mine[i];
-        attend_item_f32<BS, D>(p, plan_row_work(p, e), k_lds, v_lds);
-        __syncthreads();   // the output rows left through the K tile's memory
-        e = e_next;
+    float* mine = p.partials + (size_t)(it.tag - 1) * PART;
+    for_each_out_vec<NO>([&](int mt, int ig) {
+        const f32x4 out = {o[mt][ig * 4 + 0], o[mt][ig * 4 + 1], o[mt][ig * 4 + 2], o[mt][ig * 4 + 3]};
+        coherent_store4(mine + partial_offset<BS>(mt, ig, half, q_in_block), out);
+    });
+    if (half == 0) {
+        const f32x4 sv = {m_used, m_true, total, 0.f};
+        coherent_store4(mine + BS * D + q_in_block * 4, sv);
     }
+    return it.tag;
+}
+
+__device__ __forceinline__ void stream_set_flag(const FusedParams& p, uint32_t part_plus_1) {
+    __hip_atomic_store(p.st_flags + (part_plus_1 - 1), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Merge tasks of a work-group, done after its stream: wait (bounded) for the flags of the row's partial records, add
+// the records, write the row, clear the flags for the next launch.  lds: at least BS * (D * 4 + 16) bytes that nobody
+// uses any more.
+template <int BS, int D>
+__device__ __forceinline__ void stream_merges(const FusedParams& p, const_words merges, uint32_t n_merges, uint8_t* lds) {
+    constexpr int PART = BS * D + 4 * BS;
+    constexpr uint32_t kMaxPolls = 1u << 20;   // of about a microsecond each
+    const uint32_t t = threadIdx.x, lane = t & 63, q_in_block = (t >> 6) * 32 + (lane & 31);
+    const uint32_t o_row_bytes = p.heads * D * (p.o_bf16 ? 2u : 4u);
+    uint8_t* const slab = lds + (t >> 6) * (32u * (D * 4 + 16));
+    for (uint32_t i = 0; i < n_merges; ++i) {
+        const const_words w = merges + (size_t)i * (sizeof(sfb_stream_merge) / 4);
+        const uint32_t q_off = w[0], batch = w[1], head = w[2], row = w[3], part = w[4], nparts = w[5];
+        float* o_row = output_row(p, ((size_t)q_off + (size_t)q_in_block * p.heads) * D);
+        float* lse_row = p.lse ? p.lse + ((size_t)(batch * p.heads + head) * p.nb + row) * BS + q_in_block : nullptr;
+        if (nparts == 0) {
+            store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
+            if (lse_row && (lane >> 5) == 0) *lse_row = 0.f;
+            continue;
+        }
+        int ready = 1;
+        for (uint32_t f = t; f < nparts; f += BS * 2) {
+            uint32_t polls = 0;
+            while (__hip_atomic_load(p.st_flags + part + f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u) {
+                if (++polls > kMaxPolls) { ready = 0; break; }
+                __builtin_amdgcn_s_sleep(32);
+            }
+        }
+        ready = __syncthreads_and(ready);
+        if (!ready) {
+            if (t == 0) __hip_atomic_store(p.st_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
+        }
+        merge_partials<BS, D>(p.partials + (size_t)part * PART, nparts, o_row, o_row_bytes, p.o_bf16, lse_row,
+                              p.scale_log2e, q_in_block, lane, slab);
+        for (uint32_t f = t; f < nparts; f += BS * 2)
+            __hip_atomic_store(p.st_flags + part + f, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();   // the slabs are used again by the next merge
+    }
+}
+
+// bf16 tensors: the items of a stream are chained.  The loop over an item's key blocks is the one of attend_item_bf16
+// (one barrier per block, K(j+2) and V(j+1) in flight while block j is worked on), but the blocks it fetches ahead are
+// taken from the stream, so that the last two iterations of an item fetch the first tiles of the next one instead of
+// nothing; the next item's queries and record are requested before the loop and arrive under it.  Between two items
+// stand only the end of one (normalisation and stores straight from the accumulators) and the first score block of
+// the other, whose tiles are already in LDS.  Block g of the stream uses tile buffers g % 2.
+template <int BS, int D, bool MASKED>
+__device__ __forceinline__ void stream_items_bf16(const FusedParams& p, uint8_t* smem, uint32_t* retry_flag,
+                                                  const_words blocks, uint32_t n, const_words items, uint32_t n_items) {
+    constexpr bool SLIM = !MASKED;
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16;
+    constexpr int TILE = T::TILE_BYTES;
+    constexpr int KPC = KS / PU;   // score product steps per chunk
+    static_assert(KS % PU == 0, "the score product is spread evenly over the chunks");
+
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t row_bytes = p.heads * D * 2;
+    const __bf16* const Q = (const __bf16*)p.q;
+    const uint8_t* const k_base = (const uint8_t*)p.k;
+    const uint8_t* const v_base = (const uint8_t*)p.v;
+    const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+    const uint32_t lds0 = T::lds_address(smem);
+    const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
+    const float c = p.scale_log2e, slack = p.slack;
+    const sfb_stream_block* const entries = (const sfb_stream_block*)(uintptr_t)blocks;
+    auto q_row_of = [&](uint32_t q_off) { return Q + ((size_t)q_off + (size_t)q_in_block * p.heads) * D; };
+    auto loads_landed = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+
+    // the stream's entries [win, win + 64), one per lane (clamped to the last one)
+    uint32_t win = 0, w_kv = 0, w_info = 0, w_col = 0;
+    auto refill = [&](uint32_t first) {
+        win = first;
+        const uint32_t idx = first + lane < n ? first + lane : n - 1;
+        w_kv = entries[idx].kv_off;
+        if constexpr (MASKED) {
+            w_info = entries[idx].info;
+            w_col = entries[idx].col;
+        }
+    };
+    auto kv_of = [&](uint32_t g) -> size_t {
+        const uint32_t gg = g < n ? g : n - 1;
+        return (size_t)(uint32_t)__builtin_amdgcn_readlane(w_kv, gg - win) * (D * 2);
+    };
+    auto load_k = [&](uint32_t g) {   // K(g) into buffer g % 2
+        T::load_tile(lds0 + (g & 1) * TILE, k_base + kv_of(g), wave, src_even, src_odd, row_bytes);
+    };
+    auto load_v = [&](uint32_t g) {
+        T::load_tile(lds0 + (2 + (g & 1)) * TILE, v_base + kv_of(g), wave, src_even, src_odd, row_bytes);
+    };
+
+    if (SLIM && t == 0) *retry_flag = 0;
+    uint32_t pending = 0;   // partial record (index + 1) whose flag waits for the record's stores to complete
+    uint32_t pos = 0;       // stream position of the current item's first block
+    uint32_t index = 0;     // the current item
+    bool primed = false;    // the tiles of blocks pos and pos + 1 are in LDS or on their way
+
+    bf16x8 qf[KS], qf_next[KS];
+    f32x16 o_acc[NO];
+#pragma unroll
+    for (int nn = 0; nn < NO; ++nn)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[nn][i] = 0.f;
+    refill(0);
+    StreamItem rec = stream_item<MASKED>(items, 0, n_items);
+    uint32_t count = uni(((const_words)items)[8]);
+    T::load_q(qf_next, q_row_of(rec.q_off), half);
+
+    for (;;) {
+        if (!primed) {
+            if (pos + 2 >= win + 64 || pos < win) refill(pos);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            load_k(pos);
+            load_v(pos);
+            load_k(pos + 1);
+            primed = true;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = SLIM ? scale_bf16x8(qf_next[ks], c) : qf_next[ks];
+        // the record and the queries of the next item
+        const bool more = index + 1 < n_items;
+        const StreamItem rec_next = stream_item<MASKED>(items, index + 1, n_items);
+        const uint32_t count_next = uni(((const_words)items)[(size_t)(more ? index + 1 : index) * (sizeof(sfb_stream_item) / 4) + 8]);
+        asm volatile("" : : "s"(rec_next.q_off), "s"(rec_next.tag), "s"(rec_next.lse_off), "s"(count_next));   // arrived: nothing scalar is in flight under the loop
+        const uint8_t* mask = nullptr;
+        int valid = (int)L;
+        if constexpr (MASKED) {
+            mask = p.mask ? (const uint8_t*)p.mask + (size_t)rec.head * p.mask_stride * (BS / 8) : nullptr;
+            valid = p.valid_len ? p.valid_len[rec.batch] : (int)L;
+        }
+        RowState st = {kMaxSeed, kMaxSeed, 0.f};
+
+        f32x16 s_even[KT], s_odd[KT];
+        loads_landed();
+        if (more) T::load_q(qf_next, q_row_of(rec_next.q_off), half);
+        {
+            const uint8_t* const k0 = smem + (pos & 1) * TILE;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s_even[kt][i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    s_even[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(T::k_frag(k0, k_lane, kt, ks), qf[ks], s_even[kt], 0, 0, 0);
+            }
+        }
+        f32x16 off_vec;
+        float m_item = 0.f;
+        if constexpr (SLIM) {
+            m_item = block_row_max<KT>(s_even);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) off_vec[i] = -m_item;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) s_even[kt] += off_vec;
+        }
+        __syncthreads();   // every wave has read K(pos) before the first iteration overwrites its buffer
+
+        auto iteration = [&](uint32_t j, f32x16 (&s)[KT], f32x16 (&s_next)[KT]) {
+            const uint32_t g = pos + j, par = g & 1;
+            const uint8_t* const k_read = smem + (par ^ 1) * TILE;       // K(g+1)
+            const uint8_t* const v_read = smem + (2 + par) * TILE;       // V(g)
+            if (g + 2 >= win + 64) refill(g);
+            const uint8_t* const k_src = k_base + kv_of(g + 2);
+            const uint8_t* const v_src = v_base + kv_of(g + 1);
+            const uint32_t k_dst = lds0 + par * TILE, v_dst = lds0 + (2 + (par ^ 1)) * TILE;
+
+            if constexpr (MASKED) {
+                const uint32_t blk = (uint32_t)__builtin_amdgcn_readlane(w_info, g - win) & SFB_STREAM_BLOCK_INDEX;
+                const uint32_t col = (uint32_t)__builtin_amdgcn_readlane(w_col, g - win);
+                const int limit = valid - (int)(col * BS);
+                if ((mask != nullptr) || (limit < BS)) {
+                    const uint64_t keep = load_keep_word<BS>(mask, (size_t)blk * BS + q_in_block, limit);
+                    constexpr uint64_t kAll = BS == 64 ? ~0ull : 0xffffffffull;
+                    if (__builtin_amdgcn_ballot_w64((keep & kAll) != kAll) != 0) apply_keep<KT>(s, keep, half);
+                }
+                const float mloc = block_row_max<KT>(s);
+                st.m_true = fmaxf(st.m_true, mloc);
+                if (__builtin_amdgcn_ballot_w64(mloc > st.m_used + slack) != 0) {
+                    const float m_new = fmaxf(st.m_used, mloc);
+                    const float alpha = exp2_fast((st.m_used - m_new) * c);
+                    st.m_used = m_new;
+                    st.l *= alpha;
+#pragma unroll
+                    for (int nn = 0; nn < NO; ++nn) o_acc[nn] *= alpha;
+                }
+            }
+            const float mc = st.m_used * c;
+            float sum0 = 0.f, sum1 = 0.f;
+            uint32_t pk[KT * 8];
+            auto exps = [&](int u) {
+                if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, sum0, sum1);
+                else exp_chunk<KT, NO>(s, pk, u, c, mc, sum0, sum1);
+            };
+            bf16x8 kfr[PU][KPC][KT], vfr[PU][NO];
+            auto fragments = [&](int u) {
+#pragma unroll
+                for (int kk = 0; kk < KPC; ++kk)
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) kfr[u][kk][kt] = T::k_frag(k_read, k_lane, kt, u * KPC + kk);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt) vfr[u][mt] = T::v_frag(v_read, v_lane, mt, u);
+            };
+            fragments(0);
+            exps(0);
+#pragma unroll
+            for (int i = 0; i < T::LOADS; ++i) {
+                T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
+                T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
+            }
+            if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the tile loads are issued here, not later
+#pragma unroll
+            for (int u = 0; u < PU; ++u) {
+                if (u + 1 < PU) {
+                    fragments(u + 1);
+                    exps(u + 1);
+                }
+#pragma unroll
+                for (int kk = 0; kk < KPC; ++kk)
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) {
+                        const int ks = u * KPC + kk;
+                        if (ks == 0) {
+                            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                            s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u][kk][kt], qf[ks], SLIM ? off_vec : zero, 0, 0, 0);
+                        } else {
+                            s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u][kk][kt], qf[ks], s_next[kt], 0, 0, 0);
+                        }
+                    }
+                const u32x4 pb = {pk[u * 4 + 0], pk[u * 4 + 1], pk[u * 4 + 2], pk[u * 4 + 3]};
+                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+#pragma unroll
+                for (int mt = 0; mt < NO; ++mt)
+                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[u][mt], bfrag, o_acc[mt], 0, 0, 0);
+            }
+            if constexpr (SLIM) {
+                schedule_chunks<BS, D>();
+            }
+            st.l += sum0 + sum1;
+            if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the wait for the tiles comes last
+            loads_landed();
+        };
+
+        for (uint32_t j = 0; j < count; j += 2) {
+            iteration(j, s_even, s_odd);
+            if (j + 1 < count) iteration(j + 1, s_odd, s_even);
+        }
+
+        // the record left by the item before this one is complete by now (every iteration waited for memory)
+        if (pending != 0) {
+            if (t == 0) stream_set_flag(p, pending);
+            pending = 0;
+        }
+        bool redo = false;
+        if constexpr (SLIM) {
+            const float total = st.l + __shfl_xor(st.l, 32);
+            if (__builtin_amdgcn_ballot_w64(!(total < 0x1p100f)) != 0 && lane == 0) *retry_flag = 1;   // overflow, or NaN
+            __syncthreads();
+            redo = __builtin_amdgcn_readfirstlane(*retry_flag) != 0;
+            st.m_used = st.m_true = m_item / c;
+        }
+        if (!redo) {
+            pending = uni(stream_end_item<BS, D>(p, rec, o_acc, st.m_used, st.m_true, st.l, c, t));
+        } else {
+            // The sum overflowed with the offset of the item's first block: the item is done again by the loop that
+            // follows the running maximum, and the tiles of the next item are fetched anew behind it.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (t == 0) *retry_flag = 0;
+            const RowWork w = stream_row_work(p, items, index);
+            uint32_t made = 0;
+            attend_item_bf16<BS, D, MASKED, false>(p, w, smem, retry_flag, lut_window(p, w, 0, lane),
+                                                   [&](f32x16 (&o)[NO], const RowState& rs) {
+                                                       made = stream_end_item<BS, D>(p, rec, o, rs.m_used, rs.m_true, rs.l, c, t);
+                                                   });
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (made != 0 && t == 0) stream_set_flag(p, made);
+            primed = false;
+        }
+#pragma unroll
+        for (int nn = 0; nn < NO; ++nn)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o_acc[nn][i] = 0.f;
+        if (!more) break;
+        pos = uni(pos + count);
+        index = uni(index + 1);
+        rec = uni(rec_next);
+        count = count_next;
+    }
+    if (pending != 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t == 0) stream_set_flag(p, pending);
+    }
+}
+
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 2) void fused_attention_stream_bf16_kernel(FusedParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int TILE = T::TILE_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+    __shared__ uint32_t retry_flag;
+    static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
+    const const_words slot = (const_words)(uintptr_t)p.st_slots + (size_t)blockIdx.x * (sizeof(sfb_stream_slot) / 4);
+    const uint32_t block_begin = slot[0], n_blocks = slot[1], item_begin = slot[2], n_items = slot[3];
+    const uint32_t merge_begin = slot[4], n_merges = slot[5];
+    if (n_blocks != 0)
+        stream_items_bf16<BS, D, MASKED>(p, smem, &retry_flag,
+                                         (const_words)(uintptr_t)p.st_blocks + (size_t)block_begin * (sizeof(sfb_stream_block) / 4), n_blocks,
+                                         (const_words)(uintptr_t)p.st_items + (size_t)item_begin * (sizeof(sfb_stream_item) / 4), n_items);
+    if (n_merges != 0) {
+        __syncthreads();   // the tiles' memory becomes the output slabs
+        stream_merges<BS, D>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4), n_merges, smem);
+    }
+}
+
+// Other element types and head sizes: the work-group does the items of its stream one after the other.
+template <int BS, int D>
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream_f32_kernel(FusedParams p) {
+    using T = F32Tiles<BS, D>;
+    __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
+    __shared__ __attribute__((aligned(16))) float v_lds[T::V_FLOATS];
+    static_assert(T::K_FLOATS * 4 >= BS * (D * 4 + 16), "the K tile's memory doubles as the output slabs");
+    const const_words slot = (const_words)(uintptr_t)p.st_slots + (size_t)blockIdx.x * (sizeof(sfb_stream_slot) / 4);
+    const uint32_t item_begin = slot[2], n_items = slot[3], merge_begin = slot[4], n_merges = slot[5];
+    const const_words items = (const_words)(uintptr_t)p.st_items + (size_t)item_begin * (sizeof(sfb_stream_item) / 4);
+    const uint32_t t = threadIdx.x;
+    for (uint32_t i = 0; i < n_items; ++i) {
+        const StreamItem it = stream_item(items, i, n_items);
+        uint32_t made = 0;
+        attend_item_f32<BS, D>(p, stream_row_work(p, items, i), k_lds, v_lds, [&](f32x16 (&o)[D / 32], const RowState& rs) {
+            made = stream_end_item<BS, D>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
+        });
+        if (made != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (made != 0 && t == 0) stream_set_flag(p, made);
+    }
+    if (n_merges != 0)
+        stream_merges<BS, D>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4), n_merges,
+                             (uint8_t*)k_lds);
 }
 
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
-    const uint32_t grid = p.plan ? ranks : p.groups * 8u * ranks;   // planned launches: ranks = resident work-groups
+    const bool streamed = p.st_slots != nullptr;
+    const uint32_t grid = streamed ? ranks : p.groups * 8u * ranks;   // streamed launches: ranks = resident work-groups
     clear_stale_error();
-    const bool masked = p.mask || p.valid_len, planned = p.plan != nullptr;
+    // the loop that folds scale and offset into the score product rounds the scaled queries to bf16 once more: fine
+    // for the output, but a log-sum-exp that a backward pass pairs with its own scores is made by the exact loop
+    const bool masked = p.mask || p.valid_len || p.lse;
     const dim3 g(grid), b(BS * 2);
     if (in_dtype == SFB_BF16) {
         if constexpr (D == 64) {
-            if (masked && planned) fused_attention_bf16_kernel<BS, D, true, true><<<g, b, 0, stream>>>(p);
-            else if (masked) fused_attention_bf16_kernel<BS, D, true, false><<<g, b, 0, stream>>>(p);
-            else if (planned) fused_attention_bf16_kernel<BS, D, false, true><<<g, b, 0, stream>>>(p);
-            else fused_attention_bf16_kernel<BS, D, false, false><<<g, b, 0, stream>>>(p);
+            if (masked && streamed) fused_attention_stream_bf16_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+            else if (masked) fused_attention_bf16_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+            else if (streamed) fused_attention_stream_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
+            else fused_attention_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
         } else {
             return SFB_ERR_HEAD_STATE;   // the bf16 kernel is built for head size 64 only
         }
-    } else if (planned)
-        fused_attention_f32_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+    } else if (streamed)
+        fused_attention_stream_f32_kernel<BS, D><<<g, b, 0, stream>>>(p);
     else
-        fused_attention_f32_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
+        fused_attention_f32_kernel<BS, D><<<g, b, 0, stream>>>(p);
     return launch_status();
 }
 
@@ -897,7 +1314,8 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.lse = nullptr;
     p.nn_lut = nn_lut; p.mask = mask; p.valid_len = valid_len;
     p.row_order = nullptr; p.items = nullptr; p.counters = nullptr; p.partials = nullptr;
-    p.plan = nullptr; p.plan_stride = 0;
+    p.st_slots = nullptr; p.st_blocks = nullptr; p.st_items = nullptr; p.st_merges = nullptr;
+    p.st_flags = nullptr; p.st_status = nullptr;
     p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
@@ -1016,39 +1434,57 @@ extern "C" int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
 }
 
-extern "C" int sfb_fused_attention_planned(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
-                                           float* lse, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
-                                           const void* mask, const int32_t* valid_len, const sfb_plan_entry* plan,
-                                           uint32_t wg_slots, uint32_t plan_stride, uint32_t n_slots,
-                                           uint32_t n_parts, void* workspace, size_t workspace_bytes,
-                                           uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
-                                           uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
-                                           uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale) {
+extern "C" size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim) {
+    if (!plan) return 0;
+    const size_t flags = ((size_t)plan->n_parts * sizeof(uint32_t) + 255) / 256 * 256;
+    const size_t part = ((size_t)plan->block_size * state_dim + 4 * (size_t)plan->block_size) * sizeof(float);
+    return flags + (size_t)plan->n_parts * part + 256;   // the last 256 bytes hold the status word (at their end)
+}
+
+extern "C" int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const void* workspace) {
+    if (!plan || !workspace) return -1;
+    uint32_t word = 0;
+    if (hipMemcpy(&word, (const uint8_t*)workspace + sfb_stream_workspace_bytes(plan, state_dim) - 4, 4, hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    return word != 0 ? 1 : 0;
+}
+
+extern "C" int sfb_fused_attention_streamed(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                            float* lse, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
+                                            const void* mask, const int32_t* valid_len, const sfb_stream_plan* plan,
+                                            const void* blob, void* workspace, size_t workspace_bytes,
+                                            uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                            uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                            uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale) {
     using namespace sfb;
     const int rc = check_common(q, k, v, o, in_dtype, nn_lut, block_size, blocks, batch_dim, ctx_blks, head_dim,
                                 state_dim, lut_heads, lut_dim, mask_heads, scale);
     if (rc != SFB_OK) return rc;
     if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
-    if (!plan) return SFB_ERR_NULL_POINTER;
-    if (wg_slots == 0 || plan_stride < 3) return SFB_ERR_SHAPE;
-    if ((uintptr_t)plan & 15u) return SFB_ERR_ALIGNMENT;
-    const size_t need = sfb_schedule_workspace_bytes(n_slots, n_parts, batch_dim, head_dim, block_size, state_dim);
-    if (n_parts > 0 && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)))
-        return SFB_ERR_WORKSPACE;
+    if (!plan || !blob) return SFB_ERR_NULL_POINTER;
+    if (plan->wg_slots == 0 || plan->block_size != block_size || plan->batch_dim != batch_dim ||
+        plan->head_dim != head_dim || plan->ctx_blks != ctx_blks)
+        return SFB_ERR_SHAPE;
+    if ((uintptr_t)blob & 15u) return SFB_ERR_ALIGNMENT;
+    const size_t need = sfb_stream_workspace_bytes(plan, state_dim);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u)) return SFB_ERR_WORKSPACE;
     FusedParams p;
     fill_common(p, q, k, v, o, out_dtype, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
                 lut_heads, lut_dim, mask_heads, scale);
-    p.plan = plan;
-    p.plan_stride = plan_stride;
     p.lse = lse;
-    p.n_slots = n_slots; p.n_parts = n_parts;
-    const size_t bh = (size_t)batch_dim * head_dim;
-    const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
-    p.counters = (uint32_t*)workspace;
-    p.partials = (float*)((uint8_t*)workspace + counters);
+    p.st_slots = (const uint8_t*)blob + plan->slots_offset;
+    p.st_blocks = (const uint8_t*)blob + plan->blocks_offset;
+    p.st_items = (const uint8_t*)blob + plan->items_offset;
+    p.st_merges = (const uint8_t*)blob + plan->merges_offset;
+    const size_t flags = ((size_t)plan->n_parts * sizeof(uint32_t) + 255) / 256 * 256;
+    p.st_flags = (uint32_t*)workspace;
+    p.partials = (float*)((uint8_t*)workspace + flags);
+    p.st_status = (uint32_t*)((uint8_t*)workspace + need - 4);
     hipStream_t s = (hipStream_t)stream;
-    if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, wg_slots, state_dim);
-    return launch_fused_any<32>(s, p, in_dtype, wg_slots, state_dim);
+    if (block_size == 64) return launch_fused_any<64>(s, p, in_dtype, plan->wg_slots, state_dim);
+    return launch_fused_any<32>(s, p, in_dtype, plan->wg_slots, state_dim);
 }
 
 // ------------------------------------------------------------------------------------------------

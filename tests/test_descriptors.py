@@ -167,47 +167,126 @@ def test_schedule_covers_every_block_once(max_blocks):
     assert nbytes == (4 * 12 * sched["n_slots"] * 4 + 255) // 256 * 256 + 4 * 12 * sched["n_parts"] * (64 * 64 + 256) * 4
 
 
-def test_plan_lists_cover_every_item_once():
-    nb, B, H = 64, 4, 12
-    luts = sfb.build_luts(sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234)))
-    plan = sfb.build_plan(luts["nn_lut"], nb, B, H, max_blocks=37, wg_slots=1024)
-    sched = sfb.build_schedule(luts["nn_lut"], nb, 37)
-    entries = plan["plan"]
-    assert entries.shape == (1024, plan["plan_stride"])
-    live = entries["count"] != sfb.PLAN_END
-    assert live.sum() == B * H * sched["n_items"]
-    assert (plan["n_slots"], plan["n_parts"]) == (sched["n_slots"], sched["n_parts"])
-    # every (batch, head) gets every work item of the schedule exactly once
-    fields = ("row", "first", "count", "nchunks", "chunk", "slot", "part", "lut_first")
-    want = sorted(tuple(int(it[f]) for f in fields) for it in sched["items"])
+def check_stream(stream, luts_per_head, nb, B, H, bs):
+    """Every key block of every (batch, head, row) appears exactly once, in LUT order inside its item; the flags,
+    the item records, the partial records and the merge tasks are consistent."""
+    plan, slots, blocks, items, merges = (stream[k] for k in ("plan", "slots", "blocks", "items", "merges"))
+    L = nb * bs
+    assert slots["n_blocks"].sum() == plan.n_blocks == len(blocks)
+    assert slots["n_items"].sum() == plan.n_items == len(items)
+    assert slots["n_merges"].sum() == plan.n_merges == len(merges)
+    seen = {}       # (b, h, row) -> list of (first, count, kind, part, chunk, nchunks)
+    for s in range(plan.wg_slots):
+        so = slots[s]
+        blk = blocks[so["block_begin"]:so["block_begin"] + so["n_blocks"]]
+        its = items[so["item_begin"]:so["item_begin"] + so["n_items"]]
+        # the FIRST flags of the run are the item boundaries, in the order of the item records
+        starts = np.flatnonzero(blk["info"] & sfb.STREAM_FIRST)
+        ends = np.flatnonzero(blk["info"] & sfb.STREAM_LAST)
+        assert len(starts) == len(ends) == len(its)
+        assert np.array_equal(ends - starts + 1, its["count"]) and (len(starts) == 0 or starts[0] == 0)
+        assert np.array_equal(starts[1:], ends[:-1] + 1)
+        kinds = its["kind"]
+        assert (np.diff(kinds.astype(int)) <= 0).all(), "chunks of cut rows lead the stream"
+        for it, a in zip(its, starts):
+            b, h, row = int(it["batch"]), int(it["head"]), int(it["row"])
+            lut = luts_per_head[h if len(luts_per_head) > 1 else 0]["nn_lut"]
+            assert it["q_off"] == (b * L + row * bs) * H + h and it["lse_off"] == (b * H + h) * L + row * bs
+            assert it["lut_first"] == lut[row, 0] + it["first"] and it["first"] + it["count"] <= lut[row, 1]
+            ent = lut[it["lut_first"]:it["lut_first"] + it["count"]]
+            mine = blk[a:a + it["count"]]
+            assert np.array_equal(mine["info"] & sfb.STREAM_BLOCK_INDEX, ent[:, 0])
+            assert np.array_equal(mine["col"], ent[:, 1])
+            assert mine["q_off"][0] == it["q_off"] and (mine["q_off"][1:] == 0).all()
+            assert np.array_equal(mine["kv_off"], (b * L + ent[:, 1] * bs) * H + h)
+            assert (it["kind"] == 1) == (it["nchunks"] > 1)
+            seen.setdefault((b, h, row), []).append(tuple(int(it[f]) for f in ("first", "count", "kind", "part", "chunk", "nchunks")))
+    merge_of = {(int(m["batch"]), int(m["head"]), int(m["row"])): m for m in merges}
+    parts_used = []
     for b in range(B):
         for h in range(H):
-            sel = live & (entries["batch"] == b) & (entries["head"] == h)
-            assert sorted(tuple(int(e[f]) for f in fields) for e in entries[sel]) == want
-    # live entries lead every list, followed by at least two end marks
-    assert (np.diff(live.astype(int), axis=1) <= 0).all() and not live[:, -2:].any()
-    # a (batch, head) only appears in the lists of slots of the same residue mod 8
-    slot = np.broadcast_to(np.arange(1024)[:, None], live.shape)
-    bh = entries["batch"] * H + entries["head"]
-    assert np.array_equal(slot[live] % 8, bh[live] % 8)
-    # the lists are balanced (key blocks + 2 per item) and the cut global rows lead their lists
-    loads = np.where(live, entries["count"].astype(np.int64) + 2, 0).sum(axis=1)
-    assert loads.max() <= loads.mean() + 10, (loads.max(), loads.mean())
-    assert (entries["count"][:, 1:][live[:, 1:]] <= 8).all()
+            lut = luts_per_head[h if len(luts_per_head) > 1 else 0]["nn_lut"]
+            for row in range(nb):
+                count = int(lut[row, 1])
+                pieces = sorted(seen.get((b, h, row), []))
+                if count == 0:
+                    assert not pieces and merge_of[(b, h, row)]["nparts"] == 0
+                    continue
+                assert sum(pc[1] for pc in pieces) == count
+                assert [pc[0] for pc in pieces] == list(np.cumsum([0] + [pc[1] for pc in pieces[:-1]]))
+                if len(pieces) == 1:
+                    assert pieces[0][2] == 0 and (b, h, row) not in merge_of
+                else:
+                    m = merge_of[(b, h, row)]
+                    assert m["nparts"] == len(pieces) and m["q_off"] == (b * L + row * bs) * H + h
+                    assert [pc[3] for pc in pieces] == list(range(int(m["part"]), int(m["part"]) + len(pieces)))
+                    assert [pc[4] for pc in pieces] == list(range(len(pieces))) and all(pc[5] == len(pieces) for pc in pieces)
+                    parts_used += [pc[3] for pc in pieces]
+    assert sorted(parts_used) == list(range(plan.n_parts))
 
 
-def test_plan_per_head_tables_and_odd_sizes():
-    nb, B, H = 16, 3, 4
+def test_stream_covers_every_block_once():
+    nb, B, H, bs = 64, 4, 12, 64
+    luts = sfb.build_luts(sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 1234)))
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=1024)
+    check_stream(stream, [luts], nb, B, H, bs)
+    plan, slots, items = stream["plan"], stream["slots"], stream["items"]
+    assert plan.n_blocks == 622 * B * H
+    # a (batch, head) only appears in the streams of slots of the same residue mod 8
+    for s in range(plan.wg_slots):
+        its = items[slots[s]["item_begin"]:slots[s]["item_begin"] + slots[s]["n_items"]]
+        assert ((its["batch"] * H + its["head"]) % 8 == s % 8).all()
+    # the streams are level: only the two 64-block rows of a head are cut, every stream costs about the same
+    assert plan.balance > 0.93
+    assert (items["count"][items["kind"] == 0] <= 8).all()
+    assert plan.n_merges == 2 * B * H
+    assert slots["n_blocks"].max() <= 33
+    # few, long chunks instead: streams differ by up to a short row
+    coarse = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=1024, level=False)
+    check_stream(coarse, [luts], nb, B, H, bs)
+    assert coarse["plan"].n_parts == 3 * 2 * B * H and coarse["plan"].balance > 0.9
+    assert coarse["plan"].resident == coarse["plan"].wg_slots == 1024
+    # resident streams filled to 70 % of their share, the shortest rows and the merges in streams of their own behind
+    tailed = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=1024, level=False, tail_percent=30)
+    check_stream(tailed, [luts], nb, B, H, bs)
+    tp, ts, ti = tailed["plan"], tailed["slots"], tailed["items"]
+    assert tp.resident == 1024 and tp.wg_slots > 1024 and (tp.wg_slots - 1024) % 8 == 0
+    late = ts[1024:]
+    assert ((late["n_items"] + late["n_merges"]) <= 1).all()
+    assert ts[:1024]["n_merges"].sum() == 0 and late["n_merges"].sum() == 2 * B * H
+    assert 0.6 < ts[:1024]["n_blocks"].sum() / tp.n_blocks < 0.8
+    for s in np.flatnonzero(late["n_items"]):
+        it = ti[late[s]["item_begin"]]
+        assert (it["batch"] * H + it["head"]) % 8 == (1024 + s) % 8 and it["kind"] == 0
+    # a merge stands in a stream behind those of all chunks of its row
+    owner = np.repeat(np.arange(tp.wg_slots), ts["n_items"])
+    for m, s in zip(tailed["merges"], np.repeat(np.arange(tp.wg_slots), ts["n_merges"])):
+        if m["nparts"]:
+            mine = (ti["kind"] == 1) & (ti["part"] >= m["part"]) & (ti["part"] < m["part"] + m["nparts"])
+            assert mine.sum() == m["nparts"] and owner[mine].max() < s
+    nbytes = sfb.stream_workspace_bytes(stream, 64)
+    assert nbytes == (plan.n_parts * 4 + 255) // 256 * 256 + plan.n_parts * (64 * 64 + 256) * 4 + 256
+
+
+def test_stream_per_head_tables_odd_sizes_and_empty_rows():
+    nb, B, H, bs = 16, 3, 4, 32
     lay = sfb.layout_fixed(H, nb, 4, causal=True)
     per_head = [sfb.build_luts(lay[h]) for h in range(H)]
     nn = np.concatenate([p["nn_lut"] for p in per_head])
-    for wg_slots in (1, 7, 40):
-        plan = sfb.build_plan(nn, nb, B, H, max_blocks=2, lut_heads=H, wg_slots=wg_slots)
-        entries = plan["plan"]
-        live = entries["count"] != sfb.PLAN_END
-        for h in range(H):
-            sched = sfb.build_schedule(per_head[h]["nn_lut"], nb, 2)
-            sel = live & (entries["head"] == h)
-            assert sel.sum() == B * sched["n_items"]
-            assert sorted(entries["lut_first"][sel & (entries["batch"] == 0)]) == sorted(sched["items"]["lut_first"])
-        assert not live[:, -2:].any()
+    for wg_slots in (1, 7, 40, 256):
+        for level in (True, False):
+            stream = sfb.build_stream(nn, nb, B, H, bs, lut_heads=H, wg_slots=wg_slots, level=level)
+            check_stream(stream, per_head, nb, B, H, bs)
+    holed = sfb.layout_bigbird(nb, 1, 2, True, sfb.bigbird_draw(nb, 1, 2, True, 3, 5)).copy()
+    holed[5, :] = 0        # a block-row without key blocks
+    holed = sfb.build_luts(holed)
+    for wg_slots in (3, 64, 1024):   # 1024: far more streams than rows
+        for level in (True, False):
+            stream = sfb.build_stream(holed["nn_lut"], nb, B, H, bs, wg_slots=wg_slots, level=level)
+            check_stream(stream, [holed], nb, B, H, bs)
+            assert (stream["merges"]["nparts"] == 0).sum() == B * H
+            assert (stream["items"]["count"] > 0).all()
+    dense = sfb.build_luts(sfb.layout_full(8, causal=False))
+    for wg_slots, B2 in ((16, 1), (1024, 2)):
+        stream = sfb.build_stream(dense["nn_lut"], 8, B2, 3, 64, wg_slots=wg_slots)
+        check_stream(stream, [dense], 8, B2, 3, 64)

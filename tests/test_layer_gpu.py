@@ -191,3 +191,57 @@ def test_encoder_layer_matches_oracle(bf16, max_blocks):
         err = rel_err(got, want)
         print("layer rel err", err)
         assert err <= (1e-2 if bf16 else 1e-4)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("pre_ln", [False, True])
+def test_encoder_layer_streamed_matches_oracle(bf16, pre_ln):
+    """The layer with its attention launched over streams (sfb_encoder_layer_forward_streamed), both wirings."""
+    B, L, H, d, ffn, bs = 2, 1024, 12, 64, 3072, 64
+    n, nb = H * d, L // bs
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    w = layer_weights(n, ffn, 100)
+    x = orc.fill_normal((B * L, n), 300)
+    oracle = orc.encoder_layer_pre_ln if pre_ln else orc.encoder_layer
+    want = oracle(x, w, luts["nn_lut"], B, L, H, d, ffn, bs, luts["blocks"], operands_bf16=bf16, nthreads=16)
+    layer = sfb.EncoderLayer({k: T(v) for k, v in w.items()}, luts, bs, H, d, ffn,
+                             dtype=sfb.BF16 if bf16 else sfb.F32, pre_ln=pre_ln, streamed=True)
+    for _ in range(2):
+        got = layer.forward(T(x), B, L).cpu().numpy()
+        torch.cuda.synchronize()
+        assert rel_err(got, want) <= (1e-2 if bf16 else 1e-4)
+
+
+def test_encoder_layer_per_head_luts_and_masks():
+    """The reference's `fixed` pattern gives every head its own layout and mask (fixed_fusion_test.cu:38-39, 58-106):
+    the streamed layer against the same layer put together from the oracle's operations (fp32)."""
+    B, L, H, d, ffn, bs = 2, 512, 4, 64, 512, 32
+    n, nb = H * d, L // bs
+    lay = sfb.layout_fixed(H, nb, 4, causal=True)
+    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
+    blocks = per_head[0]["blocks"]
+    nn = np.concatenate([p["nn_lut"] for p in per_head])
+    masks = np.concatenate([sfb.pack_mask(sfb.element_mask(p["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG)) for p in per_head])
+    w = layer_weights(n, ffn, 500)
+    x = orc.fill_normal((B * L, n), 700)
+
+    def proj(a, wn, bn):
+        return orc.bias(orc.sgemm(a, w[wn], nthreads=16), w[bn])
+    q, k, v = (proj(x, "w" + c, "b" + c).reshape(B, L, H, d) for c in "qkv")
+    attn = orc.attention(q, k, v, nn, bs, 1.0 / np.sqrt(d), mask=masks, lut_heads=H, mask_heads=H, blocks=blocks,
+                         nthreads=16).reshape(B * L, n)
+    x1 = orc.layernorm(x + proj(attn, "wo", "bo"), w["ln1_g"], w["ln1_b"])[0]
+    want = orc.layernorm(x1 + proj(orc.gelu(proj(x1, "w1", "b1")), "w2", "b2"), w["ln2_g"], w["ln2_b"])[0]
+
+    luts = sfb.Luts(nn_lut=nn, blocks=blocks, nb=nb)
+    layer = sfb.EncoderLayer({k_: T(v_) for k_, v_ in w.items()}, luts, bs, H, d, ffn, dtype=sfb.F32, streamed=True,
+                             lut_heads=H, mask_heads=H)
+    got = layer.forward(T(x), B, L, mask=sfb.to_device(masks)).cpu().numpy()
+    torch.cuda.synchronize()
+    assert rel_err(got, want) <= 1e-4
+    # the same in bf16 against the fp32 result (operand rounding only)
+    layer16 = sfb.EncoderLayer({k_: T(v_) for k_, v_ in w.items()}, luts, bs, H, d, ffn, dtype=sfb.BF16, streamed=True,
+                               lut_heads=H, mask_heads=H)
+    got16 = layer16.forward(T(x), B, L, mask=sfb.to_device(masks)).cpu().numpy()
+    torch.cuda.synchronize()
+    assert rel_err(got16, want) <= 2e-2
