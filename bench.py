@@ -122,6 +122,36 @@ def _time(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def _median_ms(torch, fn, groups=40, per_group=50):
+    """Median over groups of back-to-back launches (one event pair per group, so the events' own cost and the gaps
+    they open between launches stay out of the figure)."""
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(groups)]
+    for a, b in pairs:
+        a.record()
+        for _ in range(per_group):
+            fn()
+        b.record()
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b) / per_group for a, b in pairs)
+    return times[len(times) // 2]
+
+
+def time_streamed(sfb, torch, luts, q, k, v, bs, blocks, scale, flops, peak):
+    """The same attention launched over streams (resident work-groups walking chained items, sfb_build_stream):
+    few long chunks of the cut rows, no dynamic tail."""
+    B, L, H, d = q.shape
+    stream = sfb.build_stream(luts["nn_lut"], L // bs, B, H, bs, level=False)
+    blob = sfb.to_device(stream["blob"])
+    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    out = torch.empty((B, L, H, d), device="cuda", dtype=torch.float32)
+    nn = sfb.to_device(luts["nn_lut"])
+    fn = lambda: sfb.fused_attention_streamed(q, k, v, nn, blob, stream, ws, bs, blocks, scale, out=out)
+    ms = _time(torch, fn, 500, 100)
+    assert sfb.stream_status(stream, d, ws) == 0
+    return {"ms_per_call": ms, "frac_of_mfma_peak": flops / (ms * 1e-3) / 1e12 / peak, "streams": int(stream["plan"].wg_slots),
+            "partial_records": int(stream["plan"].n_parts), "balance": float(stream["plan"].balance)}
+
+
 def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
     """sdd -> masked softmax -> dsd with S and P in HBM (bf16 storage for bf16 inputs, else fp32)."""
     B, L, H, d = q.shape
@@ -141,6 +171,12 @@ def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
     parts = {"sdd_ms": _time(torch, lambda: sfb.bst_sgemm_nt(nt, q, k, bs, blocks, c=S), 200, 20),
              "softmax_ms": _time(torch, lambda: sfb.BlocksparseMaskedSoftmax(nn, None, S, nb, scale, y=P), 200, 20),
              "dsd_ms": _time(torch, lambda: sfb.bst_sgemm_xn(nn, P, v, nb, c=O), 200, 20)}
+    # HBM rate of each stage on its algorithmic bytes: the sparse tensor once, the dense operands / result once
+    sparse_bytes = S.numel() * S.element_size()
+    dense_bytes = q.numel() * q.element_size()
+    parts["sdd_hbm_GBs"] = (2 * dense_bytes + sparse_bytes) / parts["sdd_ms"] / 1e6
+    parts["softmax_hbm_GBs"] = 2 * sparse_bytes / parts["softmax_ms"] / 1e6
+    parts["dsd_hbm_GBs"] = (sparse_bytes + dense_bytes + O.numel() * 4) / parts["dsd_ms"] / 1e6
     # sdd + softmax in one kernel (P still goes through HBM): one work-group per block-row against the
     # reference's own decomposition, one work-group per block with flag / spin exchange
     order = sfb.to_device(luts["row_order"])
@@ -229,9 +265,15 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
     x = sfb.embedding_lookup(tok, ids, pos).reshape(B * L, n)
     out = {"shape": "B8 L4096 hidden 768 heads 12 ffn 3072, BigBird block 64", "gemm_flops": 2.0 * B * L * (4 * n * n + 2 * n * ffn)}
     y = torch.empty_like(x)
+    attn_flops = luts["blocks"] * B * H * 4.0 * bs * bs * d
     for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
         layer = sfb.EncoderLayer(w, luts, bs, H, d, ffn, dtype=code, max_blocks=max_blocks)
-        out["ms_per_layer_" + name] = _time(torch, lambda: layer.forward(x, B, L, out=y), 20, 5)
+        ms = _time(torch, lambda: layer.forward(x, B, L, out=y), 20, 5)
+        out["ms_per_layer_" + name] = ms
+        # the layer's matrix work (GEMMs + attention blocks) against the MFMA peak of its operand type
+        out["roofline_" + name] = {"bound": "mfma", "achieved": (out["gemm_flops"] + attn_flops) / (ms * 1e-3) / 1e12,
+                                   "peak": PEAK_TFLOPS[name], "unit": "TFLOP/s",
+                                   "frac": (out["gemm_flops"] + attn_flops) / (ms * 1e-3) / 1e12 / PEAK_TFLOPS[name]}
         assert torch.isfinite(y).all()
         del layer
     return out
@@ -347,6 +389,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
 
+    # untimed: bring the clocks up before the warm-up steps (a handful of 50 us launches does not)
+    ramp_until = time.perf_counter() + 0.3
+    while time.perf_counter() < ramp_until:
+        for _ in range(200):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -361,6 +409,7 @@ def main():
     kernel_ms = start.elapsed_time(stop) / args.steps   # HIP events on the launch stream
     ms_per_step = wall_ms / args.steps
     assert torch.isfinite(out).all()
+    median_ms = _median_ms(torch, step)
 
     traffic = read_traffic(args.workload, dtype)
     tflops = flops / (ms_per_step * 1e-3) / 1e12
@@ -375,16 +424,19 @@ def main():
                                "blocks, %s inputs, fp32 accumulate/output" %
                                (args.workload, pattern, B, H, L, d, bs, blocks, dtype),
                    "max_blocks": args.max_blocks},
-        "ms_per_attention_call": kernel_ms,
+        "ms_per_attention_call": kernel_ms, "ms_per_attention_call_median": median_ms,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
                      "frac": achieved / peak, "traffic": traffic,
                      "kernel": "fused_attention_%s_kernel<%d,%d>" % (dtype if bf16 else "f32", bs, d),
-                     "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms,
+                     "algorithmic_flops_per_launch": flops, "avg_launch_ms": kernel_ms, "median_launch_ms": median_ms,
+                     "frac_at_median": flops / (median_ms * 1e-3) / 1e12 / peak,
                      "hbm_algorithmic_bytes_per_launch": algo_bytes,
                      "hbm_achieved_GBs": algo_bytes / (kernel_ms * 1e-3) / 1e9,
                      "hbm_frac": algo_bytes / (kernel_ms * 1e-3) / 1e9 / PEAK_HBM_GBS},
     }
     if not args.skip_extras:
+        if bf16 or d == 64:
+            result["streamed"] = time_streamed(sfb, torch, luts, q, k, v, bs, blocks, scale, flops, peak)
         result["unfused"] = time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
         result["backward_unfused"] = time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
         if bf16:
