@@ -55,10 +55,19 @@ struct Bf16DirectTiles {
         const uint32_t rr = lane >> 3, pos = lane & 7u;
         return rr * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
     }
+    // The same for a tile whose LDS rows hold the source rows in the order that makes the 8 k-slots of a lane
+    // in the second product, rows 16u + 8(j/4) + 4*half + j%4 of the tile, the 8 consecutive source rows
+    // 32*half + 8u + j: LDS row 16u + 8a + 4h + c holds source row 32h + 8u + 4a + c, which is 4n + 32(rr/4) + rr%4
+    // for row rr of 8-row group n.  Used with load_rows<4>: the group's base advances by 4 source rows.
+    static __device__ __forceinline__ uint32_t lane_source_by_halves(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
+        const uint32_t rr = lane >> 3, pos = lane & 7u;
+        return (32u * (rr >> 2) + (rr & 3u)) * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
+    }
     // Load number i (0 .. LOADS-1) of this wave's share of one tile: 8 rows = 1 KiB.  g_tile: address of
     // the tile's first row (uniform); lds_tile: LDS byte address of the tile (uniform); src_even /
     // src_odd from lane_source().
     static constexpr int LOADS = GROUPS / NW;
+    template <int GROUP_ROWS = 8>
     static __device__ __forceinline__ void load_rows(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
         static_assert(D == 64, "128-byte rows");
@@ -68,7 +77,7 @@ struct Bf16DirectTiles {
         else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
         // scalar 64-bit base + 32-bit lane offset: no vector address arithmetic.  The instruction takes its
         // LDS destination from M0, which is written here; nothing else in these kernels depends on M0.
-        const uint64_t ga = (uint64_t)(g_tile + (size_t)n * 8u * row_bytes);
+        const uint64_t ga = (uint64_t)(g_tile + (size_t)n * (uint32_t)GROUP_ROWS * row_bytes);
         const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
         const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
         const uint64_t base = ((uint64_t)ga_hi << 32) | (uint64_t)ga_lo;
@@ -82,6 +91,13 @@ struct Bf16DirectTiles {
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) load_rows(lds_tile, g_tile, i, wave, src_even, src_odd, row_bytes);
+    }
+    // with src_even / src_odd from lane_source_by_halves()
+    static __device__ __forceinline__ void load_tile_by_halves(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
+                                                               uint32_t src_even, uint32_t src_odd,
+                                                               uint32_t row_bytes) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) load_rows<4>(lds_tile, g_tile, i, wave, src_even, src_odd, row_bytes);
     }
     // Per-lane byte offset of the score fragment of k-step 0 in key tile 0; k-step ks is at (base ^ ks*32),
     // key tile kt 4096 bytes further.

@@ -193,19 +193,114 @@ struct SddParams {
     uint32_t blocks, heads, ctx_a, ctx_b, lut_stride;
 };
 
+// Blocks per work-group: a launch of one work-group per block is bound by the rate at which work-groups start,
+// not by memory; a group of consecutive blocks also keeps the next block's operands in flight under the
+// current block's product and write-out.
+constexpr uint32_t kSddGroup = 2;
+
 template <int BS, int D, typename TIn, typename TOut>
 __global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
-    const uint32_t blk = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+    const uint32_t b = blockIdx.y, h = blockIdx.z;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
-    const sfb_uint2 e = p.lut[(size_t)h * p.lut_stride + blk];
+    const uint32_t blk0 = blockIdx.x * kSddGroup;
+    const uint32_t n = p.blocks - blk0 < kSddGroup ? p.blocks - blk0 : kSddGroup;
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride + blk0;
     const uint32_t row_stride = p.heads * D;
-    const TIn* q_row = (const TIn*)p.a + token_offset(b, e.x * BS + wave * 32 + qn, h, p.ctx_a, p.heads, D);
-    const TIn* k_blk = (const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, D);
-    f32x16 s[BS / 32];
-    score_tile_direct<BS, D, TIn>(s, q_row, k_blk, row_stride, qn, half);
     __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TOut>::BYTES];
-    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32) * BS;
-    RowSlab<BS, TOut>::store(out, s, slabs[wave], lane);
+    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk0) * BS + wave * 32) * BS;
+    KTile<BS, D, TIn> k_tile[2];
+    QRow<D, TIn> q_row[2];
+    auto fetch = [&](uint32_t g, int buf) {
+        const sfb_uint2 e = lut[g];
+        q_row[buf].load((const TIn*)p.a + token_offset(b, e.x * BS + wave * 32 + qn, h, p.ctx_a, p.heads, D), half);
+        k_tile[buf].load((const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, D), row_stride, qn, half);
+    };
+    fetch(0, 0);
+#pragma unroll
+    for (uint32_t g = 0; g < kSddGroup; ++g) {
+        if (g < n) {
+            if (g + 1 < n) fetch(g + 1, (g + 1) & 1);
+            f32x16 s[BS / 32];
+            score_tile<BS, D, TIn>(s, k_tile[g & 1], q_row[g & 1]);
+            RowSlab<BS, TOut>::store(out + (size_t)g * BS * BS, s, slabs[wave], lane);
+        }
+    }
+}
+
+// The same product for bf16 operands, 64 x 64 blocks and 64 features: a work-group of two waves walks
+// kSddStreamGroup consecutive blocks of the look-up table.  K tiles go straight into LDS (whole 128-byte lines,
+// fetched once per block; read as fragments out of memory every line is fetched by both waves in 32-byte pieces),
+// two blocks ahead in a ring of three; the query fragments stay in registers while the block-row does not change.
+// Every wait is counted in the loads and stores actually issued, which complete in issue order: K(g) is followed
+// by the stores of blocks g-2 and g-1 and the loads of K(g+1).
+constexpr uint32_t kSddStreamGroup = 8;
+
+template <typename TOut>
+__global__ __launch_bounds__(128) void sdd_nt_stream_kernel(SddParams p) {
+    constexpr int BS = 64, D = 64, KT = BS / 32;
+    using TD = Bf16DirectTiles<BS, D>;
+    using Slab = RowSlab<BS, TOut>;
+    constexpr int TILE = TD::TILE_BYTES;
+    typedef const uint32_t __attribute__((address_space(4)))* const_words;
+    __shared__ __attribute__((aligned(1024))) uint8_t tiles[3 * TILE];
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][Slab::BYTES];
+    const uint32_t b = blockIdx.y, h = blockIdx.z;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    const uint32_t blk0 = blockIdx.x * kSddStreamGroup;
+    const uint32_t n = p.blocks - blk0 < kSddStreamGroup ? p.blocks - blk0 : kSddStreamGroup, last = n - 1;
+    const const_words lut_words = (const_words)(uintptr_t)(p.lut + (size_t)h * p.lut_stride + blk0);
+    const uint32_t row_bytes = p.heads * D * 2;
+    const uint8_t* const k_base = (const uint8_t*)p.b + token_offset(b, 0, h, p.ctx_b, p.heads, D) * 2;
+    const uint8_t* const q_base = (const uint8_t*)p.a + token_offset(b, 0, h, p.ctx_a, p.heads, D) * 2;
+    const uint32_t src_even = TD::lane_source(lane, 0, row_bytes), src_odd = TD::lane_source(lane, 1, row_bytes);
+    const uint32_t lds0 = TD::lds_address(tiles), k_lane = TD::k_lane_base(qn, half);
+    const uint32_t q_lane = (wave * 32 + qn) * row_bytes + half * 16;   // k-step ks: 32 bytes further each
+    TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk0) * BS + wave * 32) * BS;
+    auto fetch_k = [&](uint32_t g, uint32_t buf) {
+        const uint32_t col = lut_words[2 * g + 1];
+        TD::load_tile(lds0 + buf * TILE, k_base + (size_t)col * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+    };
+    // a fetch past the group's end repeats the last block: the counts stay the same in every step
+    fetch_k(0, 0);
+    fetch_k(1 < n ? 1 : last, 1);
+    u32x4 qf[D / 16];
+    uint32_t cur_row = 0xffffffffu;
+    for (uint32_t g = 0; g < n; ++g) {
+        const uint32_t row = lut_words[2 * g];
+        if (row != cur_row) {
+            // a new block-row (always in the first step): its query fragments, waited for at once
+            static_assert(D / 16 == 4, "four k-steps");
+            const uint8_t* q_rows = q_base + (size_t)row * BS * row_bytes;
+            asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                         "global_load_dwordx4 %1, %4, %5 offset:32\n\t"
+                         "global_load_dwordx4 %2, %4, %5 offset:64\n\t"
+                         "global_load_dwordx4 %3, %4, %5 offset:96\n\t"
+                         "s_waitcnt vmcnt(0)"
+                         : "=&v"(qf[0]), "=&v"(qf[1]), "=&v"(qf[2]), "=&v"(qf[3])
+                         : "v"(q_lane), "s"(q_rows)
+                         : "memory");
+            cur_row = row;
+        }
+        if (sizeof(TOut) == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");   // 4 loads + 2 x 4 stores
+        else asm volatile("s_waitcnt vmcnt(20)" ::: "memory");                       // 4 loads + 2 x 8 stores
+        __syncthreads();   // K(g) is in LDS for every wave, and every wave is done with K(g-1)
+        fetch_k(g + 2 < n ? g + 2 : last, (g + 2) % 3u);
+        const uint8_t* k_read = tiles + (g % 3u) * TILE;
+        f32x16 s[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+                s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::k_frag(k_read, k_lane, kt, ks),
+                                                                __builtin_bit_cast(bf16x8, qf[ks]), s[kt], 0, 0, 0);
+        Slab::store(out + (size_t)g * BS * BS, s, slabs[wave], lane);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing in flight towards LDS when the group ends
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -918,13 +1013,16 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr bool kBf16 = sizeof(TV) == 2;
     using TD = Bf16DirectTiles<BS, D>;
     using TF = F32Tiles<BS, D>;
-    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
+    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 3 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c);
+    // Block-rows are taken from both ends of the context inwards, the last and the first one of every head before
+    // anything else: the long rows of causal layouts are the last ones (blocksparse.h:746-748), those of layouts
+    // with global tokens the first and the last; started late, a long row is the tail of the launch.
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c, p.nb_c >= 2 ? 2 : 0);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
-    const uint32_t r = p.nb_c - 1 - work.rank;   // long rows of causal layouts first (blocksparse.h:746-748)
+    const uint32_t r = (work.rank & 1u) ? work.rank / 2 : p.nb_c - 1 - work.rank / 2;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
@@ -942,48 +1040,91 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
 
     if constexpr (kBf16 && sizeof(TP) == 2 && BS == 64) {
-        // bf16 P and V: both tiles of a key block go straight into LDS (LDS-direct loads, double-buffered,
-        // swizzled rows, see Bf16DirectTiles); V^T fragments by transposing reads, P^T fragments by two 8-byte
-        // reads per product step.  One barrier per key block, loads of the next block in flight meanwhile.
-        constexpr int PU = BS / 16, TILE = TD::TILE_BYTES;
-        static_assert(BS == 64 || BS == 32, "block size");
+        // bf16 P and V.  P is the stream from memory: it is read once, straight into registers in operand layout,
+        // kDepth key blocks ahead, so that a work-group keeps several tiles in flight without spending LDS on
+        // them (LDS would bound the work-groups per CU, and with them the bytes in flight).  For that a lane's 8
+        // k-slots of a product step must be 8 consecutive keys (one 16-byte load): the V tile is laid into LDS
+        // with its key rows in the matching order (lane_source_by_halves).  V tiles (L2 hits mostly) go through a
+        // ring of three LDS buffers, two blocks ahead.  Loads and stores complete in issue order, which the
+        // counted waits below rely on.
+        constexpr int PU = BS / 16, TILE = TD::TILE_BYTES, kDepth = 4;
         const uint32_t row_bytes = row_stride * 2;
-        const uint32_t v_even = TD::lane_source(lane, 0, row_bytes), v_odd = TD::lane_source(lane, 1, row_bytes);
-        const uint32_t p_even = TD::lane_source(lane, 0, BS * 2), p_odd = TD::lane_source(lane, 1, BS * 2);
+        const uint32_t v_even = TD::lane_source_by_halves(lane, 0, row_bytes);
+        const uint32_t v_odd = TD::lane_source_by_halves(lane, 1, row_bytes);
         const uint32_t lds0 = TD::lds_address(smem), v_lane = TD::v_lane_base(lane);
         const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
-        const uint8_t* const p_base = (const uint8_t*)P;
-        // P tile rows are BS bf16 = BS*2 bytes: 128-byte rows for BS 64 (the V layout), 64-byte rows for BS 32
-        // (two P rows per 128-byte LDS row; handled by the generic path below)
-        auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
-            TD::load_tile(lds0 + buf * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, v_even, v_odd, row_bytes);
-            TD::load_tile(lds0 + (2 + buf) * TILE, p_base + (size_t)e.x * BS * BS * 2, wave, p_even, p_odd, BS * 2);
+        // step u of this lane: keys 32*half + 8u .. + 7 of query row q_in_block
+        const uint32_t p_lane = q_in_block * (BS * 2u) + half * 64u;
+        u32x4 pr[kDepth][PU];
+        // look-up entries through scalar loads (constant address space): a vector load here would be waited for
+        // with vmcnt(0), which drains every tile in flight
+        typedef const uint32_t __attribute__((address_space(4)))* const_words;
+        const const_words lut_words = (const_words)(uintptr_t)(lut + off);
+        // The P loads are written out (scalar base + lane offset) so that every wait in the loop can be stated in
+        // loads actually issued: the compiler does not count the LDS-direct loads of the V tiles, and its own
+        // waits for P registers would fall short of the depth.  The registers are tied to the wait below.
+        auto fetch_p = [&](u32x4 (&dst)[PU], uint32_t j, bool real) {
+            static_assert(PU == 4, "four 16-byte loads per lane and block");
+            const uint32_t blk = lut_words[2 * j];
+            const uint32_t lane_offset = real ? p_lane : 0u;   // a fetch past the row's end: one cache line
+            const uint8_t* base = (const uint8_t*)P + (size_t)blk * (BS * BS * 2u);
+            // no non-temporal hint: the four loads of a lane share their cache lines with the neighbouring lane's,
+            // and with the hint every one of them goes to L2 by itself (measured: 1.5 x the time)
+            asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
+                         "global_load_dwordx4 %1, %4, %5 offset:16\n\t"
+                         "global_load_dwordx4 %2, %4, %5 offset:32\n\t"
+                         "global_load_dwordx4 %3, %4, %5 offset:48"
+                         : "=&v"(dst[0]), "=&v"(dst[1]), "=&v"(dst[2]), "=&v"(dst[3])
+                         : "v"(lane_offset), "s"(base)
+                         : "memory");
         };
-        auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
-            const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
-            return u;
+        auto fetch_v = [&](uint32_t j, uint32_t buf) {
+            const uint32_t col = lut_words[2 * j + 1];
+            TD::load_tile_by_halves(lds0 + buf * TILE, v_base + (size_t)col * BS * row_bytes, wave, v_even, v_odd,
+                                    row_bytes);
         };
-        if (count > 0) fetch(uniform(lut[off]), 0);
-        // P^T operand of step u: keys 16u + 8(j/4) + 4*half + j%4 of query row q_in_block: 8 bytes of chunk 2u
-        // and 8 bytes of chunk 2u + 1 of that row, at byte 8*half
-        const uint32_t p_row = q_in_block * 128u + half * 8u, p_swz = TD::swz(q_in_block) << 4;
-        for (uint32_t j = 0; j < count; ++j) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();   // tiles of block j are in LDS for every wave, and every wave is done with block j-1
-            fetch(uniform(lut[off + (j + 1 < count ? j + 1 : j)]), (j + 1) & 1);
-            const uint8_t* v_read = smem + (j & 1) * TILE;
-            const uint8_t* p_read = smem + (2 + (j & 1)) * TILE + p_row;
+        // Issue order: V(0) V(1) P(0) .. P(kDepth-1), then per block j: V(j+2), [product], P(j+kDepth).  Every
+        // fetch is issued whether or not its block exists (past the row's end the last block is fetched again, a
+        // cache hit, into a buffer or registers that nobody reads): the number of loads between a tile and its use
+        // is then the same in every iteration, which is what a counted wait needs.  V(j) is followed by V(j+1)
+        // and two P tiles (more for j < 2), 4 loads per wave each.
+        if (count > 0) {
+            const uint32_t last = count - 1;
+            fetch_v(0, 0);
+            fetch_v(1 < count ? 1 : last, 1);
 #pragma unroll
-            for (int u = 0; u < PU; ++u) {
-                const u32x2 lo = *(const u32x2*)(p_read + ((uint32_t)(2 * u * 16) ^ p_swz));
-                const u32x2 hi = *(const u32x2*)(p_read + ((uint32_t)((2 * u + 1) * 16) ^ p_swz));
-                const u32x4 pb = {lo.x, lo.y, hi.x, hi.y};
-                const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pb);
+            for (int d = 0; d < kDepth; ++d) fetch_p(pr[d], (uint32_t)d < count ? d : last, (uint32_t)d < count);
+            for (uint32_t j0 = 0; j0 < count; j0 += kDepth) {
 #pragma unroll
-                for (int mt = 0; mt < NO; ++mt)
-                    o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u), bfrag,
-                                                                        o_acc[mt], 0, 0, 0);
+                for (int d = 0; d < kDepth; ++d) {
+                    const uint32_t j = j0 + d;
+                    // V(j) and, issued before it, P(j) have landed when only the 12 loads issued after V(j) remain
+                    asm volatile("s_waitcnt vmcnt(12)"
+                                 : "+v"(pr[d][0]), "+v"(pr[d][1]), "+v"(pr[d][2]), "+v"(pr[d][3])
+                                 :
+                                 : "memory");
+                    __syncthreads();   // V(j) is in LDS for every wave, and every wave is done with V(j-1)
+                    fetch_v(j + 2 < count ? j + 2 : last, (j + 2) % 3u);
+                    const uint8_t* v_read = smem + (j % 3u) * TILE;
+                    // the row is walked in whole groups of kDepth blocks: a step past its end multiplies by zeros
+                    // and keeps the sequence of loads and barriers (an exit or a branch in the middle of the group
+                    // would leave the compiler with paths on which the load counts, or the registers, differ)
+                    const uint32_t live = j < count ? 0xffffffffu : 0u;
+#pragma unroll
+                    for (int u = 0; u < PU; ++u) {
+                        const u32x4 pv = {pr[d][u].x & live, pr[d][u].y & live, pr[d][u].z & live, pr[d][u].w & live};
+                        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pv);
+#pragma unroll
+                        for (int mt = 0; mt < NO; ++mt)
+                            o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u),
+                                                                                bfrag, o_acc[mt], 0, 0, 0);
+                    }
+                    // the registers of P(j) take P(j + kDepth): not before the product has read them
+                    __builtin_amdgcn_sched_barrier(0);
+                    fetch_p(pr[d], j + kDepth < count ? j + kDepth : last, j + kDepth < count);
+                }
             }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing in flight towards LDS when the group ends
         }
     } else if constexpr (kBf16) {
         // V tiles double-buffered in LDS by LDS-direct loads, V^T fragments by transposing reads (see
@@ -1353,7 +1494,7 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
     SddParams p = {lut, a, b, c, blocks, head_dim, ctx_blks_a * block_size, ctx_blks_b * block_size,
                    lut_heads > 1 ? lut_dim : 0};
-    const dim3 grid(blocks, batch_dim, head_dim);
+    const dim3 grid((blocks + kSddGroup - 1) / kSddGroup, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (state_dim != 64) {
@@ -1363,6 +1504,12 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
         else SFB_DISPATCH_OTHER_D(state_dim, out_dtype, SFB_CALL32);
 #undef SFB_CALL64
 #undef SFB_CALL32
+        return launch_status();
+    }
+    if (block_size == 64 && in_dtype == SFB_BF16) {
+        const dim3 stream_grid((blocks + kSddStreamGroup - 1) / kSddStreamGroup, batch_dim, head_dim);
+        if (out_dtype == SFB_BF16) sdd_nt_stream_kernel<__bf16><<<stream_grid, dim3(128), 0, s>>>(p);
+        else sdd_nt_stream_kernel<float><<<stream_grid, dim3(128), 0, s>>>(p);
         return launch_status();
     }
 #define SFB_CALL(BSV, TI, TO) sdd_nt_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2), 0, s>>>(p)
