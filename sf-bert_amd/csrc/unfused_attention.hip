@@ -190,7 +190,7 @@ struct SddParams {
     const void* a;
     const void* b;
     void* c;
-    uint32_t blocks, heads, ctx_a, ctx_b, lut_stride;
+    uint32_t blocks, heads, ctx_a, ctx_b, lut_stride, batch, by_xcd;
 };
 
 // Blocks per work-group: a launch of one work-group per block is bound by the rate at which work-groups start,
@@ -244,10 +244,16 @@ __global__ __launch_bounds__(128) void sdd_nt_stream_kernel(SddParams p) {
     typedef const uint32_t __attribute__((address_space(4)))* const_words;
     __shared__ __attribute__((aligned(1024))) uint8_t tiles[3 * TILE];
     __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][Slab::BYTES];
-    const uint32_t b = blockIdx.y, h = blockIdx.z;
+    // all groups of one (batch, head) run on one XCD (consecutive work-group ids go round the 8 XCDs), one
+    // (batch, head) after the other: its K is then fetched into one L2 only and stays there while it is used
+    // (the launcher asks for that when there are enough of them to keep all XCDs busy: p.by_xcd)
+    const uint32_t groups = (p.blocks + kSddStreamGroup - 1) / kSddStreamGroup;
+    const uint32_t bh = p.by_xcd ? (blockIdx.x / 8 / groups) * 8 + blockIdx.x % 8 : blockIdx.x / groups;
+    if (bh >= p.batch * p.heads) return;
+    const uint32_t b = bh / p.heads, h = bh % p.heads;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
-    const uint32_t blk0 = blockIdx.x * kSddStreamGroup;
+    const uint32_t blk0 = (p.by_xcd ? blockIdx.x / 8 % groups : blockIdx.x % groups) * kSddStreamGroup;
     const uint32_t n = p.blocks - blk0 < kSddStreamGroup ? p.blocks - blk0 : kSddStreamGroup, last = n - 1;
     const const_words lut_words = (const_words)(uintptr_t)(p.lut + (size_t)h * p.lut_stride + blk0);
     const uint32_t row_bytes = p.heads * D * 2;
@@ -738,6 +744,252 @@ __global__ __launch_bounds__(256) void masked_softmax_kernel(SoftmaxParams p) {
         for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.template in_registers<1, 8>(w.q0 + i, masked);
     } else {
         for (uint32_t i = 0; i < kSoftmaxWaveRows; ++i) rows.in_passes(w.q0 + i);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same softmax for bf16 scores in 64 x 64 blocks, by units of 8 query rows: 8 lanes hold one row of a key
+// block (16 bytes each), so a wave instruction moves 8 whole rows = 1 KiB of consecutive bytes, the row
+// reductions stay inside groups of 8 lanes (three DPP steps), and a wave needs one register slot per block of the
+// row -- no slot is spent on blocks the row does not have.  A work-group of four waves owns 32 rows of a
+// block-row: rows of up to 16 blocks one unit per wave, rows of up to 64 blocks one unit after the other with a
+// quarter of the blocks per wave (maximum and sum combined through LDS), longer rows in three passes over memory.
+// ---------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+// all-reduce over aligned groups of 8 lanes: lane ^ 1, lane ^ 2 (quad permutes), then the mirrored half row
+__device__ __forceinline__ float max_of_8(float x) {
+    x = fmaxf(x, dpp_move<0xB1>(x));
+    x = fmaxf(x, dpp_move<0x4E>(x));
+    return fmaxf(x, dpp_move<0x141>(x));
+}
+__device__ __forceinline__ float sum_of_8(float x) {
+    x += dpp_move<0xB1>(x);
+    x += dpp_move<0x4E>(x);
+    return x + dpp_move<0x141>(x);
+}
+
+template <typename TY>
+struct SoftmaxUnit {
+    static constexpr int BS = 64, SLOTS = 16;
+    static constexpr uint32_t kMaskedPair = 0xff7fff7fu;   // two bf16 of -3.39e38
+    typedef const uint32_t __attribute__((address_space(4)))* const_words;
+    const_words lut;          // entries of this block-row part: {block, column} pairs
+    const uint8_t* mask;      // this head's row-major words, or nullptr
+    const uint8_t* x;         // this (batch, head)'s blocks
+    uint8_t* y;
+    uint32_t blocks, lane;
+    int valid;
+    float c;
+
+    __device__ __forceinline__ uint32_t keep_bits(uint32_t blk, uint32_t col, uint32_t qi) const {
+        const uint32_t key0 = (lane & 7u) * 8u;
+        const int left = valid - (int)(col * BS + key0);
+        uint32_t k = left >= 8 ? 0xffu : (left <= 0 ? 0u : ((1u << left) - 1u));
+        if (mask) k &= (uint32_t)(((const uint64_t*)mask)[(size_t)qi * blocks + blk] >> key0);
+        return k;
+    }
+    static __device__ __forceinline__ float elem(const u32x4& r, int i) {
+        return (i & 1) ? __builtin_bit_cast(float, r[i >> 1] & 0xffff0000u) : bf16_bits_to_f32(r[i >> 1] & 0xffffu);
+    }
+    // Keeps the compiler from unpacking a slot long before `dep` is known and holding the floats from one pass
+    // to the next (which would cost the registers that the packed form saves).
+    static __device__ __forceinline__ void unpack_after(u32x4& r, float& dep) {
+        uint32_t a = r[0], b = r[1], c2 = r[2], d = r[3];
+        asm volatile("" : "+v"(a), "+v"(b), "+v"(c2), "+v"(d), "+v"(dep));
+        r[0] = a; r[1] = b; r[2] = c2; r[3] = d;
+    }
+    __device__ __forceinline__ void store(uint32_t blk, uint32_t q0, const float (&out)[8]) const {
+        if constexpr (sizeof(TY) == 2) {
+            const u32x4 r = {pack_bf16(out[0], out[1]), pack_bf16(out[2], out[3]), pack_bf16(out[4], out[5]),
+                             pack_bf16(out[6], out[7])};
+            __builtin_nontemporal_store(r, (u32x4*)(y + ((size_t)blk * (BS * BS * 2) + q0 * (BS * 2)) + lane * 16u));
+        } else {
+            float* dst = (float*)(y + ((size_t)blk * (BS * BS * 4) + q0 * (BS * 4)) + lane * 32u);
+            const f32x4 lo = {out[0], out[1], out[2], out[3]}, hi = {out[4], out[5], out[6], out[7]};
+            __builtin_nontemporal_store(lo, (f32x4*)dst);
+            __builtin_nontemporal_store(hi, (f32x4*)(dst + 4));
+        }
+    }
+
+    // Rows q0 .. q0+7 over `count` <= NS blocks starting at entry `first`, all in registers.  NS is count rounded
+    // up to 4: only the last three slots need a look at count.  SHARED: the row's other blocks are with the other
+    // three waves; red: [2][4][8] floats.
+    template <int NS, bool MASKED, bool SHARED>
+    __device__ __forceinline__ void in_registers(uint32_t q0, uint32_t first, uint32_t count, float* red,
+                                                 uint32_t wave) const {
+        u32x4 v[NS];
+        uint32_t blk[NS];
+        const uint32_t qi = q0 + (lane >> 3), lane16 = lane * 16;
+#define SFB_LIVE(s) ((s) <= NS - 4 || (uint32_t)(s) < count)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (SFB_LIVE(s)) {
+                blk[s] = lut[2 * (first + s)];
+                // uniform base + 32-bit lane offset
+                v[s] = __builtin_nontemporal_load((const u32x4*)(x + ((size_t)blk[s] * (BS * BS * 2) + q0 * (BS * 2)) + lane16));
+                if (MASKED) {
+                    const uint32_t keep = keep_bits(blk[s], lut[2 * (first + s) + 1], qi);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t lo = 0u - ((keep >> (2 * i)) & 1u), hi = 0u - ((keep >> (2 * i + 1)) & 1u);
+                        const uint32_t sel = (lo & 0xffffu) | (hi & 0xffff0000u);
+                        v[s][i] = (v[s][i] & sel) | (kMaskedPair & ~sel);
+                    }
+                }
+            }
+        float m0 = kMaxSeed, m1 = kMaxSeed;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (SFB_LIVE(s)) {
+#pragma unroll
+                for (int i = 0; i < 8; i += 4) {
+                    m0 = fmaxf(fmaxf(m0, elem(v[s], i)), elem(v[s], i + 1));
+                    m1 = fmaxf(fmaxf(m1, elem(v[s], i + 2)), elem(v[s], i + 3));
+                }
+            }
+        float m = max_of_8(fmaxf(m0, m1));
+        if (SHARED) {
+            if ((lane & 7u) == 0) red[wave * 8 + (lane >> 3)] = m;
+            __syncthreads();
+            const uint32_t g = lane >> 3;
+            m = fmaxf(fmaxf(red[g], red[8 + g]), fmaxf(red[16 + g], red[24 + g]));
+        }
+        float mc = m * c;
+        float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (SFB_LIVE(s)) {
+                unpack_after(v[s], mc);
+#pragma unroll
+                for (int i = 0; i < 8; i += 2) {
+                    l0 += exp2_fast(__builtin_fmaf(elem(v[s], i), c, -mc));
+                    l1 += exp2_fast(__builtin_fmaf(elem(v[s], i + 1), c, -mc));
+                }
+            }
+        float l = sum_of_8(l0 + l1);
+        if (SHARED) {
+            if ((lane & 7u) == 0) red[32 + wave * 8 + (lane >> 3)] = l;
+            __syncthreads();
+            const uint32_t g = lane >> 3;
+            l = (red[32 + g] + red[40 + g]) + (red[48 + g] + red[56 + g]);
+        }
+        float inv = 1.0f / (l + 1e-6f);
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (SFB_LIVE(s)) {
+                unpack_after(v[s], inv);
+                float out[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) out[i] = exp2_fast(__builtin_fmaf(elem(v[s], i), c, -mc)) * inv;
+                store(blk[s], q0, out);
+            }
+#undef SFB_LIVE
+    }
+    template <bool SHARED>
+    __device__ __forceinline__ void in_registers(uint32_t q0, uint32_t first, uint32_t count, bool masked, float* red,
+                                                 uint32_t wave) const {
+#define SFB_ROWS(NS)                                                                      \
+    do {                                                                                  \
+        if (masked) in_registers<NS, true, SHARED>(q0, first, count, red, wave);          \
+        else in_registers<NS, false, SHARED>(q0, first, count, red, wave);                \
+    } while (0)
+        if (count <= 4) SFB_ROWS(4);
+        else if (count <= 8) SFB_ROWS(8);
+        else if (count <= 12) SFB_ROWS(12);
+        else SFB_ROWS(16);
+#undef SFB_ROWS
+    }
+
+    // rows q0 .. q0+7 of any length: three passes over memory
+    __device__ __forceinline__ void in_passes(uint32_t q0, uint32_t count) const {
+        const uint32_t qi = q0 + (lane >> 3);
+        auto fetch = [&](uint32_t j, u32x4& r, uint32_t& keep) -> uint32_t {
+            const uint32_t blk = lut[2 * j];
+            r = *(const u32x4*)(x + (size_t)blk * (BS * BS * 2) + q0 * (BS * 2) + lane * 16);
+            keep = keep_bits(blk, lut[2 * j + 1], qi);
+            return blk;
+        };
+        float m = kMaxSeed;
+        for (uint32_t j = 0; j < count; ++j) {
+            u32x4 r;
+            uint32_t keep;
+            fetch(j, r, keep);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((keep >> i) & 1u) m = fmaxf(m, elem(r, i));
+        }
+        m = max_of_8(m);
+        float l = 0.f;
+        for (uint32_t j = 0; j < count; ++j) {
+            u32x4 r;
+            uint32_t keep;
+            fetch(j, r, keep);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if ((keep >> i) & 1u) l += exp2_fast((elem(r, i) - m) * c);
+        }
+        l = sum_of_8(l);
+        const float inv = 1.0f / (l + 1e-6f);
+        for (uint32_t j = 0; j < count; ++j) {
+            u32x4 r;
+            uint32_t keep;
+            const uint32_t blk = fetch(j, r, keep);
+            float out[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = ((keep >> i) & 1u) ? exp2_fast((elem(r, i) - m) * c) * inv : 0.f;
+            store(blk, q0, out);
+        }
+    }
+};
+
+template <typename TY>
+__global__ __launch_bounds__(256) void masked_softmax_rows8_kernel(SoftmaxParams p) {
+    constexpr int BS = 64;
+    using Unit = SoftmaxUnit<TY>;
+    __shared__ float red[64];
+    // 32 rows of a block-row per work-group.  Block-rows are taken from both ends of the context inwards, the last
+    // and the first one of every (batch, head) before anything else: the long rows of causal layouts are the
+    // last ones, those of layouts with global tokens the first and the last, and a long row that starts late is
+    // the tail of the launch.
+    const uint32_t part = blockIdx.x & 1u, item = blockIdx.x >> 1, num_bh = p.batch * p.heads;
+    const uint32_t ends = p.nb >= 2 ? 2u : 0u;
+    uint32_t rank, bh;
+    if (item < ends * num_bh) {
+        rank = item / num_bh;
+        bh = item % num_bh;
+    } else {
+        rank = ends + (item - ends * num_bh) % (p.nb - ends);
+        bh = (item - ends * num_bh) / (p.nb - ends);
+    }
+    const uint32_t r = (rank & 1u) ? rank / 2 : p.nb - 1 - rank / 2;
+    const uint32_t b = bh / p.heads, h = bh % p.heads;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
+    const typename Unit::const_words head = (typename Unit::const_words)(uintptr_t)lut;
+    const uint32_t off = head[2 * r], count = head[2 * r + 1];
+    Unit u;
+    u.lut = head + 2 * (size_t)off;
+    u.mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    u.x = (const uint8_t*)p.x + (size_t)bh * p.blocks * (BS * BS * 2);
+    u.y = (uint8_t*)p.y + (size_t)bh * p.blocks * (BS * BS * sizeof(TY));
+    u.blocks = p.blocks;
+    u.lane = threadIdx.x & 63;
+    u.valid = p.valid_len ? p.valid_len[b] : (int)(p.nb * BS);
+    u.c = p.scale_log2e;
+    const bool masked = u.mask != nullptr || u.valid < (int)(p.nb * BS);
+    const uint32_t q0 = part * 32;
+    if (count <= Unit::SLOTS) {
+        if (count > 0) u.template in_registers<false>(q0 + wave * 8, 0, count, masked, red, wave);
+    } else if (count <= 4 * Unit::SLOTS) {
+        const uint32_t per = (count + 3) / 4, first = wave * per;
+        const uint32_t mine = first >= count ? 0u : (count - first < per ? count - first : per);
+        for (uint32_t unit = 0; unit < 4; ++unit)
+            u.template in_registers<true>(q0 + unit * 8, first < count ? first : 0u, mine, masked, red, wave);
+    } else {
+        u.in_passes(q0 + wave * 8, count);
     }
 }
 
@@ -1493,7 +1745,7 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
     SddParams p = {lut, a, b, c, blocks, head_dim, ctx_blks_a * block_size, ctx_blks_b * block_size,
-                   lut_heads > 1 ? lut_dim : 0};
+                   lut_heads > 1 ? lut_dim : 0, batch_dim, 0};
     const dim3 grid((blocks + kSddGroup - 1) / kSddGroup, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
@@ -1507,7 +1759,12 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
         return launch_status();
     }
     if (block_size == 64 && in_dtype == SFB_BF16) {
-        const dim3 stream_grid((blocks + kSddStreamGroup - 1) / kSddStreamGroup, batch_dim, head_dim);
+        const uint32_t num_bh = batch_dim * head_dim;
+        p.by_xcd = num_bh % 8 == 0 || num_bh >= 32;
+        const uint64_t wgs = (uint64_t)((blocks + kSddStreamGroup - 1) / kSddStreamGroup) *
+                             (p.by_xcd ? bh_groups(num_bh) * 8 : num_bh);
+        if (wgs > 0x7fffffffull) return SFB_ERR_SHAPE;
+        const dim3 stream_grid((uint32_t)wgs);
         if (out_dtype == SFB_BF16) sdd_nt_stream_kernel<__bf16><<<stream_grid, dim3(128), 0, s>>>(p);
         else sdd_nt_stream_kernel<float><<<stream_grid, dim3(128), 0, s>>>(p);
         return launch_status();
@@ -1540,6 +1797,13 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     const dim3 grid((uint32_t)groups);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (block_size == 64 && x_dtype == SFB_BF16) {
+        const uint64_t units = (uint64_t)batch_dim * head_dim * ctx_blks * 2;   // 32 rows each
+        if (units > 0x7fffffffull) return SFB_ERR_SHAPE;
+        if (y_dtype == SFB_BF16) masked_softmax_rows8_kernel<__bf16><<<dim3((uint32_t)units), dim3(256), 0, s>>>(p);
+        else masked_softmax_rows8_kernel<float><<<dim3((uint32_t)units), dim3(256), 0, s>>>(p);
+        return launch_status();
+    }
 #define SFB_CALL(BSV, TX, TY) masked_softmax_kernel<BSV, TX, TY><<<grid, dim3(256), 0, s>>>(p)
     if (block_size == 64) SFB_DISPATCH_2(64, x_dtype, y_dtype, SFB_CALL);
     else if (block_size == 32) SFB_DISPATCH_2(32, x_dtype, y_dtype, SFB_CALL);
