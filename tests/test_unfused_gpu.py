@@ -186,6 +186,48 @@ def test_softmax_every_rows_per_wave_variant(nb, bf16, masked):
     assert (got[want == 0] == 0).all()
 
 
+@pytest.mark.parametrize("out_f32", [False, True])
+def test_bf16_trio_per_head_tables_and_masks(out_f32):
+    """The bf16 kernels for blocks of 64 with one look-up table and one mask per head: a block count that is not a
+    multiple of the sdd's group of blocks, 9 (batch, head) pairs (not a multiple of the 8 XCDs), row lengths from
+    1 to 19 blocks (register slots of the softmax, a row shared by the four waves, product rows that end inside a
+    group of prefetched blocks), key padding, and both storage types for S and P."""
+    bs, nb, B, H, d = 64, 19, 3, 3, 64
+    L = nb * bs
+    rng = np.random.default_rng(5)
+    lays = []
+    for h in range(H):
+        lay = np.tril(np.ones((nb, nb), np.uint32))
+        lays.append(np.roll(lay, h, axis=1) if h else lay)   # same number of blocks, other columns
+    per_head = [sfb.build_luts(l) for l in lays]
+    blocks = per_head[0]["blocks"]
+    assert all(l["blocks"] == blocks for l in per_head) and blocks % 8 != 0
+    nt = np.concatenate([l["nt_lut"] for l in per_head])
+    nn = np.concatenate([l["nn_lut"] for l in per_head])
+    keep = (rng.random((H, blocks, bs, bs)) < 0.8).astype(np.uint8)
+    keep[:, :, :, 0] = 1
+    mask = np.concatenate([sfb.pack_mask(keep[h]) for h in range(H)])
+    mask_rows = np.concatenate([sfb.transpose_mask(sfb.pack_mask(keep[h]), blocks, bs) for h in range(H)])
+    valid = np.array([L, L - 70, L - 5 * bs], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=21, bf16=True)
+    store = sfb.F32 if out_f32 else sfb.BF16
+    S = sfb.bst_sgemm_nt(sfb.to_device(nt), dev(Q, True), dev(K, True), bs, blocks, out_dtype=store, lut_heads=H)
+    want_s = orc.sdd_nt(Q, K, nt, bs, lut_heads=H)
+    assert rel_err(S.float().cpu().numpy(), want_s) <= TOL_BF16
+    s_in = orc.round_bf16(want_s)
+    want_p = orc.masked_softmax(s_in, nn, nb, 0.125, mask=mask, valid_len=valid, lut_heads=H, mask_heads=H)
+    got_p = sfb.BlocksparseMaskedSoftmax(sfb.to_device(nn), sfb.to_device(mask_rows),
+                                         torch.from_numpy(s_in).cuda().to(torch.bfloat16), nb, 0.125, out_dtype=store,
+                                         valid_len=sfb.to_device(valid), lut_heads=H, mask_heads=H)
+    got_p = got_p.float().cpu().numpy()
+    assert rel_err(got_p, want_p) <= TOL_BF16
+    assert (got_p[want_p == 0] == 0).all()
+    p_in = orc.round_bf16(want_p)
+    O = sfb.bst_sgemm_xn(sfb.to_device(nn), torch.from_numpy(p_in).cuda().to(torch.bfloat16), dev(V, True), nb,
+                         lut_heads=H)
+    assert rel_err(O.cpu().numpy(), orc.dsd_nn(p_in, V, nn, lut_heads=H)) <= TOL_BF16
+
+
 def test_error_codes_instead_of_silent_no_op():
     q = torch.zeros((1, 64, 1, 64), device="cuda")
     lut = sfb.to_device(np.zeros((3, 2), np.uint32))
