@@ -461,7 +461,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const size_t bh_bytes = token_offset(w.b, 0, w.h, L, p.heads, D) * 2;
     const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
     const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
-    const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+    const typename T::Sources src = T::sources(lane, row_bytes);
     const uint32_t lds0 = T::lds_address(smem);
     // LUT entries of key blocks [win, win + 64) of this item, one per lane (clamped to the last one)
     uint32_t win = 0;
@@ -475,10 +475,10 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         return __builtin_amdgcn_readlane(entries.y, jj - win);
     };
     auto load_k = [&](uint32_t j, uint32_t buf) {
-        T::load_tile(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+        T::load_tile_all(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes, wave, src, row_bytes);
     };
     auto load_v = [&](uint32_t j, uint32_t buf) {
-        T::load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)column_of(j) * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+        T::load_tile_all(lds0 + (2 + buf) * TILE, v_base + (size_t)column_of(j) * BS * row_bytes, wave, src, row_bytes);
     };
     auto loads_landed = [&]() {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -577,14 +577,16 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         // Every chunk carries the same work: the exponentials of the next chunk, one slice (KS / PU product steps) of
         // the next block's scores and one step of the output product.  The fragments of a chunk are requested from
         // LDS one chunk ahead of the matrix instructions that consume them.
-        constexpr int KPC = KS / PU;   // score product steps per chunk
-        static_assert(KS % PU == 0, "the score product is spread evenly over the chunks");
+        // (chunk u takes steps u*KS/PU .. (u+1)*KS/PU - 1: one each for 64 features and 64 keys, up to two
+        // otherwise)
+        constexpr int KPC = (KS + PU - 1) / PU;   // most score product steps of a chunk
         bf16x8 kfr[PU][KPC][KT], vfr[PU][NO];
         auto fragments = [&](int u) {
 #pragma unroll
             for (int kk = 0; kk < KPC; ++kk)
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt) kfr[u][kk][kt] = T::k_frag(k_read, k_lane, kt, u * KPC + kk);
+                for (int kt = 0; kt < KT; ++kt)
+                    if (u * KS / PU + kk < (u + 1) * KS / PU) kfr[u][kk][kt] = T::k_frag(k_read, k_lane, kt, u * KS / PU + kk);
 #pragma unroll
             for (int mt = 0; mt < NO; ++mt) vfr[u][mt] = T::v_frag(v_read, v_lane, mt, u);
         };
@@ -592,8 +594,8 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         exps(0);
 #pragma unroll
         for (int i = 0; i < T::LOADS; ++i) {
-            T::load_rows(k_dst, k_src, i, wave, src_even, src_odd, row_bytes);
-            T::load_rows(v_dst, v_src, i, wave, src_even, src_odd, row_bytes);
+            T::load_rows_all(k_dst, k_src, i, wave, src, row_bytes);
+            T::load_rows_all(v_dst, v_src, i, wave, src, row_bytes);
         }
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the tile loads are issued here, not later
 #pragma unroll
@@ -606,7 +608,8 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
             for (int kk = 0; kk < KPC; ++kk)
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) {
-                    const int ks = u * KPC + kk;
+                    const int ks = u * KS / PU + kk;
+                    if (ks >= (u + 1) * KS / PU) continue;
                     if (ks == 0) {
                         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
                         s_next[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[u][kk][kt], qf[ks], SLIM ? off_vec : zero, 0, 0, 0);
@@ -620,8 +623,8 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
             for (int mt = 0; mt < NO; ++mt)
                 o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[u][mt], bfrag, o_acc[mt], 0, 0, 0);
         }
-        if constexpr (SLIM) {
-            schedule_chunks<BS, D>();
+        if constexpr (SLIM && D == 64) {
+            schedule_chunks<BS, D>();   // issue order worked out for this head size
         }
         st.l += sum0 + sum1;
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the wait for the tiles comes last
@@ -644,7 +647,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
 }
 
 template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void fused_attention_bf16_kernel(FusedParams p) {
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_bf16_kernel(FusedParams p) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int TILE = T::TILE_BYTES;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
@@ -1222,6 +1225,39 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_stream_bf16_kernel(
 }
 
 // Other element types and head sizes: the work-group does the items of its stream one after the other.
+// bf16 tensors with a head size other than 64: the stream's items one after the other (the chained form above is
+// built around one score product step per chunk, which is what 64 features give).
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream_items_bf16_kernel(FusedParams p) {
+    using T = Bf16DirectTiles<BS, D>;
+    constexpr int TILE = T::TILE_BYTES;
+    __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * TILE];   // K0 K1 V0 V1
+    __shared__ uint32_t retry_flag;
+    static_assert(4 * TILE >= BS * (D * 4 + 16), "the tiles' memory doubles as the output slabs");
+    const const_words slot = (const_words)(uintptr_t)p.st_slots + (size_t)blockIdx.x * (sizeof(sfb_stream_slot) / 4);
+    const uint32_t item_begin = slot[2], n_items = slot[3], merge_begin = slot[4], n_merges = slot[5];
+    const const_words items = (const_words)(uintptr_t)p.st_items + (size_t)item_begin * (sizeof(sfb_stream_item) / 4);
+    const uint32_t t = threadIdx.x, lane = t & 63;
+    for (uint32_t i = 0; i < n_items; ++i) {
+        const StreamItem it = stream_item(items, i, n_items);
+        const RowWork w = stream_row_work(p, items, i);
+        const sfb_uint2 window = lut_window(p, w, 0, lane);
+        uint32_t made = 0;
+        auto finish = [&](f32x16 (&o)[D / 32], const RowState& rs) {
+            made = stream_end_item<BS, D>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
+        };
+        bool done = false;
+        if constexpr (!MASKED) done = attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window, finish);
+        if (!done) attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window, finish);
+        if (made != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();   // the record is complete, and the tiles' memory is free for the next item
+        if (made != 0 && t == 0) stream_set_flag(p, made);
+    }
+    if (n_merges != 0)
+        stream_merges<BS, D>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4), n_merges,
+                             smem);
+}
+
 template <int BS, int D>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream_f32_kernel(FusedParams p) {
     using T = F32Tiles<BS, D>;
@@ -1264,7 +1300,10 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
             else if (streamed) fused_attention_stream_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
             else fused_attention_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
         } else {
-            return SFB_ERR_HEAD_STATE;   // the bf16 kernel is built for head size 64 only
+            if (masked && streamed) fused_attention_stream_items_bf16_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+            else if (masked) fused_attention_bf16_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+            else if (streamed) fused_attention_stream_items_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
+            else fused_attention_bf16_kernel<BS, D, false><<<g, b, 0, stream>>>(p);
         }
     } else if (streamed)
         fused_attention_stream_f32_kernel<BS, D><<<g, b, 0, stream>>>(p);
@@ -1273,7 +1312,7 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
     return launch_status();
 }
 
-// head sizes: 64 for both input types; 32, 96 and 128 for fp32 inputs
+// head sizes 32, 64, 96 and 128 for both input types
 template <int BS>
 static int launch_fused_any(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks, uint32_t state_dim) {
     switch (state_dim) {
@@ -1292,8 +1331,7 @@ static int check_common(const void* q, const void* k, const void* v, const void*
     if (!q || !k || !v || !o || !nn_lut) return SFB_ERR_NULL_POINTER;
     if (in_dtype != SFB_F32 && in_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64 && (in_dtype != SFB_F32 || (state_dim != 32 && state_dim != 96 && state_dim != 128)))
-        return SFB_ERR_HEAD_STATE;
+    if (state_dim != 32 && state_dim != 64 && state_dim != 96 && state_dim != 128) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (batch_dim == 0 || ctx_blks == 0 || head_dim == 0 || lut_heads == 0 || mask_heads == 0)
         return SFB_ERR_SHAPE;

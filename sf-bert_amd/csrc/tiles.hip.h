@@ -34,11 +34,18 @@ namespace sfb {
 // No registers are spent on staging and no ds_write / v_perm instructions are needed.
 template <int BS, int D>
 struct Bf16DirectTiles {
-    // the layout below is for D = 64 (128-byte rows); the loaders and fragment readers assert it, so that merely
-    // naming the type for another head size (in a branch that is not taken) stays legal
+    // Head sizes other than 64 are cut into slices of 64 features, each slice a tile of 128-byte rows in the layout
+    // above (slice f of a K or V tile starts 128*f bytes into the tensor's rows and BS*128*f bytes into the LDS
+    // tile).  A last slice of 32 features (head sizes 32 and 96) fills only the first four chunks of its rows: its
+    // lanes fetch chunk (c ^ swz) & 3 instead of c ^ swz, so that nothing beyond the row is read, and the fragment
+    // readers, which only ever ask for chunks 0..3 of such a slice, find them where they expect them.
     static constexpr int NW = BS / 32;                 // waves per work-group
-    static constexpr int TILE_BYTES = BS * D * 2;
+    static constexpr int SLICES = (D + 63) / 64;
+    static constexpr bool PARTIAL = D % 64 != 0;       // the last slice has 32 features
+    static constexpr int SLICE_BYTES = BS * 128;
+    static constexpr int TILE_BYTES = SLICES * SLICE_BYTES;
     static constexpr int GROUPS = BS / 8;              // 8-row groups (one load instruction each)
+    static_assert(D % 32 == 0 && D >= 32 && D <= 128, "head sizes 32, 64, 96, 128");
 
     typedef uint32_t __attribute__((address_space(3)))* lds_u32_ptr;
     // LDS byte address of a pointer into a __shared__ array
@@ -55,6 +62,23 @@ struct Bf16DirectTiles {
         const uint32_t rr = lane >> 3, pos = lane & 7u;
         return rr * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
     }
+    // The same for a last slice of 32 features.
+    static __device__ __forceinline__ uint32_t lane_source_part(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
+        const uint32_t rr = lane >> 3, pos = lane & 7u;
+        return rr * row_bytes + (((pos ^ swz(8u * odd + rr)) & 3u) << 4);
+    }
+    // The four lane offsets a work-group needs to fetch whole tiles.
+    struct Sources {
+        uint32_t even, odd, even_part, odd_part;
+    };
+    static __device__ __forceinline__ Sources sources(uint32_t lane, uint32_t row_bytes) {
+        Sources s;
+        s.even = lane_source(lane, 0, row_bytes);
+        s.odd = lane_source(lane, 1, row_bytes);
+        s.even_part = PARTIAL ? lane_source_part(lane, 0, row_bytes) : s.even;
+        s.odd_part = PARTIAL ? lane_source_part(lane, 1, row_bytes) : s.odd;
+        return s;
+    }
     // The same for a tile whose LDS rows hold the source rows in the order that makes the 8 k-slots of a lane
     // in the second product, rows 16u + 8(j/4) + 4*half + j%4 of the tile, the 8 consecutive source rows
     // 32*half + 8u + j: LDS row 16u + 8a + 4h + c holds source row 32h + 8u + 4a + c, which is 4n + 32(rr/4) + rr%4
@@ -70,7 +94,6 @@ struct Bf16DirectTiles {
     template <int GROUP_ROWS = 8>
     static __device__ __forceinline__ void load_rows(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
-        static_assert(D == 64, "128-byte rows");
         const uint32_t n = (uint32_t)(NW * i) + wave;   // 8-row group
         uint32_t src;
         if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
@@ -92,6 +115,21 @@ struct Bf16DirectTiles {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) load_rows(lds_tile, g_tile, i, wave, src_even, src_odd, row_bytes);
     }
+    // Load number i of this wave's share of every slice of a tile.
+    static __device__ __forceinline__ void load_rows_all(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
+                                                         const Sources& src, uint32_t row_bytes) {
+#pragma unroll
+        for (int f = 0; f < SLICES; ++f) {
+            const bool part = PARTIAL && f == SLICES - 1;
+            load_rows(lds_tile + f * SLICE_BYTES, g_tile + f * 128, i, wave, part ? src.even_part : src.even,
+                      part ? src.odd_part : src.odd, row_bytes);
+        }
+    }
+    static __device__ __forceinline__ void load_tile_all(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
+                                                         const Sources& src, uint32_t row_bytes) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) load_rows_all(lds_tile, g_tile, i, wave, src, row_bytes);
+    }
     // with src_even / src_odd from lane_source_by_halves()
     static __device__ __forceinline__ void load_tile_by_halves(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
                                                                uint32_t src_even, uint32_t src_odd,
@@ -105,7 +143,7 @@ struct Bf16DirectTiles {
         return qn * 128u + ((half ^ swz(qn)) << 4);
     }
     static __device__ __forceinline__ bf16x8 k_frag(const uint8_t* k_lds, uint32_t lane_base, int kt, int ks) {
-        return *(const bf16x8*)(k_lds + kt * 4096 + (lane_base ^ (uint32_t)(ks * 32)));
+        return *(const bf16x8*)(k_lds + (ks / 4) * SLICE_BYTES + kt * 4096 + (lane_base ^ (uint32_t)((ks % 4) * 32)));
     }
     // Per-lane byte offset of the transposing read for (column tile 0, first 4-key group of product step
     // 0); column tile mt and second group x are at (base ^ (mt*64 + x*32)) + x*1024, step u 2048 bytes on.
@@ -117,8 +155,9 @@ struct Bf16DirectTiles {
     static __device__ __forceinline__ bf16x8 v_frag(const uint8_t* v_lds, uint32_t lane_base, int mt, int u) {
         typedef short s16x4 __attribute__((ext_vector_type(4)));
         typedef s16x4 __attribute__((address_space(3)))* lds_ptr;
-        const uint8_t* a0 = v_lds + u * 2048 + (lane_base ^ (uint32_t)(mt * 64));
-        const uint8_t* a1 = v_lds + u * 2048 + 1024 + (lane_base ^ (uint32_t)(mt * 64 + 32));
+        const uint8_t* slice = v_lds + (mt / 2) * SLICE_BYTES;
+        const uint8_t* a0 = slice + u * 2048 + (lane_base ^ (uint32_t)((mt % 2) * 64));
+        const uint8_t* a1 = slice + u * 2048 + 1024 + (lane_base ^ (uint32_t)((mt % 2) * 64 + 32));
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a0);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a1);
         const u32x4 r = {__builtin_bit_cast(u32x2, lo).x, __builtin_bit_cast(u32x2, lo).y,

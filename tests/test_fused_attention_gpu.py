@@ -194,35 +194,46 @@ def test_rows_longer_than_64_key_blocks(bf16, scheduled):
     check(got, orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS), TOL_BF16 if bf16 else TOL_F32)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("d", [32, 96, 128])
 @pytest.mark.parametrize("bs", [32, 64])
-def test_head_sizes_other_than_64_fp32(d, bs):
-    """fp32 tensors with head size 32, 96 or 128 (the reference's K64 = false paths): fused kernel, plain and
-    scheduled with split rows, masked and padded."""
+def test_head_sizes_other_than_64(d, bs, bf16):
+    """Head size 32, 96 or 128 (the reference's K64 = false paths), fp32 and bf16 tensors: fused kernel, plain,
+    scheduled with split rows and streamed, masked and padded."""
     nb, B, H = 16, 2, 3
+    tol = TOL_BF16 if bf16 else TOL_F32
     luts = sfb.build_luts(PATTERNS["bigbird"](nb))
     keep = (np.random.default_rng(d).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
     mask = sfb.pack_mask(keep)
     valid = np.array([nb * bs, nb * bs - bs - 5], np.int32)
-    Q, K, V = qkv(B, nb * bs, H, d, seed=d + bs)
+    Q, K, V = qkv(B, nb * bs, H, d, seed=d + bs, bf16=bf16)
     scale = float(1.0 / np.sqrt(d))
     want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, mask=mask, valid_len=valid, nthreads=THREADS)
-    check(run_fused(Q, K, V, luts, bs, scale, mask=mask, valid_len=valid), want, TOL_F32)
-    check(run_fused(Q, K, V, luts, bs, scale, mask=mask, valid_len=valid, max_blocks=3), want, TOL_F32)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid), want, tol)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid, max_blocks=3), want, tol)
     plain = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, nthreads=THREADS)
-    check(run_fused(Q, K, V, luts, bs, scale), plain, TOL_F32)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16), plain, tol)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, max_blocks=3), plain, tol)
+    # streamed launches: rows cut into chunks, merged from partial records
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=64)
+    assert stream["plan"].n_parts > 0
+    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    q, k, v = (dev(x, bf16) for x in (Q, K, V))
+    nn, blob = sfb.to_device(luts["nn_lut"]), sfb.to_device(stream["blob"])
+    for m, vl, ref in ((None, None, plain), (sfb.to_device(mask), sfb.to_device(valid), want)):
+        out = sfb.fused_attention_streamed(q, k, v, nn, blob, stream, ws, bs, luts["blocks"], scale, mask=m, valid_len=vl)
+        torch.cuda.synchronize()
+        assert sfb.stream_status(stream, d, ws) == 0
+        check(out.cpu().numpy(), ref, tol)
 
 
 def test_head_size_errors():
-    q = torch.zeros((1, 64, 1, 128), device="cuda", dtype=torch.bfloat16)
     luts = sfb.build_luts(PATTERNS["full"](1))
-    with pytest.raises(sfb.SfbError) as e:   # bf16 tensors come with head size 64 only
-        sfb.fused_attention(q, q, q, sfb.to_device(luts["nn_lut"]), 64, 1, 0.125)
-    assert e.value.status == 3
-    q = torch.zeros((1, 64, 1, 80), device="cuda")
-    with pytest.raises(sfb.SfbError) as e:
-        sfb.fused_attention(q, q, q, sfb.to_device(luts["nn_lut"]), 64, 1, 0.125)
-    assert e.value.status == 3
+    for dtype in (torch.bfloat16, torch.float32):   # head sizes are 32, 64, 96 and 128
+        q = torch.zeros((1, 64, 1, 80), device="cuda", dtype=dtype)
+        with pytest.raises(sfb.SfbError) as e:
+            sfb.fused_attention(q, q, q, sfb.to_device(luts["nn_lut"]), 64, 1, 0.125)
+        assert e.value.status == 3
 
 
 @pytest.mark.parametrize("bf16_in", [False, True])
