@@ -309,8 +309,10 @@ int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const voi
  * scale, dK = dS^T Q, dQ = dS K, where delta = rowsum(dO * O) (computed here into the caller's buffer) stands for
  * the gradient's sum over the sparse row.  q, k, v, d_out [dev] bf16 [batch, ctx, heads, 64]; o [dev] fp32, the
  * forward output; lse [dev] from sfb_fused_attention_scheduled_lse; delta [dev] fp32 [batch][heads][ctx]
- * (scratch, overwritten); dq, dk, dv [dev] fp32; nn_lut, tn_lut [dev] (one layout for all heads); mask
- * block-major.  row_items / col_items [dev] (may be NULL: one work-group per block-row / block-column in index
+ * (scratch, overwritten); dq, dk, dv [dev] fp32; nn_lut, tn_lut [dev]: one layout for all heads (lut_heads 1), or
+ * one table per head, lut_dim = ctx_blks + blocks entries apart, every head with the same number of blocks
+ * (lut_heads = head_dim; then without work items: every line is done whole); mask block-major, one for all
+ * heads or one per head (mask_heads).  row_items / col_items [dev] (may be NULL: one work-group per block-row / block-column in index
  * order): work items of sfb_build_schedule over nn_lut / over tn_lut, longest first, with lines of more than
  * max_blocks blocks cut into chunks; the chunks of a split line write partial records into workspace ([dev],
  * 256-byte aligned, sfb_backward_workspace_bytes() bytes; n_*_parts as returned by sfb_build_schedule) and a
@@ -325,8 +327,8 @@ int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, const void*
                                  uint32_t n_row_heavy, uint32_t n_row_parts, const sfb_work_item* col_items,
                                  uint32_t n_col_items, uint32_t n_col_heavy, uint32_t n_col_parts, void* workspace,
                                  size_t workspace_bytes, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
-                                 uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
-                                 float scale);
+                                 uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
+                                 uint32_t lut_dim, uint32_t mask_heads, float scale);
 
 
 /* ---- the unfused trio (kept as the no_fusion comparison) ------------------------------------ */

@@ -346,11 +346,13 @@ def fused_attention_forward_lse(q, k, v, nn_lut, items, sched, workspace, block_
 
 
 def fused_attention_backward(q, k, v, o, d_out, lse, nn_lut, tn_lut, block_size, blocks, scale, mask=None,
-                             valid_len=None, mask_heads=1, row_sched=None, col_sched=None, workspace=None):
+                             valid_len=None, mask_heads=1, row_sched=None, col_sched=None, workspace=None,
+                             lut_heads=1):
     """(dq, dk, dv) fp32 from bf16 q, k, v, d_out, the forward output o and lse, in two kernels
     (sfb_fused_attention_backward); nothing sparse goes through memory.  row_sched / col_sched: build_schedule()
     over the NN / TN look-up table with its "items" already on the device under "items_dev" (None: one
-    work-group per block-row / block-column)."""
+    work-group per block-row / block-column).  lut_heads = H: nn_lut / tn_lut hold one table per head (then without
+    schedules)."""
     import torch
     B, L, H, d = q.shape
     dq, dk, dv = (torch.empty((B, L, H, d), dtype=torch.float32, device=q.device) for _ in range(3))
@@ -370,8 +372,9 @@ def fused_attention_backward(q, k, v, o, d_out, lse, nn_lut, tn_lut, block_size,
         C.c_uint32(rs.get("n_parts", 0)), _dev(cs.get("items_dev")), C.c_uint32(cs.get("n_items", 0)),
         C.c_uint32(cs.get("n_heavy", 0)), C.c_uint32(cs.get("n_parts", 0)), _dev(workspace),
         C.c_size_t(workspace.numel() if workspace is not None else 0), C.c_uint32(block_size), C.c_uint32(blocks),
-        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(mask_heads),
-        C.c_float(scale)), "sfb_fused_attention_backward")
+        C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H), C.c_uint32(d), C.c_uint32(lut_heads),
+        C.c_uint32(L // block_size + blocks), C.c_uint32(mask_heads), C.c_float(scale)),
+        "sfb_fused_attention_backward")
     return dq, dk, dv
 
 

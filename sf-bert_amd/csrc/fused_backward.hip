@@ -37,6 +37,7 @@ struct BackwardParams {
     float* partials;            // partial results of split rows / columns, or nullptr
     uint32_t ranks, heavy, n_parts;
     uint32_t batch, heads, nb, blocks, mask_stride;
+    uint32_t lut_stride;        // entries between the tables of consecutive heads, 0: one table for all
     float scale, scale_log2e;
 };
 
@@ -60,9 +61,10 @@ __device__ __forceinline__ LineWork decode_line_work(const BackwardParams& p, co
         w.count = it.count;
         if (it.nchunks > 1) w.slot = (int32_t)(it.part + it.chunk);
     } else {
+        const sfb_uint2* mine = lut + (size_t)(id.valid ? id.bh % p.heads : 0u) * p.lut_stride;
         w.line = id.rank;
-        w.first = lut[id.valid ? id.rank : 0u].x;
-        w.count = id.valid ? lut[id.rank].y : 0u;
+        w.first = mine[id.valid ? id.rank : 0u].x;
+        w.count = id.valid ? mine[id.rank].y : 0u;
     }
     return w;
 }
@@ -165,12 +167,13 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
             T::load_tile(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
             T::load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
         };
-        sfb_uint2 e = uniform(p.nn_lut[off]);
+        const sfb_uint2* const nn_lut = p.nn_lut + (size_t)h * p.lut_stride;
+        sfb_uint2 e = uniform(nn_lut[off]);
         fetch(e, 0);
         for (uint32_t j = 0; j < count; ++j) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();   // tiles of block j have landed for every wave; every wave is done with block j-1
-            const sfb_uint2 e_next = uniform(p.nn_lut[off + (j + 1 < count ? j + 1 : j)]);
+            const sfb_uint2 e_next = uniform(nn_lut[off + (j + 1 < count ? j + 1 : j)]);
             fetch(e_next, (j + 1) & 1);
             const uint8_t* k_tile = smem + (j & 1) * TILE;
             const uint8_t* v_tile = smem + (2 + (j & 1)) * TILE;
@@ -274,12 +277,13 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
             T::load_tile(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
             T::load_tile(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
         };
-        sfb_uint2 e = uniform(p.tn_lut[off]);
+        const sfb_uint2* const tn_lut = p.tn_lut + (size_t)h * p.lut_stride;
+        sfb_uint2 e = uniform(tn_lut[off]);
         fetch(e, 0);
         for (uint32_t j = 0; j < count; ++j) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            const sfb_uint2 e_next = uniform(p.tn_lut[off + (j + 1 < count ? j + 1 : j)]);
+            const sfb_uint2 e_next = uniform(tn_lut[off + (j + 1 < count ? j + 1 : j)]);
             fetch(e_next, (j + 1) & 1);
             const uint8_t* q_tile = smem + (j & 1) * TILE;
             const uint8_t* do_tile = smem + (2 + (j & 1)) * TILE;
@@ -447,7 +451,8 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
                                             uint32_t n_col_heavy, uint32_t n_col_parts, void* workspace,
                                             size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
                                             uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
-                                            uint32_t state_dim, uint32_t mask_heads, float scale) {
+                                            uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim,
+                                            uint32_t mask_heads, float scale) {
     using namespace sfb;
     if (!q || !k || !v || !o || !d_out || !lse || !delta || !dq || !dk || !dv || !nn_lut || !tn_lut)
         return SFB_ERR_NULL_POINTER;
@@ -455,8 +460,11 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (state_dim != 64) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
-    if (!batch_dim || !ctx_blks || !head_dim || !mask_heads) return SFB_ERR_SHAPE;
+    if (!batch_dim || !ctx_blks || !head_dim || !mask_heads || !lut_heads) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
+    if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks + blocks)) return SFB_ERR_SHAPE;
+    // work items describe one layout: with a table per head every line is done whole by one work-group
+    if (lut_heads > 1 && (row_items || col_items)) return SFB_ERR_SHAPE;
     if ((row_items && (!n_row_items || n_row_heavy >= n_row_items)) ||
         (col_items && (!n_col_items || n_col_heavy >= n_col_items)))
         return SFB_ERR_SHAPE;
@@ -477,6 +485,7 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     p.nn_lut = nn_lut; p.tn_lut = tn_lut; p.mask = mask; p.valid_len = valid_len;
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
+    p.lut_stride = lut_heads > 1 ? lut_dim : 0;
     p.scale = scale; p.scale_log2e = scale * kLog2e;
     float* row_partials = (float*)workspace;
     float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * state_dim;

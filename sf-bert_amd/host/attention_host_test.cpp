@@ -237,7 +237,8 @@ int main() {
                                                     (const sfb_uint2*)d_nn, (const sfb_uint2*)d_tn, d_mask_np, nullptr,
                                                     rows.dev, rows.n, rows.heavy, rows.parts, cols.dev, cols.n,
                                                     cols.heavy, cols.parts, bwd_ws, bwd_bytes + 256, blk_size_, blocks,
-                                                    batch_dim, ctx_blks, heads_, head_state_, 1, scale);
+                                                    batch_dim, ctx_blks, heads_, head_state_, 1, ctx_blks + blocks, 1,
+                                                    scale);
         if (rc != SFB_OK) {
             std::fprintf(stderr, "fused training pair failed: %s\n", sfb_status_string(rc));
             return 1;

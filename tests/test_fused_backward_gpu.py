@@ -88,6 +88,56 @@ def test_fused_backward_matches_oracle(pattern, masked, bs):
         assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize("bs", [32, 64])
+def test_fused_backward_per_head_tables_and_masks(bs):
+    """One look-up table and one element mask per head (the reference's `fixed` pattern): forward with its
+    log-sum-exp through the streamed entry point, backward with every line done whole; the oracle head by head."""
+    nb, B, H, d = 8, 2, 4, 64
+    L = nb * bs
+    lays = sfb.layout_fixed(H, nb, 4, causal=True)
+    per_head = [sfb.build_luts(lays[h]) for h in range(H)]
+    blocks = per_head[0]["blocks"]
+    assert all(l["blocks"] == blocks for l in per_head)
+    assert any((per_head[0]["nn_lut"] != per_head[h]["nn_lut"]).any() for h in range(1, H))
+    nn = np.concatenate([l["nn_lut"] for l in per_head])
+    tn = np.concatenate([l["tn_lut"] for l in per_head])
+    rng = np.random.default_rng(bs)
+    masks = []
+    for h in range(H):
+        keep = (rng.random((blocks, bs, bs)) < 0.8).astype(np.uint8)
+        keep[:, np.arange(bs), np.arange(bs)] = 1
+        masks.append(sfb.pack_mask(keep))
+    mask = np.concatenate(masks)
+    valid = np.array([L, L - bs - 7], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=300 + bs, bf16=True)
+    dO = orc.round_bf16(orc.fill_normal((B, L, H, d), 310))
+    q, k, v, do = (dev(x, True) for x in (Q, K, V, dO))
+    m, vl = sfb.to_device(mask), sfb.to_device(valid)
+    stream = sfb.build_stream(nn, nb, B, H, bs, lut_heads=H)
+    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    o = torch.empty((B, L, H, d), device="cuda")
+    lse = torch.empty((B, H, L), device="cuda")
+    sfb.fused_attention_streamed(q, k, v, sfb.to_device(nn), sfb.to_device(stream["blob"]), stream, ws, bs, blocks,
+                                 0.125, mask=m, valid_len=vl, mask_heads=H, out=o, lse=lse)
+    dq, dk, dv = sfb.fused_attention_backward(q, k, v, o, do, lse, sfb.to_device(nn), sfb.to_device(tn), bs, blocks,
+                                              0.125, mask=m, valid_len=vl, mask_heads=H, lut_heads=H)
+    torch.cuda.synchronize()
+    assert sfb.stream_status(stream, d, ws) == 0
+    for h in range(H):
+        one = lambda x: np.ascontiguousarray(x[:, :, h:h + 1])
+        dQ, dK, dV, _ = orc.attention_backward(one(Q), one(K), one(V), one(dO), per_head[h], bs, 0.125, mask=masks[h],
+                                               valid_len=valid)
+        for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+            assert rel_err(got[:, :, h:h + 1].cpu().numpy(), want) <= TOL_BF16, (name, h)
+    # work items describe one layout only
+    rs = sfb.build_schedule(per_head[0]["nn_lut"], nb, 3)
+    rs["items_dev"] = sfb.to_device(rs["items"])
+    with pytest.raises(sfb.SfbError) as e:
+        sfb.fused_attention_backward(q, k, v, o, do, lse, sfb.to_device(nn), sfb.to_device(tn), bs, blocks, 0.125,
+                                     row_sched=rs, lut_heads=H)
+    assert e.value.status == 4
+
+
 def test_fused_backward_rejects_fp32():
     q = torch.zeros((1, 64, 1, 64), device="cuda")
     lut = sfb.to_device(np.zeros((2, 2), np.uint32))
