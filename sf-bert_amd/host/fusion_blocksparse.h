@@ -14,7 +14,7 @@
 
 namespace sfb_host {
 template <typename T>
-inline bool fused_sdd_softmax(CUstream stream, const uint2* nn_lut, const float* a, const float* b, const uint* Mask,
+inline bool fused_sdd_softmax(CUstream stream, const uint2* nn_lut, const float* a, const float* b, const void* Mask,
                               T* Y, uint block_size, uint blocks, uint batch_dim, uint ctx_blks_a, uint head_dim,
                               uint state_dim, uint lut_heads, uint lut_dim, uint mask_heads, float scale) {
     // the reference passes the NT LUT length as lut_dim and derives the NN stride itself (:434)
@@ -35,10 +35,12 @@ bool fusion_attention1(CUstream stream, const uint2* nt_lut, const float* a, con
                                           head_dim, state_dim, lut_heads, lut_dim, mask_heads, scale);
 }
 
-#define SFB_FUSION_VARIANT(NAME)                                                                                  \
+// MASK: the reference's mask word of the variant (one word per query row and block: uint up to 32 x 32 blocks,
+// uint64 for fusion_attention2_64, fusion_blocksparse.h:2465)
+#define SFB_FUSION_VARIANT(NAME, MASK)                                                                            \
     template <typename T, typename V>                                                                             \
     bool NAME(CUstream stream, const uint2* nt_lut, const float* a, const float* b, bhalf* c, const uint2* nn_lut, \
-              int* rblk_flag, int* rblk_flag1, const uint* Mask, float* Max, float* Sum, T* Y, uint block_size,    \
+              int* rblk_flag, int* rblk_flag1, const MASK* Mask, float* Max, float* Sum, T* Y, uint block_size,    \
               uint blocks, uint batch_dim, uint ctx_blks_a, uint ctx_blks_b, uint head_dim, uint state_dim,        \
               uint lut_heads, uint lut_dim, uint mask_heads, float scale) {                                        \
         (void)nt_lut; (void)c; (void)rblk_flag; (void)rblk_flag1; (void)Max; (void)Sum; (void)ctx_blks_b;          \
@@ -46,10 +48,10 @@ bool fusion_attention1(CUstream stream, const uint2* nt_lut, const float* a, con
                                               ctx_blks_a, head_dim, state_dim, lut_heads, lut_dim, mask_heads,     \
                                               scale);                                                              \
     }
-SFB_FUSION_VARIANT(fusion_attention2)
-SFB_FUSION_VARIANT(fusion_attention_full)
-SFB_FUSION_VARIANT(fusion_attention_local)
-SFB_FUSION_VARIANT(fusion_attention2_64)
+SFB_FUSION_VARIANT(fusion_attention2, uint)
+SFB_FUSION_VARIANT(fusion_attention_full, uint)
+SFB_FUSION_VARIANT(fusion_attention_local, uint)
+SFB_FUSION_VARIANT(fusion_attention2_64, uint64)
 #undef SFB_FUSION_VARIANT
 
 // Full fusion (fusion_blocksparse.h:2990-3007): O (f) = softmax(scale * a b^T, masked) e.
