@@ -1150,10 +1150,12 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_tn_kernel(DsdParams p) {
     constexpr int LDS_BYTES = kFast ? 4 * TILE : BS * X_STRIDE * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c);
+    // block-columns from both ends of the context inwards, the last and the first one of every head before anything
+    // else (the columns of global tokens are the long ones; see dsd_nn_kernel)
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c, p.nb_c >= 2 ? 2 : 0);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
-    const uint32_t col = work.rank;
+    const uint32_t col = (work.rank & 1u) ? work.rank / 2 : p.nb_c - 1 - work.rank / 2;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t kn = lane & 31, half = lane >> 5;
     const uint32_t key_in_block = wave * 32 + kn;
