@@ -1267,7 +1267,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr bool kBf16 = sizeof(TV) == 2;
     using TD = Bf16DirectTiles<BS, D>;
     using TF = F32Tiles<BS, D>;
-    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 3 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
+    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
     // Block-rows are taken from both ends of the context inwards, the last and the first one of every head before
@@ -1299,8 +1299,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         // them (LDS would bound the work-groups per CU, and with them the bytes in flight).  For that a lane's 8
         // k-slots of a product step must be 8 consecutive keys (one 16-byte load): the V tile is laid into LDS
         // with its key rows in the matching order (lane_source_by_halves).  V tiles (L2 hits mostly) go through a
-        // ring of three LDS buffers, two blocks ahead.  Loads and stores complete in issue order, which the
-        // counted waits below rely on.
+        // ring of four LDS buffers, two blocks per barrier.  Loads complete in issue order, which the counted
+        // waits below rely on.
         constexpr int PU = BS / 16, TILE = TD::TILE_BYTES, kDepth = 4;
         const uint32_t row_bytes = row_stride * 2;
         const uint32_t v_even = TD::lane_source_by_halves(lane, 0, row_bytes);
@@ -1337,11 +1337,13 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
             TD::load_tile_by_halves(lds0 + buf * TILE, v_base + (size_t)col * BS * row_bytes, wave, v_even, v_odd,
                                     row_bytes);
         };
-        // Issue order: V(0) V(1) P(0) .. P(kDepth-1), then per block j: V(j+2), [product], P(j+kDepth).  Every
-        // fetch is issued whether or not its block exists (past the row's end the last block is fetched again, a
-        // cache hit, into a buffer or registers that nobody reads): the number of loads between a tile and its use
-        // is then the same in every iteration, which is what a counted wait needs.  V(j) is followed by V(j+1)
-        // and two P tiles (more for j < 2), 4 loads per wave each.
+        // Issue order: V(0) V(1) P(0) .. P(kDepth-1), then per pair of blocks j, j+1: V(j+2) V(j+3), [products],
+        // P(j+kDepth) P(j+kDepth+1).  Every fetch is issued whether or not its block exists (past the row's end
+        // the last block is fetched again, a cache hit, into a buffer or registers that nobody reads, and the
+        // step multiplies by zeros): the number of loads between a tile and its use is then the same in every
+        // step, which is what a counted wait needs -- an exit or a branch inside the unrolled group would leave
+        // the compiler with paths on which the counts, or the registers, differ.  V(j+1) is followed by two P
+        // tiles (more in the first step), 4 loads per wave each; P(j), P(j+1) were issued before V(j).
         if (count > 0) {
             const uint32_t last = count - 1;
             fetch_v(0, 0);
@@ -1350,35 +1352,38 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
             for (int d = 0; d < kDepth; ++d) fetch_p(pr[d], (uint32_t)d < count ? d : last, (uint32_t)d < count);
             for (uint32_t j0 = 0; j0 < count; j0 += kDepth) {
 #pragma unroll
-                for (int d = 0; d < kDepth; ++d) {
+                for (int d = 0; d < kDepth; d += 2) {
                     const uint32_t j = j0 + d;
-                    // V(j) and, issued before it, P(j) have landed when only the 12 loads issued after V(j) remain
-                    asm volatile("s_waitcnt vmcnt(12)"
-                                 : "+v"(pr[d][0]), "+v"(pr[d][1]), "+v"(pr[d][2]), "+v"(pr[d][3])
+                    asm volatile("s_waitcnt vmcnt(8)"
+                                 : "+v"(pr[d][0]), "+v"(pr[d][1]), "+v"(pr[d][2]), "+v"(pr[d][3]), "+v"(pr[d + 1][0]),
+                                   "+v"(pr[d + 1][1]), "+v"(pr[d + 1][2]), "+v"(pr[d + 1][3])
                                  :
                                  : "memory");
-                    __syncthreads();   // V(j) is in LDS for every wave, and every wave is done with V(j-1)
-                    fetch_v(j + 2 < count ? j + 2 : last, (j + 2) % 3u);
-                    const uint8_t* v_read = smem + (j % 3u) * TILE;
-                    // the row is walked in whole groups of kDepth blocks: a step past its end multiplies by zeros
-                    // and keeps the sequence of loads and barriers (an exit or a branch in the middle of the group
-                    // would leave the compiler with paths on which the load counts, or the registers, differ)
-                    const uint32_t live = j < count ? 0xffffffffu : 0u;
+                    __syncthreads();   // V(j), V(j+1) are in LDS for every wave; every wave is done with V(j-2), V(j-1)
+                    fetch_v(j + 2 < count ? j + 2 : last, (j + 2) % 4u);
+                    fetch_v(j + 3 < count ? j + 3 : last, (j + 3) % 4u);
 #pragma unroll
-                    for (int u = 0; u < PU; ++u) {
-                        const u32x4 pv = {pr[d][u].x & live, pr[d][u].y & live, pr[d][u].z & live, pr[d][u].w & live};
-                        const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pv);
+                    for (int e = 0; e < 2; ++e) {
+                        const uint8_t* v_read = smem + ((j + e) % 4u) * TILE;
+                        const uint32_t live = j + e < count ? 0xffffffffu : 0u;
 #pragma unroll
-                        for (int mt = 0; mt < NO; ++mt)
-                            o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u),
-                                                                                bfrag, o_acc[mt], 0, 0, 0);
+                        for (int u = 0; u < PU; ++u) {
+                            const u32x4 pv = {pr[d + e][u].x & live, pr[d + e][u].y & live, pr[d + e][u].z & live,
+                                              pr[d + e][u].w & live};
+                            const bf16x8 bfrag = __builtin_bit_cast(bf16x8, pv);
+#pragma unroll
+                            for (int mt = 0; mt < NO; ++mt)
+                                o_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::v_frag(v_read, v_lane, mt, u),
+                                                                                    bfrag, o_acc[mt], 0, 0, 0);
+                        }
                     }
-                    // the registers of P(j) take P(j + kDepth): not before the product has read them
+                    // the registers of P(j), P(j+1) take the next tiles: not before the products have read them
                     __builtin_amdgcn_sched_barrier(0);
                     fetch_p(pr[d], j + kDepth < count ? j + kDepth : last, j + kDepth < count);
+                    fetch_p(pr[d + 1], j + kDepth + 1 < count ? j + kDepth + 1 : last, j + kDepth + 1 < count);
                 }
             }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing in flight towards LDS when the group ends
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
     } else if constexpr (kBf16) {
         // V tiles double-buffered in LDS by LDS-direct loads, V^T fragments by transposing reads (see
