@@ -1500,6 +1500,113 @@ struct SddSoftmaxParams {
     float scale_log2e;
 };
 
+// bf16 operands, 64 x 64 blocks, 64 features: the work-group of a block-row (two waves, 32 queries each, the
+// query fragments in registers) walks the row's key blocks twice -- statistics, then probabilities; the scores are
+// recomputed rather than kept -- with the K tiles coming through a ring of three LDS buffers two blocks ahead
+// (LDS-direct loads of whole lines; K is read from L2 the second time) and P leaving through the waves' LDS slabs
+// as whole rows.  Every wait is counted in the loads and stores actually issued (they complete in issue order): in
+// the second pass K(j) is followed by the stores of blocks j-2 and j-1 and the loads of K(j+1).
+template <typename TOut>
+__global__ __launch_bounds__(128) void sdd_softmax_stream_kernel(SddSoftmaxParams p) {
+    constexpr int BS = 64, D = 64, KT = BS / 32, KS = D / 16;
+    using TD = Bf16DirectTiles<BS, D>;
+    using Slab = RowSlab<BS, TOut>;
+    constexpr int TILE = TD::TILE_BYTES;
+    typedef const uint32_t __attribute__((address_space(4)))* const_words;
+    __shared__ __attribute__((aligned(1024))) uint8_t tiles[3 * TILE];
+    __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][Slab::BYTES];
+    // the two longest block-rows of every (batch, head) before anything else (with row_order: its first two; else
+    // the last and the first row, where causal layouts and layouts with global tokens have them)
+    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb, p.nb >= 2 ? 2 : 0);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t r = p.row_order ? p.row_order[work.rank]
+                                   : ((work.rank & 1u) ? work.rank / 2 : p.nb - 1 - work.rank / 2);
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t qn = lane & 31, half = lane >> 5, q_in_block = wave * 32 + qn;
+    const uint32_t L = p.nb * BS, row_bytes = p.heads * D * 2;
+    const const_words head = (const_words)(uintptr_t)(p.nn_lut + (size_t)h * p.lut_stride);
+    const uint32_t off = head[2 * r], count = head[2 * r + 1];
+    if (count == 0) return;
+    const uint32_t last = count - 1;
+    const const_words lut_words = head + 2 * (size_t)off;
+    const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+    const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+    const float c = p.scale_log2e;
+    TOut* Y = (TOut*)p.y + (size_t)work.bh * p.blocks * BS * BS;
+    const uint8_t* const k_base = (const uint8_t*)p.b + token_offset(b, 0, h, L, p.heads, D) * 2;
+    const uint32_t src_even = TD::lane_source(lane, 0, row_bytes), src_odd = TD::lane_source(lane, 1, row_bytes);
+    const uint32_t lds0 = TD::lds_address(tiles), k_lane = TD::k_lane_base(qn, half);
+    auto fetch_k = [&](uint32_t j, uint32_t buf) {
+        const uint32_t col = lut_words[2 * j + 1];
+        TD::load_tile(lds0 + buf * TILE, k_base + (size_t)col * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+    };
+    bf16x8 qf[KS];
+    TD::load_q(qf, (const __bf16*)p.a + token_offset(b, r * BS + q_in_block, h, L, p.heads, D), half);
+    // a use here, so that the fragments are waited for before the loop: inside it the compiler would wait for them
+    // at their first use in every step, with a count that ignores the LDS-direct loads, and drain the tiles in flight
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
+    float m = kMaxSeed, l = 0.f;   // exact running maximum and the sum relative to it (this lane's keys)
+    float inv = 0.f;
+    for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+            inv = 1.0f / (l + __shfl_xor(l, 32) + 1e-6f);
+            __syncthreads();   // every wave is done with the tiles of the first pass
+        }
+        // a fetch past the row's end repeats the last block: the counts stay the same in every step
+        fetch_k(0, 0);
+        fetch_k(1 < count ? 1 : last, 1);
+        for (uint32_t j = 0; j < count; ++j) {
+            // K(j) has landed once only what was issued after it is outstanding: K(j+1), and in the second pass
+            // the stores of blocks j-2 and j-1 (4 or 8 per wave each) -- for j < 2 fewer, so the stricter count
+            if (pass == 0 || j < 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else if (sizeof(TOut) == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+            __syncthreads();   // K(j) is in LDS for every wave, and every wave is done with K(j-1)
+            fetch_k(j + 2 < count ? j + 2 : last, (j + 2) % 3u);
+            const uint8_t* k_read = tiles + (j % 3u) * TILE;
+            const uint32_t blk = lut_words[2 * j], col = lut_words[2 * j + 1];
+            f32x16 s[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TD::k_frag(k_read, k_lane, kt, ks), qf[ks], s[kt], 0, 0, 0);
+            const int limit = valid - (int)(col * BS);
+            if ((mask != nullptr) || (limit < BS))
+                apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)blk * BS + q_in_block, limit), half);
+            if (pass == 0) {
+                const float m_new = fmaxf(m, block_row_max<KT>(s));
+                l *= exp2_fast((m - m_new) * c);
+                m = m_new;
+                const float mc = m * c;
+                float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; i += 2) {
+                        l0 += exp2_fast(__builtin_fmaf(s[kt][i], c, -mc));
+                        l1 += exp2_fast(__builtin_fmaf(s[kt][i + 1], c, -mc));
+                    }
+                l += l0 + l1;
+            } else {
+                const float mc = m * c;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) s[kt][i] = exp2_fast(__builtin_fmaf(s[kt][i], c, -mc)) * inv;
+                Slab::store(Y + ((size_t)blk * BS + wave * 32) * BS, s, slabs[wave], lane);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing in flight towards LDS when the group ends
+}
+
 // Waves of a work-group: BS/32 query halves x kSddSoftmaxKeyGroups key groups.  Key group g takes the row's blocks
 // g, g + 2, ...; the groups meet once, through LDS, to agree on the row maximum and sum.  A long block-row thus
 // has two independent streams of tile loads in flight per query half instead of one (four measured the same on
@@ -1930,6 +2037,11 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
         else SFB_DISPATCH_OTHER_D(state_dim, y_dtype, SFB_CALL32);
 #undef SFB_CALL64
 #undef SFB_CALL32
+        return launch_status();
+    }
+    if (block_size == 64 && in_dtype == SFB_BF16) {
+        if (y_dtype == SFB_BF16) sdd_softmax_stream_kernel<__bf16><<<grid, dim3(128), 0, s>>>(p);
+        else sdd_softmax_stream_kernel<float><<<grid, dim3(128), 0, s>>>(p);
         return launch_status();
     }
 #define SFB_CALL(BSV, TI, TO) sdd_softmax_kernel<BSV, 64, TI, TO><<<grid, dim3(BSV * 2 * kSddSoftmaxKeyGroups), 0, s>>>(p)
