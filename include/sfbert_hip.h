@@ -196,7 +196,14 @@ typedef struct {
 } sfb_stream_plan;
 /*   nn_lut [host] lut_heads tables of lut_dim entries (lut_heads = 1: one layout for all heads; = head_dim:
  *   per-head layouts as fixed_fusion_test.cu:38-39 builds them).  blob [host] NULL: only *plan (sizes) is filled;
- *   otherwise blob_bytes >= plan->total_bytes as returned by such a call. */
+ *   otherwise blob_bytes >= plan->total_bytes as returned by such a call.
+ *   wg_slots: work-groups of the launch; at most sfb_resident_work_groups() if every merge is to find its records'
+ *   producers running (more slots than that still give correct results as long as no bounded wait runs out, which
+ *   sfb_stream_status() reports).  level != 0: cut rows are poured into the streams up to a common level (pieces of
+ *   any length from 2 blocks up); 0: cut into equal pieces of at least 2 blocks, placed like whole rows.
+ *   tail_percent (0..90, used with level = 0): that share of every stream's cost is held back and handed, as
+ *   additional short streams of one row or one merge beyond the first plan->resident ones, to whichever work-group
+ *   slots free up first; 0: none. */
 int sfb_build_stream(sfb_stream_plan* plan, void* blob, size_t blob_bytes, const sfb_uint2* nn_lut, int nb,
                      uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim, uint32_t head_dim, uint32_t block_size,
                      uint32_t wg_slots, int level, uint32_t tail_percent);

@@ -828,19 +828,6 @@ __device__ __forceinline__ StreamItem stream_item(const_words base, uint32_t i, 
     // words: q_off, batch, head, row | kind, part, lse_off, lut_first | count, first, nchunks, chunk
     return StreamItem{uni(w[0]), w[4] != 0 ? uni(w[5]) + 1u : 0u, uni(w[6]), MASKED ? uni(w[1]) : 0u, MASKED ? uni(w[2]) : 0u};
 }
-// Inside the pipeline the entries are fetched with vector loads (every lane the same 16 bytes) instead: a scalar load
-// in flight would turn every wait for an LDS fragment into a wait for all of them (the two share one counter that
-// then counts out of order), whereas these are simply waited for together with the tiles at the end of the iteration.
-__device__ __forceinline__ u32x4 entry_load(const_words base, uint32_t index, uint32_t n, uint32_t words_per_entry, uint32_t word) {
-    index = uni(index);
-    const uint64_t address = (uint64_t)(uintptr_t)(base + (size_t)(index < n ? index : n - 1) * words_per_entry + word);
-    u32x4 out;
-    const uint32_t zero = 0;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(out) : "v"(zero), "s"(address) : "memory");
-    return out;
-}
-// To be called behind the wait for memory: makes what follows use the loaded values, not what the registers held before.
-__device__ __forceinline__ void entry_landed(u32x4& e) { asm volatile("" : "+v"(e)); }
 __device__ __forceinline__ StreamBlock uni(const StreamBlock& e) { return StreamBlock{uni(e.kv_off), uni(e.info), uni(e.col), uni(e.q_off)}; }
 __device__ __forceinline__ StreamItem uni(const StreamItem& it) {
     return StreamItem{uni(it.q_off), uni(it.tag), uni(it.lse_off), uni(it.batch), uni(it.head)};
