@@ -245,7 +245,7 @@ def time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, max_blocks
             "backward_TFLOPs": 2.5 * flops_forward / (ms_b * 1e-3) / 1e12}
 
 
-def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
+def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), steps=20):
     """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
     B, L, ffn = 8, 4096, 3072
     n = H * d
@@ -267,8 +267,10 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks):
     y = torch.empty_like(x)
     attn_flops = luts["blocks"] * B * H * 4.0 * bs * bs * d
     for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
+        if name not in dtypes:
+            continue
         layer = sfb.EncoderLayer(w, luts, bs, H, d, ffn, dtype=code, max_blocks=max_blocks)
-        ms = _time(torch, lambda: layer.forward(x, B, L, out=y), 20, 5)
+        ms = _time(torch, lambda: layer.forward(x, B, L, out=y), steps, 5)
         out["ms_per_layer_" + name] = ms
         # the layer's matrix work (GEMMs + attention blocks) against the MFMA peak of its operand type
         out["roofline_" + name] = {"bound": "mfma", "achieved": (out["gemm_flops"] + attn_flops) / (ms * 1e-3) / 1e12,
@@ -327,6 +329,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (reference kernel for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--layer-only", action="store_true",
+                    help="only the bf16 encoder layer at B8 L4096, 200 timed calls (for a kernel trace of the layer)")
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the fused-attention line: no unfused comparison, no encoder-layer timing")
     ap.add_argument("--heavy", type=int, default=-1,
@@ -352,6 +356,11 @@ def main():
     nb = L // bs
     luts = sfb.build_luts(make_layout(sfb, pattern, nb))
     blocks = luts["blocks"]
+    if args.layer_only:
+        layer_blocks = sfb.suggest_max_blocks(luts["nn_lut"], nb, 8 * H)
+        print(json.dumps({"encoder_layer": time_layer(sfb, torch, luts, bs, H, d, layer_blocks, dtypes=("bf16",),
+                                                      steps=200)}))
+        return
     flops_per_bh = blocks * 4.0 * bs * bs * d
     flops = flops_per_bh * B * H
     elem = 2 if bf16 else 4
