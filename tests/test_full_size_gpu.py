@@ -49,6 +49,47 @@ def test_c4_bigbird_as_benchmarked(bf16):
     assert errs.max() <= (TOL_BF16 if bf16 else TOL_F32)
 
 
+def test_c4_unfused_trio_full_size():
+    """The unfused sdd -> softmax -> dsd sequence and the two-stage fusion at the benchmarked size (bf16 tensors, bf16
+    S and P): the output against the oracle per (batch, head), the two ways to P against each other, and every
+    stage bit-identical over repeated launches (the streaming kernels wait on counts of loads and stores in
+    flight; a count that is too generous would show here as a difference between launches)."""
+    B, H, L, d, bs = 4, 12, 4096, 64, 64
+    nb = L // bs
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    blocks = luts["blocks"]
+    Q, K, V = qkv(B, L, H, d, seed=405, bf16=True)
+    q, k, v = (dev(x, True) for x in (Q, K, V))
+    nt, nn = sfb.to_device(luts["nt_lut"]), sfb.to_device(luts["nn_lut"])
+    runs = []
+    for _ in range(3):
+        S = sfb.bst_sgemm_nt(nt, q, k, bs, blocks, out_dtype=sfb.BF16)
+        P = sfb.BlocksparseMaskedSoftmax(nn, None, S, nb, 0.125)
+        O = sfb.bst_sgemm_xn(nn, P, v, nb)
+        P2 = sfb.fusion_attention2(nn, q, k, bs, blocks, 0.125, out_dtype=sfb.BF16,
+                                   row_order=sfb.to_device(luts["row_order"]))
+        torch.cuda.synchronize()
+        runs.append((S, P, O, P2))
+    for later in runs[1:]:
+        for a, b in zip(runs[0], later):
+            assert torch.equal(a, b)
+    S, P, O, P2 = runs[0]
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    errs = per_head_errors(O.cpu().numpy(), want)
+    print("worst (batch, head) error %.3e" % errs.max(), flush=True)
+    # S and P go through memory as bf16: two roundings more than the fused kernel's output carries (each stage
+    # alone is held to TOL_BF16 against the oracle in test_unfused_gpu.py); a (batch, head) mix-up would be near 1
+    assert errs.max() <= 2 * TOL_BF16
+    # P from bf16-rounded scores against P from the fused product's fp32 scores: the rounding of S moves a
+    # probability by at most |s| * 2^-9 * scale relative
+    diff = (P.float() - P2.float()).abs().amax(dim=(2, 3, 4)) / P2.float().amax(dim=(2, 3, 4))
+    assert float(diff.max()) <= 3e-2
+    rows = P2.float().sum(dim=-1)   # every query row of every block: the blocks of a row add up to 1
+    total = torch.zeros((B, H, nb, bs), device="cuda")
+    total.index_add_(2, torch.from_numpy(luts["nt_lut"][:, 0].astype(np.int64)).cuda(), rows)
+    assert float((total - 1).abs().max()) <= 2e-2
+
+
 @pytest.mark.parametrize("bf16", [True, False])
 def test_c3_strided_full_batch(bf16):
     B, H, L, d, bs = 8, 12, 2048, 64, 64
