@@ -263,6 +263,17 @@ int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const v
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
+/* sfb_fused_attention_scheduled_to for Q, K and V whose token rows are token_stride elements apart instead of
+ * head_dim * state_dim (o stays dense): q, k, v may then be column slices of one [batch * ctx, token_stride] matrix,
+ * e.g. of the result of one merged Q/K/V projection (transformer.cpp:516-522 does three products).  token_stride >=
+ * head_dim * state_dim and a multiple of 8 (bf16) or 4 (fp32) elements; q, k, v 16-byte aligned. */
+int sfb_fused_attention_scheduled_strided(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                          int in_dtype, int out_dtype, const sfb_uint2* nn_lut, const void* mask,
+                                          const int32_t* valid_len, const sfb_work_item* items, uint32_t n_items,
+                                          uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts, void* workspace,
+                                          size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                          uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                          uint32_t token_stride, uint32_t mask_heads, float scale);
 /* No counterpart in the reference.  For callers that cannot allocate device memory or pass a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The same launch as
  * sfb_fused_attention_scheduled_to, with the arrival counters and partial records of split rows kept in a static

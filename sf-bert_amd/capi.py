@@ -68,6 +68,7 @@ EXPORTED = [
     "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
+    "sfb_fused_attention_scheduled_strided",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
@@ -411,6 +412,29 @@ def fused_attention_scheduled(q, k, v, nn_lut, items, sched, workspace, block_si
         C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes), C.c_uint32(block_size),
         C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d),
         C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled")
+    return out
+
+
+def fused_attention_scheduled_strided(qkv, nn_lut, items, sched, workspace, block_size, blocks, scale, heads,
+                                      mask=None, valid_len=None, mask_heads=1, out_dtype=F32):
+    """sfb_fused_attention_scheduled_strided on one [B, L, 3 * H * d] tensor holding Q | K | V side by side in every
+    token row (the result of a merged projection)."""
+    import torch
+    B, L, width = qkv.shape
+    d = width // (3 * heads)
+    if not qkv.is_contiguous() or width != 3 * heads * d:
+        raise SfbError(4, "qkv must be a contiguous [B, L, 3 * heads * d] tensor")
+    out = torch.empty((B, L, heads, d), dtype=_torch_dtype(out_dtype), device=qkv.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    esz = qkv.element_size()
+    base = qkv.data_ptr()
+    _check(lib.sfb_fused_attention_scheduled_strided(
+        _stream(), C.c_void_p(base), C.c_void_p(base + heads * d * esz), C.c_void_p(base + 2 * heads * d * esz),
+        _dev(out), _dtype_code(qkv), out_dtype, _dev(nn_lut), _dev(mask), _dev(valid_len), _dev(items),
+        C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]), C.c_uint32(sched["n_slots"]),
+        C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes), C.c_uint32(block_size),
+        C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(heads), C.c_uint32(d),
+        C.c_uint32(width), C.c_uint32(mask_heads), C.c_float(scale)), "sfb_fused_attention_scheduled_strided")
     return out
 
 

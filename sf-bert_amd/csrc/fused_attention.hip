@@ -44,6 +44,7 @@ struct FusedParams {
     uint32_t n_slots, n_parts;
     uint32_t o_bf16;                // output element type: 0 fp32, 1 bf16 (rounded once from the fp32 result)
     uint32_t batch, heads, nb, blocks;
+    uint32_t in_stride;             // elements between the rows of consecutive tokens in Q, K and V (heads * d when dense)
     uint32_t lut_stride;            // entries between heads' LUTs (0 = shared)
     uint32_t mask_stride;           // words between heads' masks (0 = shared)
     uint32_t groups;                // ceil(batch*heads / 8)
@@ -52,6 +53,12 @@ struct FusedParams {
     float scale_log2e;
     float slack;                    // raw-score distance a block maximum may exceed the reference maximum
 };
+
+// Element offset of (b, token, h, 0) in Q, K or V, whose token rows are p.in_stride elements apart.
+__device__ __forceinline__ size_t input_offset(const FusedParams& p, uint32_t b, uint32_t token, uint32_t h, uint32_t L,
+                                               uint32_t d) {
+    return ((size_t)b * L + token) * p.in_stride + (size_t)h * d;
+}
 
 // What this work-group has to do.
 struct RowWork {
@@ -448,7 +455,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_bytes = p.heads * D * 2;
+    const uint32_t row_bytes = p.in_stride * 2;
 
     const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
     float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
@@ -458,7 +465,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
 
     // byte address of (b, token 0, h, 0) in K and V; key block column col starts col*BS rows further
-    const size_t bh_bytes = token_offset(w.b, 0, w.h, L, p.heads, D) * 2;
+    const size_t bh_bytes = input_offset(p, w.b, 0, w.h, L, D) * 2;
     const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
     const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
     const typename T::Sources src = T::sources(lane, row_bytes);
@@ -492,7 +499,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const float c = p.scale_log2e, slack = p.slack;
 
     bf16x8 qf[KS];
-    T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
+    T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
     if constexpr (SLIM) {
         // the score product then delivers base-2 exponents; the second rounding of Q moves them by less than the
         // rounding of the probabilities does
@@ -689,7 +696,7 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t row_stride = p.in_stride;
 
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
     const uint32_t lut_off = w.lut_first, count = w.count;
@@ -708,7 +715,7 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
     const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
 
     f32x4 qf[QG];
-    T::load_q(qf, Q + token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D), half);
+    T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
 
     typename T::Regs gk, gv;
 
@@ -722,7 +729,7 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
 
     sfb_uint2 entry = lut[lut_off];
     {
-        const size_t base = token_offset(w.b, entry.y * BS, w.h, L, p.heads, D);
+        const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, D);
         T::fetch(gk, K, base, row_stride, t);
         T::fetch(gv, V, base, row_stride, t);
     }
@@ -734,7 +741,7 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
         __syncthreads();
         if (j + 1 < count) {
             entry = lut[lut_off + j + 1];
-            const size_t base = token_offset(w.b, entry.y * BS, w.h, L, p.heads, D);
+            const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, D);
             T::fetch(gk, K, base, row_stride, t);
             T::fetch(gv, V, base, row_stride, t);
         }
@@ -1302,6 +1309,7 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
 // head sizes 32, 64, 96 and 128 for both input types
 template <int BS>
 static int launch_fused_any(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks, uint32_t state_dim) {
+    if (p.in_stride == 0) p.in_stride = p.heads * state_dim;
     switch (state_dim) {
         case 64: return launch_fused<BS, 64>(stream, p, in_dtype, ranks);
         case 32: return launch_fused<BS, 32>(stream, p, in_dtype, ranks);
@@ -1343,6 +1351,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.st_flags = nullptr; p.st_status = nullptr;
     p.n_slots = 0; p.n_parts = 0; p.heavy = 0;
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
+    p.in_stride = 0;   // set by the launcher: heads * d unless the caller gives a token stride
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
     p.groups = bh_groups(batch_dim * head_dim);
@@ -1389,13 +1398,16 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
                                              uint32_t n_parts, void* workspace, size_t workspace_bytes,
                                              uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                              uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
-                                             uint32_t mask_heads, float scale) {
+                                             uint32_t mask_heads, float scale, uint32_t token_stride = 0) {
     using namespace sfb;
     const int rc = check_common(q, k, v, o, in_dtype, nn_lut, block_size, blocks, batch_dim, ctx_blks,
                                 head_dim, state_dim, 1, ctx_blks + blocks, mask_heads, scale);
     if (rc != SFB_OK) return rc;
     if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (!items) return SFB_ERR_NULL_POINTER;
+    // rows of 16-byte vectors: the stride keeps every row aligned
+    if (token_stride != 0 && (token_stride < head_dim * state_dim || token_stride % (in_dtype == SFB_BF16 ? 8u : 4u) != 0))
+        return SFB_ERR_SHAPE;
     if (n_items == 0 || n_heavy >= n_items) return SFB_ERR_SHAPE;
     if ((uint64_t)batch_dim * head_dim * n_items > 0x7fffffffull / 64) return SFB_ERR_SHAPE;
     const size_t need = sfb_schedule_workspace_bytes(n_slots, n_parts, batch_dim, head_dim, block_size, state_dim);
@@ -1406,6 +1418,7 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
                 1, ctx_blks + blocks, mask_heads, scale);
     p.items = items;
     p.lse = lse;
+    p.in_stride = token_stride;
     p.n_slots = n_slots; p.n_parts = n_parts; p.heavy = n_heavy;
     const size_t bh = (size_t)batch_dim * head_dim;
     const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
@@ -1442,6 +1455,21 @@ extern "C" int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void*
     return fused_attention_scheduled(stream, q, k, v, o, nullptr, in_dtype, out_dtype, nn_lut, mask, valid_len, items, n_items,
                                      n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
+}
+
+extern "C" int sfb_fused_attention_scheduled_strided(sfb_stream_t stream, const void* q, const void* k,
+                                                     const void* v, void* o, int in_dtype, int out_dtype,
+                                                     const sfb_uint2* nn_lut, const void* mask,
+                                                     const int32_t* valid_len, const sfb_work_item* items,
+                                                     uint32_t n_items, uint32_t n_heavy, uint32_t n_slots,
+                                                     uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                                     uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                                                     uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                                     uint32_t token_stride, uint32_t mask_heads, float scale) {
+    if (token_stride == 0) return SFB_ERR_SHAPE;
+    return fused_attention_scheduled(stream, q, k, v, o, nullptr, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
+                                     n_items, n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale, token_stride);
 }
 
 extern "C" int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void* q, const void* k,

@@ -227,6 +227,48 @@ def test_head_sizes_other_than_64(d, bs, bf16):
         check(out.cpu().numpy(), ref, tol)
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("d", [64, 32])
+def test_token_stride_of_a_merged_projection(bf16, d):
+    """Q, K and V as column slices of one [B, L, 3 H d] tensor (sfb_fused_attention_scheduled_strided): the same
+    bits as the launch on three dense tensors, split rows, mask and padding included."""
+    bs, nb, B, H = 64, 16, 2, 3
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    keep = (np.random.default_rng(7).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
+    mask = sfb.to_device(sfb.pack_mask(keep))
+    valid = sfb.to_device(np.array([nb * bs, nb * bs - bs - 5], np.int32))
+    Q, K, V = qkv(B, nb * bs, H, d, seed=91 + d, bf16=bf16)
+    q, k, v = (dev(x, bf16) for x in (Q, K, V))
+    merged = torch.cat([t.reshape(B, nb * bs, H * d) for t in (q, k, v)], dim=2).contiguous()
+    sched = sfb.build_schedule(luts["nn_lut"], nb, 3)
+    assert sched["n_parts"] > 0
+    nn, items = sfb.to_device(luts["nn_lut"]), sfb.to_device(sched["items"])
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    scale = float(1.0 / np.sqrt(d))
+    for m, vl in ((None, None), (mask, valid)):
+        for out_dtype in (sfb.F32, sfb.BF16):
+            dense = sfb.fused_attention_scheduled(q, k, v, nn, items, sched, ws, bs, luts["blocks"], scale, mask=m,
+                                                  valid_len=vl, out_dtype=out_dtype)
+            strided = sfb.fused_attention_scheduled_strided(merged, nn, items, sched, ws, bs, luts["blocks"], scale, H,
+                                                            mask=m, valid_len=vl, out_dtype=out_dtype)
+            torch.cuda.synchronize()
+            assert torch.equal(dense, strided)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, nthreads=THREADS)
+    got = sfb.fused_attention_scheduled_strided(merged, nn, items, sched, ws, bs, luts["blocks"], scale, H)
+    check(got.cpu().numpy(), want, TOL_BF16 if bf16 else TOL_F32)
+    with pytest.raises(sfb.SfbError) as e:   # a stride that is not a multiple of 16 bytes
+        bad = torch.zeros((B, nb * bs, 3 * H * d + 3), device="cuda", dtype=merged.dtype)
+        lib_call = sfb.lib.sfb_fused_attention_scheduled_strided
+        sfb.capi._check(lib_call(None, C.c_void_p(bad.data_ptr()), C.c_void_p(bad.data_ptr()), C.c_void_p(bad.data_ptr()),
+                                 C.c_void_p(got.data_ptr()), sfb.BF16 if bf16 else sfb.F32, sfb.F32, C.c_void_p(nn.data_ptr()),
+                                 None, None, C.c_void_p(items.data_ptr()), C.c_uint32(sched["n_items"]),
+                                 C.c_uint32(sched["n_heavy"]), C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]),
+                                 C.c_void_p(ws.data_ptr()), C.c_size_t(ws.numel()), C.c_uint32(bs),
+                                 C.c_uint32(luts["blocks"]), C.c_uint32(B), C.c_uint32(nb), C.c_uint32(H), C.c_uint32(d),
+                                 C.c_uint32(3 * H * d + 3), C.c_uint32(1), C.c_float(scale)), "strided")
+    assert e.value.status == 4
+
+
 def test_head_size_errors():
     luts = sfb.build_luts(PATTERNS["full"](1))
     for dtype in (torch.bfloat16, torch.float32):   # head sizes are 32, 64, 96 and 128
