@@ -517,7 +517,15 @@ typedef struct {
     const void *wq, *wk, *wv, *wo, *w1, *w2;
     const float *bq, *bk, *bv, *bo, *b1, *b2;
     const float *ln1_g, *ln1_b, *ln2_g, *ln2_b;
+    /* optional (NULL: three products, as transformer.cpp:516-522 makes them): [Wq | Wk | Wv] as one [n][3n] matrix
+     * and [bq | bk | bv], filled by sfb_pack_qkv; layers whose attention is a scheduled launch then make Q, K and V
+     * with one product and hand the attention column slices of its result */
+    const void* wqkv;
+    const float* bqkv;
 } sfb_layer_weights;
+/* wqkv [dev] n x 3n of dtype, bqkv [dev] 3n floats from the layer's wq, wk, wv (n x n) and bq, bk, bv (copies on the
+ * stream; the caller then stores the two pointers in the layer's sfb_layer_weights). */
+int sfb_pack_qkv(sfb_stream_t stream, void* wqkv, float* bqkv, const sfb_layer_weights* wt, int dtype, uint32_t n);
 size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim,
                                          uint32_t state_dim, uint32_t ffn, int dtype);
 /* One post-LN encoder layer forward (op arithmetic and order of transformer.cpp:513-580, no dropout):

@@ -73,7 +73,7 @@ EXPORTED = [
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_transpose_0213", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
-    "sfb_gemm_release", "sfb_gemm", "sfb_gemm_bias", "sfb_gemm_bias_gelu", "sfb_gemm_bias_gelu_scaled", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
+    "sfb_pack_qkv", "sfb_gemm_release", "sfb_gemm", "sfb_gemm_bias", "sfb_gemm_bias_gelu", "sfb_gemm_bias_gelu_scaled", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
     "sfb_encoder_layer_forward_streamed",
     "sfb_encoder_layer_forward_pre_ln", "sfb_gemm_nt", "sfb_softmax_cross_entropy", "sfb_model_workspace_bytes",
     "sfb_model_forward",
@@ -777,7 +777,19 @@ def softmax_cross_entropy(logits, labels, want_grad=False, in_place=False):
 
 class LayerWeights(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "bq", "bk", "bv", "bo", "b1", "b2",
-                                          "ln1_g", "ln1_b", "ln2_g", "ln2_b")]
+                                          "ln1_g", "ln1_b", "ln2_g", "ln2_b", "wqkv", "bqkv")]
+
+
+def _pack_qkv(c_weights, tensors, dtype, n):
+    """Fills wqkv / bqkv of a LayerWeights from its wq, wk, wv, bq, bk, bv (sfb_pack_qkv); the new tensors are kept
+    in `tensors`."""
+    import torch
+    w = tensors["wq"]
+    tensors["wqkv"] = torch.empty((n, 3 * n), dtype=w.dtype, device=w.device)
+    tensors["bqkv"] = torch.empty(3 * n, dtype=torch.float32, device=w.device)
+    _check(lib.sfb_pack_qkv(_stream(), _dev(tensors["wqkv"]), _dev(tensors["bqkv"]), C.byref(c_weights), dtype,
+                            C.c_uint32(n)), "sfb_pack_qkv")
+    c_weights.wqkv, c_weights.bqkv = tensors["wqkv"].data_ptr(), tensors["bqkv"].data_ptr()
 
 
 class EncoderLayer:
@@ -787,9 +799,10 @@ class EncoderLayer:
     dtype BF16 casts the six matrices to bf16 once."""
 
     def __init__(self, weights, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16, pre_ln=False,
-                 streamed=False, lut_heads=1, mask_heads=1):
+                 streamed=False, lut_heads=1, mask_heads=1, merge_qkv=True):
         """streamed: the attention runs over build_stream()'s streams (sfb_encoder_layer_forward_streamed); then
-        luts["nn_lut"] may hold lut_heads tables (one per head) and the mask passed to forward() mask_heads masks."""
+        luts["nn_lut"] may hold lut_heads tables (one per head) and the mask passed to forward() mask_heads masks.
+        merge_qkv: Q, K and V as one product (used by layers whose attention is a scheduled launch)."""
         import torch
         self.dtype, self.bs, self.heads, self.d, self.ffn = dtype, block_size, heads, head_state, ffn
         self.luts = luts
@@ -803,6 +816,8 @@ class EncoderLayer:
                 t = cast_bf16(t)
             self.tensors[name] = t
         self.c_weights = LayerWeights(**{n: t.data_ptr() for n, t in self.tensors.items()})
+        if merge_qkv:
+            _pack_qkv(self.c_weights, self.tensors, dtype, heads * head_state)
         self.nn_lut = to_device(luts["nn_lut"])
         self.sched = build_schedule(luts["nn_lut"], luts["nb"], max_blocks) if max_blocks and not streamed else None
         self.items = to_device(self.sched["items"]) if self.sched else None
@@ -867,7 +882,7 @@ class Model:
     tok [vocab, state], pos [ctx, state] fp32 CUDA tensors; layers: list of weight dicts as for EncoderLayer."""
 
     def __init__(self, tok, pos, layers, luts, block_size, heads, head_state, ffn, dtype=F32, max_blocks=16,
-                 pre_ln=True):
+                 pre_ln=True, merge_qkv=True):
         self.dtype, self.bs, self.heads, self.d, self.ffn, self.pre_ln = dtype, block_size, heads, head_state, ffn, pre_ln
         self.luts = luts
         self.tok, self.pos = tok.contiguous(), pos.contiguous()
@@ -883,6 +898,9 @@ class Model:
             self.layer_tensors.append(tensors)
         self.c_layers = (LayerWeights * max(len(layers), 1))(
             *[LayerWeights(**{n: t.data_ptr() for n, t in tensors.items()}) for tensors in self.layer_tensors])
+        if merge_qkv:
+            for i, tensors in enumerate(self.layer_tensors):
+                _pack_qkv(self.c_layers[i], tensors, dtype, heads * head_state)
         self.c_weights = ModelWeights(self.tok.data_ptr(), self.pos.data_ptr(),
                                       self.tok16.data_ptr() if self.tok16 is not None else None, self.c_layers,
                                       len(layers))

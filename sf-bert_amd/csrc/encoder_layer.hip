@@ -325,6 +325,27 @@ extern "C" int sfb_gemm_nt(sfb_stream_t stream, float* c, const void* a, const v
     return st == rocblas_status_success ? SFB_OK : SFB_ERR_LAUNCH;
 }
 
+extern "C" int sfb_pack_qkv(sfb_stream_t stream, void* wqkv, float* bqkv, const sfb_layer_weights* wt, int dtype,
+                            uint32_t n) {
+    if (!wqkv || !bqkv || !wt || !wt->wq || !wt->wk || !wt->wv || !wt->bq || !wt->bk || !wt->bv)
+        return SFB_ERR_NULL_POINTER;
+    if (dtype != SFB_F32 && dtype != SFB_BF16) return SFB_ERR_DTYPE;
+    if (n == 0) return SFB_ERR_SHAPE;
+    const size_t esz = dtype == SFB_BF16 ? 2 : 4;
+    const void* w[3] = {wt->wq, wt->wk, wt->wv};
+    const float* b[3] = {wt->bq, wt->bk, wt->bv};
+    hipStream_t s = (hipStream_t)stream;
+    for (int i = 0; i < 3; ++i) {
+        // row r of W_i becomes columns [i n, (i + 1) n) of row r
+        if (hipMemcpy2DAsync((uint8_t*)wqkv + (size_t)i * n * esz, (size_t)3 * n * esz, w[i], (size_t)n * esz,
+                             (size_t)n * esz, n, hipMemcpyDeviceToDevice, s) != hipSuccess)
+            return SFB_ERR_LAUNCH;
+        if (hipMemcpyAsync(bqkv + (size_t)i * n, b[i], (size_t)n * sizeof(float), hipMemcpyDeviceToDevice, s) != hipSuccess)
+            return SFB_ERR_LAUNCH;
+    }
+    return SFB_OK;
+}
+
 extern "C" size_t sfb_encoder_layer_workspace_bytes(uint32_t batch_dim, uint32_t ctx, uint32_t head_dim,
                                                     uint32_t state_dim, uint32_t ffn, int dtype) {
     const size_t m = (size_t)batch_dim * ctx, n = (size_t)head_dim * state_dim;
@@ -417,6 +438,32 @@ static int attention_call(sfb_stream_t stream, const LayerArgs& g, const void* q
                                scale);
 }
 
+// Q, K and V as one product when the caller supplies the merged matrix (sfb_pack_qkv) and the attention is a
+// scheduled launch on the compute dtype: C [m][3n] = a [Wq | Wk | Wv] + [bq | bk | bv] into the q, k, v buffers (which
+// are consecutive), then the attention reads its three operands as column slices, 3n elements per token.  Returns
+// false when the conditions are not met and the three separate products are to be made.
+static bool merged_projection(sfb_stream_t stream, const LayerArgs& g, const sfb_layer_weights* wt, const void* a,
+                              void* q, void* k, void* v, float* t, void* lp, float* attn, size_t m, size_t n, void* gws,
+                              const void** ain, int* rc) {
+    const size_t act = g.dtype == SFB_BF16 ? 2 : 4;
+    if (!wt->wqkv || !wt->bqkv || !g.items || g.st_plan) return false;
+    if ((uint8_t*)k != (uint8_t*)q + m * n * act || (uint8_t*)v != (uint8_t*)k + m * n * act) return false;
+    if ((3 * n) % (g.dtype == SFB_BF16 ? 8 : 4) != 0) return false;
+    // without a library kernel for this shape the separate products (which have a fallback) are made instead
+    if (gemm_bias_ws(stream, q, g.dtype, a, wt->wqkv, wt->bqkv, g.dtype, (uint32_t)m, (uint32_t)(3 * n), (uint32_t)n, gws,
+                     kGemmWorkspaceBytes) != SFB_OK)
+        return false;
+    const float scale = 1.0f / sqrtf((float)g.state_dim);
+    void* const out = g.dtype == SFB_BF16 ? lp : (void*)attn;
+    *ain = out;
+    *rc = sfb_fused_attention_scheduled_strided(stream, q, (const uint8_t*)q + n * act, (const uint8_t*)q + 2 * n * act, out,
+                                                g.dtype, g.dtype, g.nn_lut, g.mask, g.valid_len, g.items, g.n_items,
+                                                g.n_heavy, g.n_slots, g.n_parts, g.attn_workspace,
+                                                g.attn_workspace_bytes, g.block_size, g.blocks, g.batch_dim, g.ctx_blks,
+                                                g.head_dim, g.state_dim, (uint32_t)(3 * n), 1, scale);
+    return true;
+}
+
 // The reference's own wiring (transformer.cpp:513-580, transformer_inference_part.cpp:209-232), dropout omitted:
 //     a = LN1(x);  x1 = x + (Attn(a Wq + bq, a Wk + bk, a Wv + bv) Wo + bo);  y = x1 + (gelu(LN2(x1) W1 + b1) W2 + b2)
 static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, const sfb_layer_weights* wt,
@@ -443,11 +490,15 @@ static int layer_forward_pre_ln(sfb_stream_t stream, float* y, const float* x, c
     // until the attention runs
     void* a = bf ? xa : (void*)attn;
     SFB_TRY(sfb_layernorm(stream, a, dtype, nullptr, nullptr, x, wt->ln1_g, wt->ln1_b, (uint32_t)m, (uint32_t)n));
-    SFB_TRY(project(stream, q, dtype, t, a, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
-    SFB_TRY(project(stream, k, dtype, t, a, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
-    SFB_TRY(project(stream, v, dtype, t, a, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
     const void* ain = nullptr;
-    SFB_TRY(attention_operand(stream, g, q, k, v, attn, xa, m * n, &ain));
+    if (merged_projection(stream, g, wt, a, q, k, v, t, xa, attn, m, n, gws, &ain, &rc)) {
+        if (rc != SFB_OK) return rc;
+    } else {
+        SFB_TRY(project(stream, q, dtype, t, a, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(project(stream, k, dtype, t, a, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(project(stream, v, dtype, t, a, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(attention_operand(stream, g, q, k, v, attn, xa, m * n, &ain));
+    }
     SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n, gws));
     SFB_TRY(sfb_bias_act(stream, x1, SFB_F32, t, nullptr, x, 0, m, (uint32_t)n));
     // LN2 into the compute dtype (fp32: the attention output buffer again, consumed by the GEMM above)
@@ -536,13 +587,16 @@ static int layer_forward_post_ln(sfb_stream_t stream, float* y, const float* x, 
     // Q, K, V projections (+ bias), stored in the compute dtype for the attention kernel
     const void* xin = x;
     if (bf) { SFB_TRY(sfb_cast_f32_bf16(stream, xa, x, m * n)); xin = xa; }
-    SFB_TRY(project(stream, q, dtype, t, xin, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
-    SFB_TRY(project(stream, k, dtype, t, xin, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
-    SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
-
     // attention, [B, L, H, d] is the token-major activation layout itself: no transposes
     const void* ain = nullptr;
-    SFB_TRY(attention_operand(stream, la, q, k, v, attn, xa, m * n, &ain));
+    if (merged_projection(stream, la, wt, xin, q, k, v, t, xa, attn, m, n, gws, &ain, &rc)) {
+        if (rc != SFB_OK) return rc;
+    } else {
+        SFB_TRY(project(stream, q, dtype, t, xin, wt->wq, wt->bq, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(project(stream, k, dtype, t, xin, wt->wk, wt->bk, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(project(stream, v, dtype, t, xin, wt->wv, wt->bv, dtype, m, (uint32_t)n, (uint32_t)n, gws));
+        SFB_TRY(attention_operand(stream, la, q, k, v, attn, xa, m * n, &ain));
+    }
 
     // output projection + bias, residual, LayerNorm 1
     SFB_TRY(project(stream, t, SFB_F32, t, ain, wt->wo, wt->bo, dtype, m, (uint32_t)n, (uint32_t)n, gws));

@@ -117,6 +117,15 @@ int main(int argc, char** argv) {
         l.b1 = normal_on_device(ffn, 0, 0);   l.b2 = normal_on_device(state, 0, 0);
         l.ln1_g = normal_on_device(state, 0, 1); l.ln1_b = normal_on_device(state, 0, 0);
         l.ln2_g = normal_on_device(state, 0, 1); l.ln2_b = normal_on_device(state, 0, 0);
+        // Q, K and V as one product: [Wq | Wk | Wv] and [bq | bk | bv] side by side
+        void* wqkv = nullptr;
+        float* bqkv = nullptr;
+        HIP_OK(hipMalloc(&wqkv, (size_t)3 * state * state * (dtype == SFB_BF16 ? 2 : 4)));
+        HIP_OK(hipMalloc((void**)&bqkv, (size_t)3 * state * sizeof(float)));
+        if (sfb_pack_qkv(nullptr, wqkv, bqkv, &l, dtype, (uint32_t)state) != SFB_OK) return 2;
+        HIP_OK(hipDeviceSynchronize());
+        l.wqkv = wqkv;
+        l.bqkv = bqkv;
     }
     sfb_model_weights w;
     w.tok_embed = normal_on_device((size_t)vocab_size * state, 0.02f, 0.f);

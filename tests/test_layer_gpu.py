@@ -212,6 +212,32 @@ def test_encoder_layer_streamed_matches_oracle(bf16, pre_ln):
         assert rel_err(got, want) <= (1e-2 if bf16 else 1e-4)
 
 
+@pytest.mark.parametrize("pre_ln", [False, True])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_encoder_layer_merged_qkv_product(bf16, pre_ln):
+    """Q, K and V as one product (sfb_pack_qkv, the attention reading column slices of its result): same result as
+    the three products of transformer.cpp:516-522, both wirings, and the oracle's within tolerance."""
+    B, L, H, d, ffn, bs = 2, 1024, 12, 64, 3072, 64
+    n, nb = H * d, L // bs
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    w = layer_weights(n, ffn, 120)
+    for name in ("bq", "bk", "bv"):
+        w[name] = orc.fill_normal((n,), 121 + len(name) + ord(name[1])) * 0.1   # distinct biases: a mix-up shows
+    x = orc.fill_normal((B * L, n), 320)
+    oracle = orc.encoder_layer_pre_ln if pre_ln else orc.encoder_layer
+    want = oracle(x, w, luts["nn_lut"], B, L, H, d, ffn, bs, luts["blocks"], operands_bf16=bf16, nthreads=16)
+    outs = []
+    for merge in (False, True):
+        layer = sfb.EncoderLayer({k: T(v) for k, v in w.items()}, luts, bs, H, d, ffn,
+                                 dtype=sfb.BF16 if bf16 else sfb.F32, pre_ln=pre_ln, max_blocks=4, merge_qkv=merge)
+        assert (layer.c_weights.wqkv is not None) == merge
+        outs.append(layer.forward(T(x), B, L))
+        torch.cuda.synchronize()
+        assert rel_err(outs[-1].cpu().numpy(), want) <= (1e-2 if bf16 else 1e-4)
+    # the same products over the same k, only laid side by side: bf16 identical, fp32 to rounding of another kernel
+    assert float((outs[0] - outs[1]).abs().max()) <= (0 if bf16 else 1e-4) * float(outs[0].abs().max())
+
+
 def test_encoder_layer_per_head_luts_and_masks():
     """The reference's `fixed` pattern gives every head its own layout and mask (fixed_fusion_test.cu:38-39, 58-106):
     the streamed layer against the same layer put together from the oracle's operations (fp32)."""
