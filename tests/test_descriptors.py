@@ -112,6 +112,15 @@ def test_error_codes():
     assert sfb.lib.sfb_pack_mask(lay.ctypes.data_as(C.c_void_p), lay.ctypes.data_as(C.c_void_p), 1, 24) == 2
     with pytest.raises(sfb.capi.SfbError):
         sfb.layout_local(4, -1)
+    # device entry points check their arguments before they touch the device
+    assert sfb.lib.sfb_pack_qkv(None, None, None, None, sfb.BF16, C.c_uint32(64)) == 1
+    u32 = C.c_uint32
+    strided = sfb.lib.sfb_fused_attention_scheduled_strided
+    args_tail = (u32(64), u32(1), u32(1), u32(1), u32(1), u32(64))
+    assert strided(None, None, None, None, None, sfb.BF16, sfb.F32, None, None, None, None, u32(1), u32(0), u32(0),
+                   u32(0), None, C.c_size_t(0), *args_tail, u32(0), u32(1), C.c_float(0.125)) == 4   # no stride given
+    assert strided(None, None, None, None, None, sfb.BF16, sfb.F32, None, None, None, None, u32(1), u32(0), u32(0),
+                   u32(0), None, C.c_size_t(0), *args_tail, u32(64), u32(1), C.c_float(0.125)) == 1   # NULL tensors
 
 
 def test_suggested_chunk_length():
