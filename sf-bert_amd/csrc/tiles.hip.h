@@ -12,6 +12,7 @@
 #pragma once
 
 #include "common.hip.h"
+#include "tile_index.h"
 
 namespace sfb {
 
@@ -39,33 +40,29 @@ struct Bf16DirectTiles {
     // tile).  A last slice of 32 features (head sizes 32 and 96) fills only the first four chunks of its rows: its
     // lanes fetch chunk (c ^ swz) & 3 instead of c ^ swz, so that nothing beyond the row is read, and the fragment
     // readers, which only ever ask for chunks 0..3 of such a slice, find them where they expect them.
-    static constexpr int NW = BS / 32;                 // waves per work-group
-    static constexpr int SLICES = (D + 63) / 64;
-    static constexpr bool PARTIAL = D % 64 != 0;       // the last slice has 32 features
-    static constexpr int SLICE_BYTES = BS * 128;
-    static constexpr int TILE_BYTES = SLICES * SLICE_BYTES;
-    static constexpr int GROUPS = BS / 8;              // 8-row groups (one load instruction each)
-    static_assert(D % 32 == 0 && D >= 32 && D <= 128, "head sizes 32, 64, 96, 128");
+    // Every offset comes from TileIndex (tile_index.h), which a host program can compile and check.
+    using I = TileIndex<BS, D>;
+    static constexpr int NW = I::NW;                   // waves per work-group
+    static constexpr int SLICES = I::SLICES;
+    static constexpr bool PARTIAL = I::PARTIAL;        // the last slice has 32 features
+    static constexpr int SLICE_BYTES = I::SLICE_BYTES;
+    static constexpr int TILE_BYTES = I::TILE_BYTES;
+    static constexpr int GROUPS = I::GROUPS;           // 8-row groups (one load instruction each)
 
     typedef uint32_t __attribute__((address_space(3)))* lds_u32_ptr;
     // LDS byte address of a pointer into a __shared__ array
     static __device__ __forceinline__ uint32_t lds_address(const void* p) {
         return (uint32_t)(uintptr_t)(lds_u32_ptr)p;
     }
-    static __device__ __forceinline__ uint32_t swz(uint32_t row) {
-        const uint32_t x = (row >> 1) & 7u;
-        return ((x & 1u) << 2) | (x >> 1);
-    }
+    static __device__ __forceinline__ uint32_t swz(uint32_t row) { return I::swz(row); }
     // Byte offset, relative to row 0 of an 8-row group, of the 16 bytes this lane fetches; `odd` says
     // whether the group index is odd (rows 8..15 of a 16-row period).
     static __device__ __forceinline__ uint32_t lane_source(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
-        const uint32_t rr = lane >> 3, pos = lane & 7u;
-        return rr * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
+        return I::lane_source(lane, odd, row_bytes);
     }
     // The same for a last slice of 32 features.
     static __device__ __forceinline__ uint32_t lane_source_part(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
-        const uint32_t rr = lane >> 3, pos = lane & 7u;
-        return rr * row_bytes + (((pos ^ swz(8u * odd + rr)) & 3u) << 4);
+        return I::lane_source_part(lane, odd, row_bytes);
     }
     // The four lane offsets a work-group needs to fetch whole tiles.
     struct Sources {
@@ -80,26 +77,26 @@ struct Bf16DirectTiles {
         return s;
     }
     // The same for a tile whose LDS rows hold the source rows in the order that makes the 8 k-slots of a lane
-    // in the second product, rows 16u + 8(j/4) + 4*half + j%4 of the tile, the 8 consecutive source rows
-    // 32*half + 8u + j: LDS row 16u + 8a + 4h + c holds source row 32h + 8u + 4a + c, which is 4n + 32(rr/4) + rr%4
-    // for row rr of 8-row group n.  Used with load_rows<4>: the group's base advances by 4 source rows.
+    // in the second product 8 consecutive source rows.  Used with load_rows<4>: the group's base advances by 4
+    // source rows.
     static __device__ __forceinline__ uint32_t lane_source_by_halves(uint32_t lane, uint32_t odd, uint32_t row_bytes) {
-        const uint32_t rr = lane >> 3, pos = lane & 7u;
-        return (32u * (rr >> 2) + (rr & 3u)) * row_bytes + ((pos ^ swz(8u * odd + rr)) << 4);
+        return I::lane_source_by_halves(lane, odd, row_bytes);
     }
     // Load number i (0 .. LOADS-1) of this wave's share of one tile: 8 rows = 1 KiB.  g_tile: address of
     // the tile's first row (uniform); lds_tile: LDS byte address of the tile (uniform); src_even /
     // src_odd from lane_source().
-    static constexpr int LOADS = GROUPS / NW;
+    static constexpr int LOADS = I::LOADS;
     template <int GROUP_ROWS = 8>
     static __device__ __forceinline__ void load_rows(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                      uint32_t src_even, uint32_t src_odd, uint32_t row_bytes) {
-        const uint32_t n = (uint32_t)(NW * i) + wave;   // 8-row group
-        uint32_t src;
-        if (NW % 2 == 0) src = (wave & 1u) ? src_odd : src_even;   // parity of n is the wave's
-        else src = (i & 1) ? src_odd : src_even;                   // one wave: parity of i
+        const uint32_t n = I::load_group(i, wave);      // 8-row group
+        const uint32_t src = I::load_group_odd(i, wave) ? src_odd : src_even;
         // scalar 64-bit base + 32-bit lane offset: no vector address arithmetic.  The instruction takes its
-        // LDS destination from M0, which is written here; nothing else in these kernels depends on M0.
+        // LDS destination from M0, which is written in the same statement.  M0 cannot be named as a clobber (the
+        // compiler reserves it and rejects it there); it never keeps a value in M0 across statements -- it writes
+        // M0 directly before each instruction of its own that reads it -- and these kernels use none of the
+        // operations for which it would (LDS-direct builtins, messages, relative register moves): in the compiled
+        // kernels every write of M0 is one of these, each followed by its load, which a test of the assembly checks.
         const uint64_t ga = (uint64_t)(g_tile + (size_t)n * (uint32_t)GROUP_ROWS * row_bytes);
         const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
         const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);   // unsigned: no sign extension
@@ -140,24 +137,21 @@ struct Bf16DirectTiles {
     // Per-lane byte offset of the score fragment of k-step 0 in key tile 0; k-step ks is at (base ^ ks*32),
     // key tile kt 4096 bytes further.
     static __device__ __forceinline__ uint32_t k_lane_base(uint32_t qn, uint32_t half) {
-        return qn * 128u + ((half ^ swz(qn)) << 4);
+        return I::k_lane_base(qn, half);
     }
     static __device__ __forceinline__ bf16x8 k_frag(const uint8_t* k_lds, uint32_t lane_base, int kt, int ks) {
-        return *(const bf16x8*)(k_lds + (ks / 4) * SLICE_BYTES + kt * 4096 + (lane_base ^ (uint32_t)((ks % 4) * 32)));
+        return *(const bf16x8*)(k_lds + I::k_frag_const(kt, ks) + I::k_frag_lane(lane_base, ks));
     }
     // Per-lane byte offset of the transposing read for (column tile 0, first 4-key group of product step
     // 0); column tile mt and second group x are at (base ^ (mt*64 + x*32)) + x*1024, step u 2048 bytes on.
     static __device__ __forceinline__ uint32_t v_lane_base(uint32_t lane) {
-        const uint32_t G = lane >> 4, s = lane & 15u, j = s >> 2, q = s & 3u, h = G >> 1, g2 = G & 1u;
-        const uint32_t lp = (2u * g2 + (q >> 1)) ^ (((j >> 1) << 2) | h);
-        return (h * 4u + j) * 128u + (lp << 4) + (q & 1u) * 8u;
+        return I::v_lane_base(lane);
     }
     static __device__ __forceinline__ bf16x8 v_frag(const uint8_t* v_lds, uint32_t lane_base, int mt, int u) {
         typedef short s16x4 __attribute__((ext_vector_type(4)));
         typedef s16x4 __attribute__((address_space(3)))* lds_ptr;
-        const uint8_t* slice = v_lds + (mt / 2) * SLICE_BYTES;
-        const uint8_t* a0 = slice + u * 2048 + (lane_base ^ (uint32_t)((mt % 2) * 64));
-        const uint8_t* a1 = slice + u * 2048 + 1024 + (lane_base ^ (uint32_t)((mt % 2) * 64 + 32));
+        const uint8_t* a0 = v_lds + I::v_frag_const(mt, u, 0) + I::v_frag_lane(lane_base, mt, 0);
+        const uint8_t* a1 = v_lds + I::v_frag_const(mt, u, 1) + I::v_frag_lane(lane_base, mt, 1);
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a0);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)a1);
         const u32x4 r = {__builtin_bit_cast(u32x2, lo).x, __builtin_bit_cast(u32x2, lo).y,

@@ -133,11 +133,12 @@ __device__ __forceinline__ void score_tile(f32x16 (&s)[BS / 32], const KTile<BS,
 // or 16 bytes each, here every instruction moves 1 KiB of consecutive bytes.
 template <int BS, typename T>
 struct RowSlab {
-    static constexpr int ROW_BYTES = BS * (int)sizeof(T);
-    static constexpr int PITCH = ROW_BYTES + 16;          // padded LDS row
-    static constexpr int BYTES = 32 * PITCH;              // per wave
-    static constexpr int CHUNKS = ROW_BYTES / 16;         // 16-byte chunks per row
-    static constexpr int ROWS_PER_PASS = 64 / CHUNKS, PASSES = 32 / ROWS_PER_PASS;
+    using I = RowSlabIndex<BS, (int)sizeof(T)>;
+    static constexpr int ROW_BYTES = I::ROW_BYTES;
+    static constexpr int PITCH = I::PITCH;                // padded LDS row
+    static constexpr int BYTES = I::BYTES;                // per wave
+    static constexpr int CHUNKS = I::CHUNKS;              // 16-byte chunks per row
+    static constexpr int ROWS_PER_PASS = I::ROWS_PER_PASS, PASSES = I::PASSES;
 
     // registers (this lane's query row, groups of 4 keys) -> memory; rows: the wave's first row in memory
     static __device__ __forceinline__ void store(T* rows, const f32x16 (&s)[BS / 32], uint8_t* slab, uint32_t lane) {
@@ -275,7 +276,8 @@ __global__ __launch_bounds__(128) void sdd_nt_stream_kernel(SddParams p) {
     for (uint32_t g = 0; g < n; ++g) {
         const uint32_t row = lut_words[2 * g];
         if (row != cur_row) {
-            // a new block-row (always in the first step): its query fragments, waited for at once
+            // a new block-row (in the first step, and wherever the group of entries crosses into the next
+            // block-row): its query fragments, waited for at once -- which also drains the tiles in flight
             static_assert(D / 16 == 4, "four k-steps");
             const uint8_t* q_rows = q_base + (size_t)row * BS * row_bytes;
             asm volatile("global_load_dwordx4 %0, %4, %5\n\t"
@@ -288,8 +290,10 @@ __global__ __launch_bounds__(128) void sdd_nt_stream_kernel(SddParams p) {
                          : "memory");
             cur_row = row;
         }
-        if (sizeof(TOut) == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");   // 4 loads + 2 x 4 stores
-        else asm volatile("s_waitcnt vmcnt(20)" ::: "memory");                       // 4 loads + 2 x 8 stores
+        // K(g+1)'s loads and the stores of two blocks: 4 + 2 x 4 (bf16 S) or 4 + 2 x 8 (fp32 S)
+        static_assert(Slab::PASSES == SddStreamWait<sizeof(TOut)>::PASSES && TD::LOADS == SddStreamWait<sizeof(TOut)>::LOADS,
+                      "the wait counts what this loop issues");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SddStreamWait<sizeof(TOut)>::COUNT) : "memory");
         __syncthreads();   // K(g) is in LDS for every wave, and every wave is done with K(g-1)
         fetch_k(g + 2 < n ? g + 2 : last, (g + 2) % 3u);
         const uint8_t* k_read = tiles + (g % 3u) * TILE;
@@ -1301,7 +1305,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         // with its key rows in the matching order (lane_source_by_halves).  V tiles (L2 hits mostly) go through a
         // ring of four LDS buffers, two blocks per barrier.  Loads complete in issue order, which the counted
         // waits below rely on.
-        constexpr int PU = BS / 16, TILE = TD::TILE_BYTES, kDepth = 4;
+        constexpr int PU = BS / 16, TILE = TD::TILE_BYTES, kDepth = DsdStreamWait::DEPTH;
+        static_assert(PU == DsdStreamWait::P_LOADS && TD::LOADS == DsdStreamWait::V_LOADS, "the wait counts what this loop issues");
         const uint32_t row_bytes = row_stride * 2;
         const uint32_t v_even = TD::lane_source_by_halves(lane, 0, row_bytes);
         const uint32_t v_odd = TD::lane_source_by_halves(lane, 1, row_bytes);
@@ -1354,10 +1359,10 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
 #pragma unroll
                 for (int d = 0; d < kDepth; d += 2) {
                     const uint32_t j = j0 + d;
-                    asm volatile("s_waitcnt vmcnt(8)"
+                    asm volatile("s_waitcnt vmcnt(%8)"
                                  : "+v"(pr[d][0]), "+v"(pr[d][1]), "+v"(pr[d][2]), "+v"(pr[d][3]), "+v"(pr[d + 1][0]),
                                    "+v"(pr[d + 1][1]), "+v"(pr[d + 1][2]), "+v"(pr[d + 1][3])
-                                 :
+                                 : "n"(DsdStreamWait::COUNT)
                                  : "memory");
                     __syncthreads();   // V(j), V(j+1) are in LDS for every wave; every wave is done with V(j-2), V(j-1)
                     fetch_v(j + 2 < count ? j + 2 : last, (j + 2) % 4u);
@@ -1560,9 +1565,10 @@ __global__ __launch_bounds__(128) void sdd_softmax_stream_kernel(SddSoftmaxParam
         for (uint32_t j = 0; j < count; ++j) {
             // K(j) has landed once only what was issued after it is outstanding: K(j+1), and in the second pass
             // the stores of blocks j-2 and j-1 (4 or 8 per wave each) -- for j < 2 fewer, so the stricter count
-            if (pass == 0 || j < 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-            else if (sizeof(TOut) == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+            static_assert(Slab::PASSES == SddStreamWait<sizeof(TOut)>::PASSES && TD::LOADS == SddStreamWait<sizeof(TOut)>::LOADS,
+                          "the wait counts what this loop issues");
+            if (pass == 0 || j < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SddStreamWait<sizeof(TOut)>::LOADS) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SddStreamWait<sizeof(TOut)>::COUNT) : "memory");
             __syncthreads();   // K(j) is in LDS for every wave, and every wave is done with K(j-1)
             fetch_k(j + 2 < count ? j + 2 : last, (j + 2) % 3u);
             const uint8_t* k_read = tiles + (j % 3u) * TILE;

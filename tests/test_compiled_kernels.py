@@ -1,0 +1,200 @@
+"""Checks of the compiled gfx950 assembly of the attention kernels (hipcc cross-compiles without a GPU).
+
+The counted waits of the streaming kernels (tests/test_counted_waits.py models them) are only right while a step of
+their loops issues exactly the vector memory operations the count was made from: no register spill to scratch, no
+split store, no load the compiler added.  And the LDS-direct loads write M0 from inline assembly without being able
+to name it as a clobber, which is only safe while nothing else in the kernels uses M0.  Both are properties of the
+compiler's output, so they are checked there."""
+import importlib.util
+import os
+import re
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+import pytest
+
+from tile_index_lib import BUILD, ROOT, lib
+
+CSRC = os.path.join(ROOT, "sf-bert_amd", "csrc")
+FILES = ["unfused_attention.hip", "fused_attention.hip", "fused_backward.hip"]
+VMEM = re.compile(r"^\s+(global_|buffer_|scratch_|flat_)(\w+)")
+
+
+def _device_flags():
+    spec = importlib.util.spec_from_file_location("sfb_build_flags", os.path.join(ROOT, "sf-bert_amd", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.HIPCC, mod.DEVICE_FLAGS
+
+
+def _assemble(name):
+    """csrc/<name> -> assembly text of its device code (cached until a source changes)."""
+    hipcc, flags = _device_flags()
+    out = os.path.join(BUILD, name + ".s")
+    sources = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hip", ".h"))]
+    sources.append(os.path.join(ROOT, "include", "sfbert_hip.h"))
+    if not os.path.exists(out) or os.path.getmtime(out) < max(os.path.getmtime(s) for s in sources):
+        os.makedirs(BUILD, exist_ok=True)
+        subprocess.run([hipcc] + flags + ["-x", "hip", "--cuda-device-only", "-S", "-o", out, os.path.join(CSRC, name)],
+                       check=True, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+    with open(out) as f:
+        return f.read()
+
+
+@pytest.fixture(scope="module")
+def kernels():
+    """{demangled-ish symbol: list of assembly lines} over all three files."""
+    with ThreadPoolExecutor(len(FILES)) as pool:
+        texts = list(pool.map(_assemble, FILES))
+    out = {}
+    for text in texts:
+        name, body = None, []
+        for line in text.split("\n"):
+            m = re.match(r"^(_Z\w+):", line)
+            if m:
+                name, body = m.group(1), []
+                out[name] = body
+            elif name is not None:
+                body.append(line)          # up to the next symbol: the resource comments follow .Lfunc_end
+    assert len(out) > 100
+    return out
+
+
+def find(kernels, *parts):
+    hits = [k for k in kernels if all(p in k for p in parts)]
+    assert len(hits) == 1, (parts, hits)
+    return kernels[hits[0]]
+
+
+def scratch_bytes(body):
+    for line in body:
+        m = re.match(r"^; ScratchSize: (\d+)", line)
+        if m:
+            return int(m.group(1))
+    raise AssertionError("no ScratchSize line")
+
+
+def loop_lines(body):
+    """Lines inside any loop: the union of [label, backward branch to it] spans."""
+    labels = {m.group(1): i for i, line in enumerate(body) if (m := re.match(r"^(\.LBB\w+):", line))}
+    inside = [False] * len(body)
+    for i, line in enumerate(body):
+        m = re.match(r"^\s+s_c?branch\w*\s+(\.LBB\w+)", line)
+        if m and labels.get(m.group(1), len(body)) < i:
+            for k in range(labels[m.group(1)], i + 1):
+                inside[k] = True
+    return [line for line, keep in zip(body, inside) if keep]
+
+
+def events(lines):
+    """Vector memory operations and vmcnt waits in text order: ('lds' | 'load' | 'store' | 'other', mnemonic) and
+    ('wait', N)."""
+    out = []
+    for line in lines:
+        m = re.match(r"^\s+s_waitcnt .*vmcnt\((\d+)\)", line)
+        if m:
+            out.append(("wait", int(m.group(1))))
+            continue
+        m = VMEM.match(line)
+        if m:
+            op = m.group(1) + m.group(2)
+            kind = ("lds" if "load_lds" in op else "load" if "_load_" in op else "store" if "_store_" in op else "other")
+            out.append((kind, op))
+    return out
+
+
+def between_counted_waits(ev, count):
+    """For every wait of exactly `count`: the operations up to the next wait of any count (or the end)."""
+    spans = []
+    for i, e in enumerate(ev):
+        if e == ("wait", count):
+            span = []
+            for f in ev[i + 1:]:
+                if f[0] == "wait":
+                    break
+                span.append(f)
+            spans.append(span)
+    return spans
+
+
+def kinds(span):
+    out = {}
+    for kind, _ in span:
+        out[kind] = out.get(kind, 0) + 1
+    return out
+
+
+@pytest.mark.parametrize("elem,elem_bytes", [("DF16b", 2), ("f", 4)])
+def test_sdd_stream_step_issues_what_its_wait_counts(kernels, elem, elem_bytes):
+    L = lib()
+    body = find(kernels, "sdd_nt_stream_kernelI" + elem + "E")
+    assert scratch_bytes(body) == 0
+    ev = events(loop_lines(body))
+    count, loads, passes = L.ti_sdd_wait_count(elem_bytes), L.ti_sdd_wait_loads(elem_bytes), L.ti_slab_passes(elem_bytes)
+    spans = between_counted_waits(ev, count)
+    assert len(spans) == 1
+    # a step issues the next tile's loads and the block's stores; the only other memory operations of the loop are
+    # the four query fragments of a new block-row (the loop's first block in text order), drained at once
+    assert [k for k, _ in spans[0]] == ["lds"] * loads + ["store"] * passes + ["load"] * 4
+    assert ev.count(("wait", count)) == 1 and ev.count(("wait", 0)) == 1
+    assert len([e for e in ev if e[0] != "wait"]) == len(spans[0])
+    following = ev[ev.index(("wait", count)) + 1 + len(spans[0]):] + ev[:ev.index(("wait", count))]
+    assert following[0] == ("wait", 0), "the query fragments are waited for before anything else is issued"
+
+
+@pytest.mark.parametrize("elem,elem_bytes", [("DF16b", 2), ("f", 4)])
+def test_sdd_softmax_stream_step_issues_what_its_waits_count(kernels, elem, elem_bytes):
+    L = lib()
+    body = find(kernels, "sdd_softmax_stream_kernelI" + elem + "E")
+    assert scratch_bytes(body) == 0
+    ev = events(loop_lines(body))
+    count, loads, passes = L.ti_sdd_wait_count(elem_bytes), L.ti_sdd_wait_loads(elem_bytes), L.ti_slab_passes(elem_bytes)
+    assert ("wait", count) in ev and ("wait", loads) in ev
+    # a step: [wait] K tile loads, then possibly a mask word (drained at once), then the block's stores
+    step = ev[ev.index(("wait", loads)) + 1:]
+    assert [k for k, _ in step[:loads]] == ["lds"] * loads
+    tail = step[loads:]
+    if tail and tail[0][0] == "load":
+        assert tail[1] == ("wait", 0)
+        tail = tail[2:]
+    assert [k for k, _ in tail[:passes]] == ["store"] * passes
+    assert all(k == "wait" or k == "lds" for k, _ in ev[:ev.index(("wait", count))]), "pass prologue: tile loads only"
+    assert kinds([e for e in ev if e[0] != "wait"]) in ({"lds": 3 * loads, "store": passes, "load": 1},
+                                                        {"lds": 3 * loads, "store": passes})
+
+
+def test_dsd_stream_steps_issue_what_their_wait_counts(kernels):
+    L = lib()
+    body = find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bE")
+    assert scratch_bytes(body) == 0
+    ev = events(loop_lines(body))
+    spans = between_counted_waits(ev, L.ti_dsd_wait_count())
+    assert len(spans) == L.ti_dsd_depth() // 2
+    for span in spans:
+        assert [k for k, _ in span] == ["lds"] * (2 * L.ti_dsd_v_loads()) + ["load"] * (2 * L.ti_dsd_p_loads())
+    assert sum(len(s) for s in spans) == len([e for e in ev if e[0] != "wait"]), "nothing else in the loop"
+
+
+def test_m0_is_only_written_for_the_lds_direct_loads(kernels):
+    """Every instruction that names M0 is an s_mov into it, and the next instruction (after the s_nop of the same
+    inline-assembly statement) is the LDS-direct load that reads it."""
+    seen = 0
+    for name, body in kernels.items():
+        code = [line for line in body if re.match(r"^\s+[a-z]", line)]
+        for i, line in enumerate(code):
+            if not re.search(r"\bm0\b", line):
+                continue
+            assert re.match(r"^\s+s_mov_b32 m0, (s\d+|vcc_lo|vcc_hi|ttmp\d+)\s*$", line), (name, line)
+            follow = [c.split()[0] for c in code[i + 1:i + 3]]
+            assert follow == ["s_nop", "global_load_lds_dwordx4"], (name, line, follow)
+            seen += 1
+    assert seen > 1000
+
+
+def test_the_model_of_a_step_is_not_vacuous(kernels):
+    """The span extraction does see a count that does not match: the fp32 kernel's loop against the bf16 count."""
+    L = lib()
+    ev = events(loop_lines(find(kernels, "sdd_nt_stream_kernelIfE")))
+    assert between_counted_waits(ev, L.ti_sdd_wait_count(2)) == []
+    spans = between_counted_waits(ev, L.ti_sdd_wait_count(4))
+    assert kinds(spans[0]) != {"lds": L.ti_sdd_wait_loads(2), "store": L.ti_slab_passes(2)}
