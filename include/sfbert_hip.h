@@ -197,7 +197,7 @@ typedef struct {
 /*   nn_lut [host] lut_heads tables of lut_dim entries (lut_heads = 1: one layout for all heads; = head_dim:
  *   per-head layouts as fixed_fusion_test.cu:38-39 builds them).  blob [host] NULL: only *plan (sizes) is filled;
  *   otherwise blob_bytes >= plan->total_bytes as returned by such a call.
- *   wg_slots: work-groups of the launch; at most sfb_resident_work_groups() if every merge is to find its records'
+ *   wg_slots: work-groups of the launch; at most sfb_resident_work_groups_for() if every merge is to find its records'
  *   producers running (more slots than that still give correct results as long as no bounded wait runs out, which
  *   sfb_stream_status() reports).  level != 0: cut rows are poured into the streams up to a common level (pieces of
  *   any length from 2 blocks up); 0: cut into equal pieces of at least 2 blocks, placed like whole rows.
@@ -208,9 +208,21 @@ int sfb_build_stream(sfb_stream_plan* plan, void* blob, size_t blob_bytes, const
                      uint32_t lut_heads, uint32_t lut_dim, uint32_t batch_dim, uint32_t head_dim, uint32_t block_size,
                      uint32_t wg_slots, int level, uint32_t tail_percent);
 /* Bytes of the [dev] workspace a streamed launch needs: one flag per partial record, the records, a status word.
- * The workspace must be zero-filled once before its first use; launches leave the flags at zero. */
+ * The workspace must be zero-filled once before its first use; a launch whose merges all found their records
+ * (sfb_stream_status() == 0) leaves the flags at zero.  After a launch that reports status 1 the flags of the rows
+ * it gave up on are still set (their producers set them after the merge had left) and the status word stays 1:
+ * the workspace must be cleared with sfb_stream_reset() before the next launch uses it, or that launch would add
+ * records its producers have not written yet. */
 size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim);
-/* Work-groups of the fused kernels the current device keeps resident (4 per compute unit); 0 without a device. */
+/* Clears the flags and the status word of a streamed launch's workspace (fill kernels on `stream`; the partial
+ * records need no clearing).  Also usable instead of the initial zero-fill. */
+int sfb_stream_reset(sfb_stream_t stream, const sfb_stream_plan* plan, uint32_t state_dim, void* workspace);
+/* Work-groups the current device keeps resident of the kernel that a streamed launch with these tensors runs
+ * (asked of the runtime for that kernel: 4 per compute unit for head sizes up to 64, 2 for 96 and 128, whose tiles
+ * take twice the LDS); masked != 0: the launch has an element mask, key padding or a log-sum-exp output.  This is
+ * the wg_slots for which every merge finds its records' producers running.  0 without a device. */
+uint32_t sfb_resident_work_groups_for(int in_dtype, uint32_t block_size, uint32_t state_dim, int masked);
+/* The same for bf16 tensors, blocks of 64 and head size 64 without mask. */
 uint32_t sfb_resident_work_groups(void);
 
 /* ================================================================================================

@@ -52,6 +52,7 @@ lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
 lib.sfb_resident_work_groups.restype = C.c_uint32
+lib.sfb_resident_work_groups_for.restype = C.c_uint32
 lib.sfb_stream_workspace_bytes.restype = C.c_size_t
 lib.sfb_static_scratch_bytes.restype = C.c_size_t
 lib.sfb_gemm_release.restype = None
@@ -64,7 +65,8 @@ EXPORTED = [
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
-    "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_resident_work_groups",
+    "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_stream_reset", "sfb_resident_work_groups",
+    "sfb_resident_work_groups_for",
     "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
@@ -219,8 +221,10 @@ def build_schedule(nn_lut, nb, max_blocks=16):
                 n_slots=int(n_slots.value), n_parts=int(n_parts.value))
 
 
-def resident_work_groups():
-    return int(lib.sfb_resident_work_groups())
+def resident_work_groups(bf16=True, block_size=64, d=64, masked=False):
+    """Work-groups the device keeps resident of the streamed kernel for these tensors (0 without a device)."""
+    return int(lib.sfb_resident_work_groups_for(C.c_int(BF16 if bf16 else F32), C.c_uint32(block_size), C.c_uint32(d),
+                                                C.c_int(1 if masked else 0)))
 
 
 class StreamPlan(C.Structure):
@@ -241,15 +245,17 @@ STREAM_MERGE_DTYPE = np.dtype([(n, np.uint32) for n in ("q_off", "batch", "head"
 STREAM_BLOCK_INDEX, STREAM_FIRST, STREAM_LAST = 0x0fffffff, 0x40000000, 0x80000000
 
 
-def build_stream(nn_lut, nb, batch, heads, block_size, lut_heads=1, wg_slots=None, level=True, tail_percent=0):
+def build_stream(nn_lut, nb, batch, heads, block_size, lut_heads=1, wg_slots=None, level=True, tail_percent=0,
+                 d=64, bf16=True, masked=False):
     """Streams of key blocks for the resident work-groups of a streamed launch (sfb_build_stream): dict(plan
     (StreamPlan), blob (uint8 array to copy to the device), slots / blocks / items / merges (views of the blob),
     lut_heads, lut_dim).  nn_lut: one table, or lut_heads tables of equal length concatenated.  wg_slots None: what
-    the device keeps resident (sfb_resident_work_groups)."""
+    the device keeps resident of the kernel that a launch with head size d, bf16 or fp32 tensors and (masked) an
+    element mask, key padding or log-sum-exp output runs (sfb_resident_work_groups_for)."""
     nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
     lut_dim = nn_lut.shape[0] // lut_heads
     if wg_slots is None:
-        wg_slots = resident_work_groups() or 1024
+        wg_slots = resident_work_groups(bf16, block_size, d, masked) or 1024
     plan = StreamPlan()
     args = (_np(nn_lut), nb, C.c_uint32(lut_heads), C.c_uint32(lut_dim), C.c_uint32(batch), C.c_uint32(heads),
             C.c_uint32(block_size), C.c_uint32(wg_slots), C.c_int(1 if level else 0), C.c_uint32(tail_percent))
@@ -271,7 +277,16 @@ def stream_workspace_bytes(stream, d):
 
 
 def stream_status(stream, d, workspace):
-    return int(lib.sfb_stream_status(C.byref(stream["plan"]), C.c_uint32(d), _dev(workspace)))
+    """0: every merge of the last launch found its records.  1: a bounded wait ran out; the workspace then holds
+    stale flags and is cleared here (sfb_stream_reset), so that it can be used again."""
+    status = int(lib.sfb_stream_status(C.byref(stream["plan"]), C.c_uint32(d), _dev(workspace)))
+    if status == 1:
+        stream_reset(stream, d, workspace)
+    return status
+
+
+def stream_reset(stream, d, workspace):
+    _check(lib.sfb_stream_reset(_stream(), C.byref(stream["plan"]), C.c_uint32(d), _dev(workspace)), "sfb_stream_reset")
 
 
 def schedule_workspace_bytes(sched, batch, heads, block_size, d):
@@ -844,12 +859,14 @@ class EncoderLayer:
         ws, aws = self._workspaces(B, L, x.device)
         if self.streamed:
             import torch
-            if B not in self._streams:
+            key = (B, mask is not None or valid_len is not None)   # the two kinds of launch run different kernels
+            if key not in self._streams:
                 st = build_stream(self.luts["nn_lut"], L // self.bs, B, self.heads, self.bs, lut_heads=self.lut_heads,
-                                  level=False)
-                self._streams[B] = (st, to_device(st["blob"]),
+                                  level=False, d=self.d, bf16=self.dtype == BF16,
+                                  masked=mask is not None or valid_len is not None)
+                self._streams[key] = (st, to_device(st["blob"]),
                                     torch.zeros(stream_workspace_bytes(st, self.d), dtype=torch.uint8, device=x.device))
-            st, blob, sws = self._streams[B]
+            st, blob, sws = self._streams[key]
             _check(lib.sfb_encoder_layer_forward_streamed(
                 _stream(), _dev(out), _dev(x), C.byref(self.c_weights), self.dtype, C.c_int(1 if self.pre_ln else 0),
                 _dev(self.nn_lut), _dev(mask), _dev(valid_len), C.byref(st["plan"]), _dev(blob), _dev(sws),

@@ -1277,6 +1277,12 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream
                              (uint8_t*)k_lds);
 }
 
+// Fill kernel (a captured graph must not hold a memset node): words[0 .. n) = 0.
+__global__ void clear_words_kernel(uint32_t* words, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) words[i] = 0u;
+}
+
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
@@ -1304,6 +1310,40 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
     else
         fused_attention_f32_kernel<BS, D><<<g, b, 0, stream>>>(p);
     return launch_status();
+}
+
+// Work-groups per compute unit the device keeps resident of the kernel a streamed launch of this kind runs (the
+// same choice as launch_fused makes); 0 if the runtime cannot say.
+template <int BS, int D>
+static int stream_kernel_occupancy(int in_dtype, bool masked) {
+    const void* kernel;
+    if (in_dtype == SFB_BF16) {
+        if constexpr (D == 64) {
+            kernel = masked ? (const void*)fused_attention_stream_bf16_kernel<BS, D, true>
+                            : (const void*)fused_attention_stream_bf16_kernel<BS, D, false>;
+        } else {
+            kernel = masked ? (const void*)fused_attention_stream_items_bf16_kernel<BS, D, true>
+                            : (const void*)fused_attention_stream_items_bf16_kernel<BS, D, false>;
+        }
+    } else {
+        kernel = (const void*)fused_attention_stream_f32_kernel<BS, D>;
+    }
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, BS * 2, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return per_cu;
+}
+template <int BS>
+static int stream_kernel_occupancy_any(int in_dtype, bool masked, uint32_t state_dim) {
+    switch (state_dim) {
+        case 64: return stream_kernel_occupancy<BS, 64>(in_dtype, masked);
+        case 32: return stream_kernel_occupancy<BS, 32>(in_dtype, masked);
+        case 96: return stream_kernel_occupancy<BS, 96>(in_dtype, masked);
+        case 128: return stream_kernel_occupancy<BS, 128>(in_dtype, masked);
+        default: return 0;
+    }
 }
 
 // head sizes 32, 64, 96 and 128 for both input types
@@ -1494,6 +1534,39 @@ extern "C" size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32
     return flags + (size_t)plan->n_parts * part + 256;   // the last 256 bytes hold the status word (at their end)
 }
 
+extern "C" uint32_t sfb_resident_work_groups_for(int in_dtype, uint32_t block_size, uint32_t state_dim, int masked) {
+    using namespace sfb;
+    if ((in_dtype != SFB_F32 && in_dtype != SFB_BF16) || (block_size != 32 && block_size != 64)) return 0;
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    const int per_cu = block_size == 64 ? stream_kernel_occupancy_any<64>(in_dtype, masked != 0, state_dim)
+                                        : stream_kernel_occupancy_any<32>(in_dtype, masked != 0, state_dim);
+    // (a runtime that cannot answer: what the kernels' registers and LDS allow by design)
+    return (uint32_t)(per_cu > 0 ? per_cu : (state_dim > 64 ? 2 : 4)) * (uint32_t)cus;
+}
+
+// bf16 tensors, blocks of 64, head size 64, no mask: the benched case
+extern "C" uint32_t sfb_resident_work_groups(void) { return sfb_resident_work_groups_for(SFB_BF16, 64, 64, 0); }
+
+extern "C" int sfb_stream_reset(sfb_stream_t stream, const sfb_stream_plan* plan, uint32_t state_dim, void* workspace) {
+    using namespace sfb;
+    if (!plan || !workspace) return SFB_ERR_NULL_POINTER;
+    if ((uintptr_t)workspace & 255u) return SFB_ERR_WORKSPACE;
+    const size_t need = sfb_stream_workspace_bytes(plan, state_dim);
+    const size_t flag_words = ((size_t)plan->n_parts * sizeof(uint32_t) + 255) / 256 * 64;
+    hipStream_t s = (hipStream_t)stream;
+    clear_stale_error();
+    if (flag_words > 0)
+        clear_words_kernel<<<dim3((unsigned)((flag_words + 255) / 256)), dim3(256), 0, s>>>((uint32_t*)workspace,
+                                                                                          (uint32_t)flag_words);
+    clear_words_kernel<<<dim3(1), dim3(64), 0, s>>>((uint32_t*)((uint8_t*)workspace + need - 256), 64u);
+    return launch_status();
+}
+
 extern "C" int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const void* workspace) {
     if (!plan || !workspace) return -1;
     uint32_t word = 0;
@@ -1573,12 +1646,6 @@ static int static_scratch(void** out) {
     }
     *out = scratch_ptr[device];
     return SFB_OK;
-}
-
-// Fill kernel (a captured graph must not hold a memset node): words[0 .. n) = 0.
-__global__ void clear_words_kernel(uint32_t* words, uint32_t n) {
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) words[i] = 0u;
 }
 
 }  // namespace sfb

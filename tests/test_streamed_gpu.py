@@ -15,7 +15,9 @@ THREADS = 16
 def run_streamed(Q, K, V, nn_lut, nb, bs, blocks, scale, bf16, level=True, lut_heads=1, mask=None, valid_len=None,
                  mask_heads=1, wg_slots=None, out_bf16=False, want_lse=False, launches=2):
     B, L, H, d = Q.shape
-    stream = sfb.build_stream(nn_lut, nb, B, H, bs, lut_heads=lut_heads, wg_slots=wg_slots, level=level)
+    masked = mask is not None or valid_len is not None or want_lse
+    stream = sfb.build_stream(nn_lut, nb, B, H, bs, lut_heads=lut_heads, wg_slots=wg_slots, level=level, d=d,
+                              bf16=bf16, masked=masked)
     ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
     q, k, v = (dev(x, bf16) for x in (Q, K, V))
     nn, blob = sfb.to_device(nn_lut), sfb.to_device(stream["blob"])
