@@ -214,6 +214,12 @@ int sfb_build_stream(sfb_stream_plan* plan, void* blob, size_t blob_bytes, const
  * the workspace must be cleared with sfb_stream_reset() before the next launch uses it, or that launch would add
  * records its producers have not written yet. */
 size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim);
+/* How the bf16 kernels apply `scale` in launches without mask, key padding and log-sum-exp output (host helper, no
+ * device needed): scale * log2(e) = *pow2 * *rest with *pow2 a power of two and *rest in [1/sqrt(2), sqrt(2)).  The
+ * queries are multiplied by *pow2, which is exact in bf16, so the score product delivers base-2 exponents up to the
+ * factor *rest, applied in fp32 per score: p = exp2((s - offset) * rest) follows ewops.h:86's exp((s - max) * scale)
+ * without a second rounding of the queries. */
+void sfb_scale_parts(float scale, float* pow2, float* rest);
 /* Clears the flags and the status word of a streamed launch's workspace (fill kernels on `stream`; the partial
  * records need no clearing).  Also usable instead of the initial zero-fill. */
 int sfb_stream_reset(sfb_stream_t stream, const sfb_stream_plan* plan, uint32_t state_dim, void* workspace);

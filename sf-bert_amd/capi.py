@@ -45,6 +45,7 @@ lib.sfb_status_string.restype = C.c_char_p
 lib.sfb_status_string.argtypes = [C.c_int]
 lib.sfb_count_blocks.restype = C.c_uint32
 lib.sfb_magicu64.restype = None
+lib.sfb_scale_parts.restype = None
 lib.sfb_schedule_workspace_bytes.restype = C.c_size_t
 lib.sfb_encoder_layer_workspace_bytes.restype = C.c_size_t
 lib.sfb_suggest_max_blocks.restype = C.c_uint32
@@ -66,7 +67,7 @@ EXPORTED = [
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
     "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_stream_reset", "sfb_resident_work_groups",
-    "sfb_resident_work_groups_for",
+    "sfb_resident_work_groups_for", "sfb_scale_parts",
     "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
@@ -270,6 +271,13 @@ def build_stream(nn_lut, nb, batch, heads, block_size, lut_heads=1, wg_slots=Non
                 blocks=view(plan.blocks_offset, plan.n_blocks, STREAM_BLOCK_DTYPE),
                 items=view(plan.items_offset, plan.n_items, STREAM_ITEM_DTYPE),
                 merges=view(plan.merges_offset, plan.n_merges, STREAM_MERGE_DTYPE))
+
+
+def scale_parts(scale):
+    """(pow2, rest) of sfb_scale_parts: scale * log2(e) = pow2 * rest."""
+    a, b = C.c_float(0), C.c_float(0)
+    lib.sfb_scale_parts(C.c_float(scale), C.byref(a), C.byref(b))
+    return a.value, b.value
 
 
 def stream_workspace_bytes(stream, d):

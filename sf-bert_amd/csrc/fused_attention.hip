@@ -51,6 +51,8 @@ struct FusedParams {
     uint32_t ranks;                 // work items per (batch, head)
     uint32_t heavy;                 // leading items issued for all heads first
     float scale_log2e;
+    float scale_pow2;               // scale_log2e = scale_pow2 * scale_rest, scale_pow2 a power of two (exact on bf16 queries),
+    float scale_rest;               //   scale_rest in [1/sqrt 2, sqrt 2)
     float slack;                    // raw-score distance a block maximum may exceed the reference maximum
 };
 
@@ -373,24 +375,25 @@ __device__ __forceinline__ void exp_chunk(const f32x16 (&s)[KT], uint32_t (&pk)[
     sum1 = dot2_bf16_ones(e, sum1);
 }
 
-// The same for scores that already are base-2 exponents (scale and offset folded into the score product): one
-// exponential per element and nothing else; the row sum is taken over the fp32 values with plain additions, which --
-// unlike v_dot2c -- run while the matrix pipe is busy.
+// The same for scores that carry the power-of-two part of the scale and the row's offset already (folded into the
+// score product): one multiplication by the rest of the scale and one exponential per element; the row sum is
+// taken over the fp32 values with plain additions, which -- unlike v_dot2c -- run while the matrix pipe is busy.
 template <int KT>
-__device__ __forceinline__ void exp_chunk_slim(const f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], int u, float& sum0,
+__device__ __forceinline__ void exp_chunk_slim(const f32x16 (&s)[KT], uint32_t (&pk)[KT * 8], int u, float r, float& sum0,
                                                float& sum1) {
     const int kt = u / 2, i0 = (u % 2) * 8;
-    const float p0 = exp2_fast(s[kt][i0 + 0]), p1 = exp2_fast(s[kt][i0 + 1]);
-    const float p2 = exp2_fast(s[kt][i0 + 2]), p3 = exp2_fast(s[kt][i0 + 3]);
-    const float p4 = exp2_fast(s[kt][i0 + 4]), p5 = exp2_fast(s[kt][i0 + 5]);
-    const float p6 = exp2_fast(s[kt][i0 + 6]), p7 = exp2_fast(s[kt][i0 + 7]);
+    const float p0 = exp2_fast(s[kt][i0 + 0] * r), p1 = exp2_fast(s[kt][i0 + 1] * r);
+    const float p2 = exp2_fast(s[kt][i0 + 2] * r), p3 = exp2_fast(s[kt][i0 + 3] * r);
+    const float p4 = exp2_fast(s[kt][i0 + 4] * r), p5 = exp2_fast(s[kt][i0 + 5] * r);
+    const float p6 = exp2_fast(s[kt][i0 + 6] * r), p7 = exp2_fast(s[kt][i0 + 7] * r);
     pk[u * 4 + 0] = pack_bf16(p0, p1); pk[u * 4 + 1] = pack_bf16(p2, p3);
     pk[u * 4 + 2] = pack_bf16(p4, p5); pk[u * 4 + 3] = pack_bf16(p6, p7);
     sum0 += (p0 + p2) + (p4 + p6);
     sum1 += (p1 + p3) + (p5 + p7);
 }
 
-// q * c, rounded to bf16 again (round to nearest even).
+// q * c as bf16 (round to nearest even).  The kernels call it with a power of two, for which the product is exact
+// (short of the exponent range's ends): the scores it leads to are then as exact as those of unscaled queries.
 __device__ __forceinline__ bf16x8 scale_bf16x8(bf16x8 q, float c) {
     const u32x4 bits = __builtin_bit_cast(u32x4, q);
     u32x4 out;
@@ -403,14 +406,14 @@ __device__ __forceinline__ bf16x8 scale_bf16x8(bf16x8 q, float c) {
 // The order in which the instructions of the chunks of one key block are to be issued (slim loop): the LDS reads of
 // chunk u + 1 ahead of the matrix instructions of chunk u, and behind every matrix instruction an equal share of the
 // vector work -- first the packing and adding of exponentials that were issued a slot earlier (their results are
-// ready by then), then the next exponentials.
+// ready by then) and the multiplications that feed the next exponentials, then those exponentials.
 template <int BS, int D>
 __device__ __forceinline__ void schedule_chunks() {
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, KPC = KS / PU;
     constexpr int MF = KPC * KT + NO;                    // matrix instructions per chunk
     constexpr int DS = KPC * KT + 2 * NO;                // LDS reads per chunk
     constexpr int EXP = BS / 2 / PU / MF;                // exponentials per slot (BS/2 elements per lane and key block)
-    constexpr int REST = (BS / 4 + BS / 2) / PU / MF;    // pack + add per slot
+    constexpr int REST = (BS / 4 + BS / 2 + BS / 2) / PU / MF;   // pack + add + multiply per slot
 #pragma unroll
     for (int u = 0; u < PU; ++u) {
         if (u + 1 < PU) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);
@@ -500,11 +503,14 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
 
     bf16x8 qf[KS];
     T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
+    const float c2 = p.scale_pow2, rest = p.scale_rest;
     if constexpr (SLIM) {
-        // the score product then delivers base-2 exponents; the second rounding of Q moves them by less than the
-        // rounding of the probabilities does
+        // The score product then delivers base-2 exponents up to the factor `rest`.  Only the power-of-two part of
+        // the scale goes into the queries: that product is exact, whereas rounding q * scale * log2(e) to bf16 a
+        // second time moves every exponent by up to 2^-9 of the products it is made of -- an error that grows with
+        // the scores and passes the tolerance for peaked rows (|score * scale| of a few tens).
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = scale_bf16x8(qf[ks], c);
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = scale_bf16x8(qf[ks], c2);
     }
     const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
 
@@ -529,7 +535,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     f32x16 off_vec;
     if constexpr (SLIM) {
         const float m_scaled = block_row_max<KT>(s_even);
-        st.m_used = st.m_true = m_scaled / c;
+        st.m_used = st.m_true = m_scaled / c2;
 #pragma unroll
         for (int i = 0; i < 16; ++i) off_vec[i] = -m_scaled;
 #pragma unroll
@@ -578,7 +584,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         float sum0 = 0.f, sum1 = 0.f;
         uint32_t pk[KT * 8];
         auto exps = [&](int u) {
-            if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, sum0, sum1);
+            if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, rest, sum0, sum1);
             else exp_chunk<KT, NO>(s, pk, u, c, mc, sum0, sum1);
         };
         // Every chunk carries the same work: the exponentials of the next chunk, one slice (KS / PU product steps) of
@@ -963,7 +969,7 @@ __device__ __forceinline__ void stream_items_bf16(const FusedParams& p, uint8_t*
     const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
     const uint32_t lds0 = T::lds_address(smem);
     const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
-    const float c = p.scale_log2e, slack = p.slack;
+    const float c = p.scale_log2e, slack = p.slack, c2 = p.scale_pow2, rest = p.scale_rest;
     const sfb_stream_block* const entries = (const sfb_stream_block*)(uintptr_t)blocks;
     auto q_row_of = [&](uint32_t q_off) { return Q + ((size_t)q_off + (size_t)q_in_block * p.heads) * D; };
     auto loads_landed = [&]() {
@@ -1020,7 +1026,7 @@ __device__ __forceinline__ void stream_items_bf16(const FusedParams& p, uint8_t*
             primed = true;
         }
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[ks] = SLIM ? scale_bf16x8(qf_next[ks], c) : qf_next[ks];
+        for (int ks = 0; ks < KS; ++ks) qf[ks] = SLIM ? scale_bf16x8(qf_next[ks], c2) : qf_next[ks];
         // the record and the queries of the next item
         const bool more = index + 1 < n_items;
         const StreamItem rec_next = stream_item<MASKED>(items, index + 1, n_items);
@@ -1092,7 +1098,7 @@ __device__ __forceinline__ void stream_items_bf16(const FusedParams& p, uint8_t*
             float sum0 = 0.f, sum1 = 0.f;
             uint32_t pk[KT * 8];
             auto exps = [&](int u) {
-                if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, sum0, sum1);
+                if constexpr (SLIM) exp_chunk_slim<KT>(s, pk, u, rest, sum0, sum1);
                 else exp_chunk<KT, NO>(s, pk, u, c, mc, sum0, sum1);
             };
             bf16x8 kfr[PU][KPC][KT], vfr[PU][NO];
@@ -1160,7 +1166,7 @@ __device__ __forceinline__ void stream_items_bf16(const FusedParams& p, uint8_t*
             if (__builtin_amdgcn_ballot_w64(!(total < 0x1p100f)) != 0 && lane == 0) *retry_flag = 1;   // overflow, or NaN
             __syncthreads();
             redo = __builtin_amdgcn_readfirstlane(*retry_flag) != 0;
-            st.m_used = st.m_true = m_item / c;
+            st.m_used = st.m_true = m_item / c2;
         }
         if (!redo) {
             pending = uni(stream_end_item<BS, D>(p, rec, o_acc, st.m_used, st.m_true, st.l, c, t));
@@ -1378,6 +1384,18 @@ static int check_common(const void* q, const void* k, const void* v, const void*
     return SFB_OK;
 }
 
+}  // namespace sfb
+
+extern "C" void sfb_scale_parts(float scale, float* pow2, float* rest) {
+    int e = 0;
+    const float mant = frexpf(scale * sfb::kLog2e, &e);      // scale * log2(e) = mant * 2^e, mant in [0.5, 1)
+    const bool up = mant >= 0.70710678f;                      // the nearest power of two in the logarithm
+    *pow2 = ldexpf(1.0f, up ? e : e - 1);
+    *rest = up ? mant : mant * 2.0f;
+}
+
+namespace sfb {
+
 static void fill_common(FusedParams& p, const void* q, const void* k, const void* v, void* o, int out_dtype,
                         const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
                         uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
@@ -1396,6 +1414,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
     p.groups = bh_groups(batch_dim * head_dim);
     p.scale_log2e = scale * kLog2e;
+    sfb_scale_parts(scale, &p.scale_pow2, &p.scale_rest);
     p.slack = kLazyRescaleLog2 / p.scale_log2e;
 }
 

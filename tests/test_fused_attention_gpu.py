@@ -351,6 +351,32 @@ def test_scale_and_large_scores():
         check(run_fused(Q, K, V, luts, bs, scale), want, TOL_F32)
 
 
+@pytest.mark.parametrize("qmul,scale", [(6.0, 0.125), (1.0, 1.0), (2.0, 1.0), (6.0, 1.0)])
+def test_large_scores_bf16(qmul, scale):
+    """Peaked rows with bf16 tensors, through the scheduled and the streamed launch without mask: |score * scale| of
+    30 to 90, exponents up to 2^85 above the offset of the row's first block, so the loop with the fixed offset is
+    what runs (the last case passes 2^100 and is redone by the loop that follows the maximum).  The error must not
+    grow with the scores: the scale's power-of-two part on the queries is exact and the rest is applied in fp32."""
+    bs, nb, B, H, d = 64, 8, 2, 3, 64
+    L = bs * nb
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    Q, K, V = qkv(B, L, H, d, seed=91)
+    Q, K, V = orc.round_bf16(Q * qmul), orc.round_bf16(K), orc.round_bf16(V)
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale)
+    got = run_fused(Q, K, V, luts, bs, scale, bf16=True, max_blocks=4)
+    err = rel_err(got, want)
+    q, k, v = (dev(x, True) for x in (Q, K, V))
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=16)
+    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    streamed = sfb.fused_attention_streamed(q, k, v, sfb.to_device(luts["nn_lut"]), sfb.to_device(stream["blob"]), stream,
+                                            ws, bs, luts["blocks"], scale)
+    torch.cuda.synchronize()
+    err_streamed = rel_err(streamed.cpu().numpy(), want)
+    print("scheduled %.3e, streamed %.3e" % (err, err_streamed), flush=True)
+    assert sfb.stream_status(stream, d, ws) == 0
+    assert err <= 0.75 * TOL_BF16 and err_streamed <= 0.75 * TOL_BF16
+
+
 def test_argument_errors():
     q = torch.zeros((1, 64, 1, 64), device="cuda")
     lut = sfb.to_device(np.zeros((3, 2), np.uint32))
