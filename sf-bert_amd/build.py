@@ -18,12 +18,15 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip"))) + sorted(glob.glob(os.path.join(CSRC, "*.cpp")))
 
 
-def build(verbose=True, jobs=8):
+def build(verbose=True, jobs=8, defines=(), lib=LIB, tag=""):
+    """defines / lib / tag: an experimental variant of the library built beside the product one (objects get the
+    tag in their names, the host programs are not rebuilt); loaded through the SFBERT_HIP_LIB environment variable."""
     objs, procs = [], []
     for src in sources():
-        obj = os.path.join(CSRC, os.path.basename(src) + ".o")
+        obj = os.path.join(CSRC, os.path.basename(src) + tag + ".o")
         objs.append(obj)
-        cmd = [HIPCC] + DEVICE_FLAGS + (["-x", "hip"] if src.endswith(".hip") else []) + ["-c", src, "-o", obj]
+        cmd = ([HIPCC] + DEVICE_FLAGS + ["-D" + d for d in defines] + (["-x", "hip"] if src.endswith(".hip") else []) +
+               ["-c", src, "-o", obj])
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
         while sum(p.poll() is None for _, p in procs) >= jobs:
             procs[0][1].wait()
@@ -34,11 +37,13 @@ def build(verbose=True, jobs=8):
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))
         if verbose and text.strip():
             print(text)
-    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-L/opt/rocm/lib", "-lrocblas", "-lhipblaslt"]
+    link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + objs + ["-L/opt/rocm/lib", "-lrocblas", "-lhipblaslt"]
     extra = [l for l in os.environ.get("SFB_EXTRA_LIBS", "").split() if l]
     subprocess.check_call(link + extra)
     if verbose:
-        print("built", LIB)
+        print("built", lib)
+    if lib != LIB:
+        return lib
     # C++ host program that drives the library through the reference-named launchers (run by the GPU tests)
     host = os.path.join(HERE, "host")
     exe = os.path.join(host, "attention_host_test")
@@ -59,5 +64,8 @@ def build(verbose=True, jobs=8):
 
 
 if __name__ == "__main__":
-    build()
+    if len(sys.argv) > 1:   # python build.py <tag> <define> ...: a variant library libsfbert_hip_<tag>.so
+        build(defines=sys.argv[2:], lib=os.path.join(HERE, "libsfbert_hip_%s.so" % sys.argv[1]), tag="." + sys.argv[1])
+    else:
+        build()
     sys.exit(0)

@@ -18,6 +18,10 @@
 #include "tiles.hip.h"
 
 #include <mutex>
+
+#ifndef SFB_TILE_LOAD_ONCE
+#define SFB_TILE_LOAD_ONCE 0   // 1: the fused bf16 kernel for head size 64 issues a tile's loads as one group (load_tile_once)
+#endif
 #include <type_traits>
 
 namespace sfb {
@@ -472,6 +476,14 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
     const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
     const typename T::Sources src = T::sources(lane, row_bytes);
+#if SFB_TILE_LOAD_ONCE
+    // experimental form of the tile loads (one M0 write and one scalar address per tile), head size 64 only
+    constexpr bool kOnce = D == 64;
+    typename T::OnceSources once;
+    if constexpr (kOnce) once = T::once_sources(lane, wave, row_bytes);
+#else
+    constexpr bool kOnce = false;
+#endif
     const uint32_t lds0 = T::lds_address(smem);
     // LUT entries of key blocks [win, win + 64) of this item, one per lane (clamped to the last one)
     uint32_t win = 0;
@@ -484,11 +496,20 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         const uint32_t jj = j < count ? j : count - 1;
         return __builtin_amdgcn_readlane(entries.y, jj - win);
     };
+    auto load_tile = [&](uint32_t dst, const uint8_t* g_tile) {
+#if SFB_TILE_LOAD_ONCE
+        if constexpr (kOnce) {
+            T::load_tile_once(dst, g_tile, wave, once, row_bytes);
+            return;
+        }
+#endif
+        T::load_tile_all(dst, g_tile, wave, src, row_bytes);
+    };
     auto load_k = [&](uint32_t j, uint32_t buf) {
-        T::load_tile_all(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes, wave, src, row_bytes);
+        load_tile(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes);
     };
     auto load_v = [&](uint32_t j, uint32_t buf) {
-        T::load_tile_all(lds0 + (2 + buf) * TILE, v_base + (size_t)column_of(j) * BS * row_bytes, wave, src, row_bytes);
+        load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)column_of(j) * BS * row_bytes);
     };
     auto loads_landed = [&]() {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -605,10 +626,15 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         };
         fragments(0);
         exps(0);
+        if constexpr (kOnce) {
+            load_tile(k_dst, k_src);
+            load_tile(v_dst, v_src);
+        } else {
 #pragma unroll
-        for (int i = 0; i < T::LOADS; ++i) {
-            T::load_rows_all(k_dst, k_src, i, wave, src, row_bytes);
-            T::load_rows_all(v_dst, v_src, i, wave, src, row_bytes);
+            for (int i = 0; i < T::LOADS; ++i) {
+                T::load_rows_all(k_dst, k_src, i, wave, src, row_bytes);
+                T::load_rows_all(v_dst, v_src, i, wave, src, row_bytes);
+            }
         }
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the tile loads are issued here, not later
 #pragma unroll

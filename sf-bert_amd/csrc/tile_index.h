@@ -61,6 +61,26 @@ struct TileIndex {
     static SFB_INDEX_FN uint32_t load_group_odd(int i, uint32_t wave) {
         return NW % 2 == 0 ? (wave & 1u) : ((uint32_t)i & 1u);   // an even number of waves: the parity is the wave's
     }
+    // A wave's LOADS loads of one slice issued as one group with a single LDS base: an LDS-direct load adds its
+    // instruction offset to the global address *and* to the LDS address (M0 + offset + 16 lane), so the step from
+    // one 8-row group to the wave's next (NW KiB in LDS) can ride in the instruction, with the lane's global offset
+    // making up the difference.  Load i then fetches from  base + once_lane_offset(i) + once_inst_offset(i)  into
+    // M0 + once_inst_offset(i) + 16 lane, where, relative to the slice's first source row and its LDS address,
+    //   base = wave * 8 * row_bytes + ONCE_CENTER,   M0 = wave * 1024 + ONCE_CENTER;
+    // ONCE_CENTER keeps the four instruction offsets inside the signed 13-bit field.  Only for whole slices in
+    // source-row order (8 * row_bytes >= 1024, so the lane offsets never go negative).
+    static constexpr int ONCE_CENTER = NW == 2 ? 4096 : 0;
+    static SFB_INDEX_FN int once_inst_offset(int i) { return i * NW * 1024 - ONCE_CENTER; }
+    static SFB_INDEX_FN uint32_t once_lane_offset(uint32_t lane, int i, uint32_t wave, uint32_t row_bytes) {
+        return lane_source(lane, load_group_odd(i, wave), row_bytes) + (uint32_t)(i * NW) * (8u * row_bytes - 1024u);
+    }
+    static SFB_INDEX_FN uint32_t once_base(uint32_t wave, uint32_t row_bytes) {
+        return wave * 8u * row_bytes + (uint32_t)ONCE_CENTER;
+    }
+    static SFB_INDEX_FN uint32_t once_m0(uint32_t wave) { return wave * 1024u + (uint32_t)ONCE_CENTER; }
+    static_assert(LOADS == 4 && (LOADS - 1) * NW * 1024 - ONCE_CENTER <= 4095 && -ONCE_CENTER >= -4096,
+                  "four loads per wave and slice, offsets of 13 signed bits");
+
     // Per-lane byte offset of the score fragment (16 bytes: 8 features of one row) of k-step 0 in row tile 0;
     // k-step ks (features 16 ks + 8 half ..) is at (base ^ (ks % 4) * 32) in slice ks / 4, row tile kt 4096 bytes on.
     static SFB_INDEX_FN uint32_t k_lane_base(uint32_t qn, uint32_t half) {

@@ -112,6 +112,38 @@ struct Bf16DirectTiles {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) load_rows(lds_tile, g_tile, i, wave, src_even, src_odd, row_bytes);
     }
+    // A wave's whole share of a one-slice tile as one group of loads: M0 is written once, the step from one 8-row
+    // group to the next rides in the instruction offsets (which go into the global and the LDS address alike) and
+    // the lanes' global offsets make up the difference (TileIndex::once_*).  Against load_tile that is one M0 write
+    // and one 64-bit scalar address per tile instead of four of each.  off[i] = once_lane_offset(lane, i, wave, ..).
+    struct OnceSources {
+        uint32_t off[I::LOADS];
+    };
+    static __device__ __forceinline__ OnceSources once_sources(uint32_t lane, uint32_t wave, uint32_t row_bytes) {
+        OnceSources s;
+#pragma unroll
+        for (int i = 0; i < I::LOADS; ++i) s.off[i] = I::once_lane_offset(lane, i, wave, row_bytes);
+        return s;
+    }
+    static __device__ __forceinline__ void load_tile_once(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
+                                                          const OnceSources& src, uint32_t row_bytes) {
+        static_assert(SLICES == 1 && !PARTIAL && I::LOADS == 4, "whole one-slice tiles");
+        const uint64_t ga = (uint64_t)(g_tile + I::once_base(wave, row_bytes));
+        const uint32_t ga_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(ga >> 32));
+        const uint32_t ga_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)ga);
+        const uint64_t base = ((uint64_t)ga_hi << 32) | (uint64_t)ga_lo;
+        const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane(lds_tile + I::once_m0(wave));
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %1, %5 offset:%6\n\t"
+                     "global_load_lds_dwordx4 %2, %5 offset:%7\n\t"
+                     "global_load_lds_dwordx4 %3, %5 offset:%8\n\t"
+                     "global_load_lds_dwordx4 %4, %5 offset:%9"
+                     :
+                     : "s"(m0), "v"(src.off[0]), "v"(src.off[1]), "v"(src.off[2]), "v"(src.off[3]), "s"(base),
+                       "n"(I::once_inst_offset(0)), "n"(I::once_inst_offset(1)), "n"(I::once_inst_offset(2)),
+                       "n"(I::once_inst_offset(3))
+                     : "memory");
+    }
     // Load number i of this wave's share of every slice of a tile.
     static __device__ __forceinline__ void load_rows_all(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                          const Sources& src, uint32_t row_bytes) {

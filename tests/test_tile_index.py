@@ -53,6 +53,17 @@ def fill_tile(ti, tensor, lds, lds_tile=0, by_halves=False):
                                             offsets, tensor.allowed)
 
 
+def fill_tile_once(ti, tensor, lds, lds_tile=0):
+    """What load_tile_once does: the four loads of a wave with one LDS base and the steps in the instruction offsets."""
+    assert ti.SLICES == 1 and not ti.PARTIAL
+    for wave in range(ti.NW):
+        for i in range(ti.LOADS):
+            offsets = [ti.once_lane_offset(lane, i, wave, tensor.row_bytes) for lane in range(64)]
+            lds.global_load_lds_dwordx4(lds_tile + ti.once_m0(wave), tensor.bytes,
+                                        tensor.tile_base + ti.once_base(wave, tensor.row_bytes), offsets,
+                                        tensor.allowed, inst_offset=ti.once_inst_offset(i))
+
+
 def check_fill(ti, lds, lds_tile=0):
     written = lds.writes[lds_tile:lds_tile + ti.TILE_BYTES]
     assert (written == 1).all(), "every byte of the tile is written exactly once"
@@ -123,6 +134,20 @@ def test_loaders_and_transposed_fragment_readers_agree(bs, d):
     lds = Lds(ti.TILE_BYTES)
     fill_tile(ti, tensor, lds)
     check_transposed_fragments(ti, lds, source_row=lambda r: r)
+
+
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("heads", [1, 3, 12])
+def test_one_lds_base_per_tile_fills_the_same_tile(bs, heads):
+    """The grouped form of the tile load (one M0 per tile, steps in the instruction offsets) leaves LDS exactly as
+    the one-M0-per-load form does, for the narrowest rows too."""
+    ti = TileIndex(bs, 64)
+    tensor = Tensor(bs, 64, heads=heads, head=heads // 2)
+    a, b = Lds(3 * ti.TILE_BYTES), Lds(3 * ti.TILE_BYTES)
+    fill_tile(ti, tensor, a, lds_tile=2 * ti.TILE_BYTES)
+    fill_tile_once(ti, tensor, b, lds_tile=2 * ti.TILE_BYTES)
+    assert np.array_equal(a.mem, b.mem) and np.array_equal(a.writes, b.writes)
+    check_score_fragments(ti, b, lds_tile=2 * ti.TILE_BYTES)
 
 
 def test_row_order_of_the_dsd_tile():

@@ -47,6 +47,7 @@ class _Names:
     ti_load_group = ti_load_group_odd = ti_k_lane_base = ti_k_frag_offset = ti_v_lane_base = ti_v_frag_offset = None
     ti_slab_passes = ti_sdd_wait_count = ti_sdd_wait_loads = ti_dsd_wait_count = ti_dsd_depth = None
     ti_dsd_p_loads = ti_dsd_v_loads = None
+    ti_once_inst_offset = ti_once_lane_offset = ti_once_base = ti_once_m0 = None
 
 
 class TileIndex:
@@ -78,6 +79,18 @@ class TileIndex:
     def load_group_odd(self, i, wave):
         return int(self._l.ti_load_group_odd(self.bs, self.d, i, wave))
 
+    def once_inst_offset(self, i):
+        return int(ctypes.c_int32(self._l.ti_once_inst_offset(self.bs, self.d, i)).value)
+
+    def once_lane_offset(self, lane, i, wave, row_bytes):
+        return int(self._l.ti_once_lane_offset(self.bs, self.d, lane, i, wave, row_bytes))
+
+    def once_base(self, wave, row_bytes):
+        return int(self._l.ti_once_base(self.bs, self.d, wave, row_bytes))
+
+    def once_m0(self, wave):
+        return int(self._l.ti_once_m0(self.bs, self.d, wave))
+
     def k_lane_base(self, qn, half):
         return int(self._l.ti_k_lane_base(self.bs, self.d, qn, half))
 
@@ -101,11 +114,13 @@ class Lds:
         self.mem = np.zeros(nbytes, np.uint8)
         self.writes = np.zeros(nbytes, np.int32)
 
-    def global_load_lds_dwordx4(self, m0, glob, base, lane_offsets, allowed):
-        """allowed: boolean array over glob's bytes -- the bytes this tile may read (its own rows)."""
-        assert len(lane_offsets) == 64
+    def global_load_lds_dwordx4(self, m0, glob, base, lane_offsets, allowed, inst_offset=0):
+        """allowed: boolean array over glob's bytes -- the bytes this tile may read (its own rows).  The instruction
+        offset (13 signed bits) goes into the global address and into the LDS address alike."""
+        assert len(lane_offsets) == 64 and -4096 <= inst_offset <= 4095 and 0 <= m0 < 65536
         for lane, off in enumerate(lane_offsets):
-            src, dst = base + off, m0 + 16 * lane
+            assert 0 <= off < 2 ** 32, "the lane offset is an unsigned 32-bit register"
+            src, dst = base + off + inst_offset, m0 + inst_offset + 16 * lane
             assert 0 <= src and src + 16 <= glob.size, "lane %d reads outside the allocation" % lane
             assert allowed[src:src + 16].all(), "lane %d reads bytes outside its row" % lane
             assert 0 <= dst and dst + 16 <= self.mem.size, "LDS destination outside the tile"

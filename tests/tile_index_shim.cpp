@@ -37,6 +37,12 @@ uint32_t ti_lane_source_by_halves(int bs, int d, uint32_t lane, uint32_t odd, ui
 }
 uint32_t ti_load_group(int bs, int d, int i, uint32_t wave) { DISPATCH(bs, d, I::load_group(i, wave)); }
 uint32_t ti_load_group_odd(int bs, int d, int i, uint32_t wave) { DISPATCH(bs, d, I::load_group_odd(i, wave)); }
+int ti_once_inst_offset(int bs, int d, int i) { DISPATCH(bs, d, I::once_inst_offset(i)); }
+uint32_t ti_once_lane_offset(int bs, int d, uint32_t lane, int i, uint32_t wave, uint32_t row_bytes) {
+    DISPATCH(bs, d, I::once_lane_offset(lane, i, wave, row_bytes));
+}
+uint32_t ti_once_base(int bs, int d, uint32_t wave, uint32_t row_bytes) { DISPATCH(bs, d, I::once_base(wave, row_bytes)); }
+uint32_t ti_once_m0(int bs, int d, uint32_t wave) { DISPATCH(bs, d, I::once_m0(wave)); }
 uint32_t ti_k_lane_base(int bs, int d, uint32_t qn, uint32_t half) { DISPATCH(bs, d, I::k_lane_base(qn, half)); }
 uint32_t ti_k_frag_offset(int bs, int d, uint32_t lane_base, int kt, int ks) {
     DISPATCH(bs, d, I::k_frag_offset(lane_base, kt, ks));
