@@ -131,6 +131,16 @@ typedef struct {
  * before the rest; always < n_items). */
 int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
                        uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks);
+/* The same for one layout per head (lut_heads tables of lut_dim entries, the reference's `fixed` pattern,
+ * fixed_fusion_test.cu:38-39): items [lut_heads][*n_items], every head's list longest first and filled up to the
+ * longest list's length with items whose row is SFB_WORK_ITEM_SKIP (no work).  A query call (items NULL) returns
+ * that length in *n_items; the filling call takes the stride of the array in *n_items and leaves it unchanged.
+ * n_slots and n_parts are the largest any head needs (the workspace is laid out per (batch, head)), n_heavy the
+ * number of leading ranks that are heavy in every head.  For sfb_fused_attention_scheduled_heads. */
+#define SFB_WORK_ITEM_SKIP 0xffffffffu
+int sfb_build_schedule_heads(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                             uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t lut_heads, uint32_t lut_dim,
+                             uint32_t max_blocks);
 /* MI355X addition: a max_blocks for sfb_build_schedule that suits a launch over batch_heads = batch x heads
  * (batch, head) pairs: 1.25 x the key blocks one of the device's 1024 resident work-group slots gets to process in
  * the whole launch, at least 16.  (BigBird L = 4096, 12 heads: 16 for one sequence, 19 for two, 37 -- global rows cut in
@@ -281,6 +291,16 @@ int sfb_fused_attention_scheduled_to(sfb_stream_t stream, const void* q, const v
                                   uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks,
                                   uint32_t head_dim, uint32_t state_dim, uint32_t mask_heads,
                                   float scale);
+/* sfb_fused_attention_scheduled_to with one look-up table (and work-item list) per head: nn_lut [dev] lut_heads
+ * tables of lut_dim = ctx_blks + blocks entries, items [dev] [lut_heads][n_items] from sfb_build_schedule_heads;
+ * lut_heads = head_dim (or 1, which is the plain scheduled launch); lse may be NULL. */
+int sfb_fused_attention_scheduled_heads(sfb_stream_t stream, const void* q, const void* k, const void* v, void* o,
+                                        float* lse, int in_dtype, int out_dtype, const sfb_uint2* nn_lut,
+                                        const void* mask, const int32_t* valid_len, const sfb_work_item* items,
+                                        uint32_t n_items, uint32_t n_heavy, uint32_t n_slots, uint32_t n_parts,
+                                        void* workspace, size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                        uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
+                                        uint32_t lut_heads, uint32_t lut_dim, uint32_t mask_heads, float scale);
 /* sfb_fused_attention_scheduled_to for Q, K and V whose token rows are token_stride elements apart instead of
  * head_dim * state_dim (o stays dense): q, k, v may then be column slices of one [batch * ctx, token_stride] matrix,
  * e.g. of the result of one merged Q/K/V projection (transformer.cpp:516-522 does three products).  token_stride >=

@@ -65,13 +65,13 @@ EXPORTED = [
     "sfb_layout_strided", "sfb_layout_bigbird", "sfb_bigbird_draw", "sfb_count_blocks",
     "sfb_build_nt_lut", "sfb_build_nn_lut", "sfb_build_rblk_lut", "sfb_build_tn_lut", "sfb_magicu64", "sfb_element_mask",
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
-    "sfb_build_schedule", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
+    "sfb_build_schedule", "sfb_build_schedule_heads", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
     "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_stream_reset", "sfb_resident_work_groups",
     "sfb_resident_work_groups_for", "sfb_scale_parts",
     "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
-    "sfb_fused_attention_scheduled_strided",
+    "sfb_fused_attention_scheduled_strided", "sfb_fused_attention_scheduled_heads",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
     "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
@@ -220,6 +220,46 @@ def build_schedule(nn_lut, nb, max_blocks=16):
                                   C.byref(n_parts), _np(nn_lut), nb, C.c_uint32(max_blocks)), "sfb_build_schedule")
     return Luts(items=items, n_items=int(n_items.value), n_heavy=int(n_heavy.value),
                 n_slots=int(n_slots.value), n_parts=int(n_parts.value))
+
+
+WORK_ITEM_SKIP = 0xFFFFFFFF
+
+
+def build_schedule_heads(nn_lut, nb, lut_heads, max_blocks=16):
+    """sfb_build_schedule_heads: one work-item list per head for lut_heads look-up tables of equal length
+    concatenated; dict(items structured array [lut_heads][n_items] (short lists filled with WORK_ITEM_SKIP rows),
+    n_items, n_heavy, n_slots, n_parts, lut_heads, lut_dim)."""
+    nn_lut = np.ascontiguousarray(nn_lut, np.uint32)
+    lut_dim = nn_lut.reshape(-1, 2).shape[0] // lut_heads
+    n_items, n_heavy, n_slots, n_parts = C.c_uint32(0), C.c_uint32(0), C.c_uint32(0), C.c_uint32(0)
+    args = (C.byref(n_items), C.byref(n_heavy), C.byref(n_slots), C.byref(n_parts), _np(nn_lut), nb,
+            C.c_uint32(lut_heads), C.c_uint32(lut_dim), C.c_uint32(max_blocks))
+    _check(lib.sfb_build_schedule_heads(None, *args), "sfb_build_schedule_heads")
+    items = np.zeros((lut_heads, n_items.value), WORK_ITEM_DTYPE)
+    _check(lib.sfb_build_schedule_heads(_np(items), *args), "sfb_build_schedule_heads")
+    return Luts(items=items, n_items=int(n_items.value), n_heavy=int(n_heavy.value), n_slots=int(n_slots.value),
+                n_parts=int(n_parts.value), lut_heads=int(lut_heads), lut_dim=int(lut_dim))
+
+
+def fused_attention_scheduled_heads(q, k, v, nn_lut, items, sched, workspace, block_size, blocks, scale, mask=None,
+                                    valid_len=None, mask_heads=1, out=None, lse=None):
+    """sfb_fused_attention_scheduled_heads over build_schedule_heads()'s per-head work items."""
+    import torch
+    B, L, H, d = q.shape
+    if out is None:
+        out = torch.empty((B, L, H, d), dtype=torch.float32, device=q.device)
+    for t in (q, k, v, out):
+        if not t.is_contiguous():
+            raise SfbError(4, "non-contiguous tensor")
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(lib.sfb_fused_attention_scheduled_heads(
+        _stream(), _dev(q), _dev(k), _dev(v), _dev(out), _dev(lse), _dtype_code(q), _dtype_code(out), _dev(nn_lut),
+        _dev(mask), _dev(valid_len), _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]),
+        C.c_uint32(sched["n_slots"]), C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes),
+        C.c_uint32(block_size), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(L // block_size), C.c_uint32(H),
+        C.c_uint32(d), C.c_uint32(sched["lut_heads"]), C.c_uint32(sched["lut_dim"]), C.c_uint32(mask_heads),
+        C.c_float(scale)), "sfb_fused_attention_scheduled_heads")
+    return out
 
 
 def resident_work_groups(bf16=True, block_size=64, d=64, masked=False):

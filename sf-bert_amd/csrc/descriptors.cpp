@@ -675,13 +675,11 @@ int sfb_build_stream(sfb_stream_plan* plan, void* blob, size_t blob_bytes, const
     return SFB_OK;
 }
 
-int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
-                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
-    if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
-    if (nb <= 0) return SFB_ERR_SHAPE;
-    if (max_blocks == 0) return SFB_ERR_ARGUMENT;
-    std::vector<sfb_work_item> all;
-    uint32_t slots = 0, parts = 0;
+// Work items of one layout, longest first; returns the number of leading "heavy" items.
+static uint32_t schedule_layout(std::vector<sfb_work_item>& all, uint32_t& slots, uint32_t& parts, const sfb_uint2* nn_lut,
+                                int nb, uint32_t max_blocks) {
+    all.clear();
+    slots = parts = 0;
     for (int r = 0; r < nb; ++r) {
         const uint32_t count = nn_lut[r].y;
         const uint32_t chunks = count > max_blocks ? (count + max_blocks - 1) / max_blocks : 1;
@@ -701,16 +699,60 @@ int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heav
     }
     std::stable_sort(all.begin(), all.end(),
                      [](const sfb_work_item& a, const sfb_work_item& b) { return a.count > b.count; });
-    if (items) {
-        if (*n_items < all.size()) return SFB_ERR_ARGUMENT;
-        std::copy(all.begin(), all.end(), items);
-    }
     // items at least twice as long as the median item are "heavy"
     const uint32_t median = all[all.size() / 2].count;
     uint32_t heavy = 0;
     while (heavy + 1 < all.size() && all[heavy].count >= 2 * median && all[heavy].count > median) ++heavy;
+    return heavy;
+}
+
+int sfb_build_schedule(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                       uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t max_blocks) {
+    if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
+    if (nb <= 0) return SFB_ERR_SHAPE;
+    if (max_blocks == 0) return SFB_ERR_ARGUMENT;
+    std::vector<sfb_work_item> all;
+    uint32_t slots = 0, parts = 0;
+    const uint32_t heavy = schedule_layout(all, slots, parts, nn_lut, nb, max_blocks);
+    if (items) {
+        if (*n_items < all.size()) return SFB_ERR_ARGUMENT;
+        std::copy(all.begin(), all.end(), items);
+    }
     *n_heavy = heavy;
     *n_items = (uint32_t)all.size();
+    *n_slots = slots;
+    *n_parts = parts;
+    return SFB_OK;
+}
+
+int sfb_build_schedule_heads(sfb_work_item* items, uint32_t* n_items, uint32_t* n_heavy, uint32_t* n_slots,
+                             uint32_t* n_parts, const sfb_uint2* nn_lut, int nb, uint32_t lut_heads, uint32_t lut_dim,
+                             uint32_t max_blocks) {
+    if (!n_items || !n_heavy || !n_slots || !n_parts || !nn_lut) return SFB_ERR_NULL_POINTER;
+    if (nb <= 0 || lut_heads == 0 || lut_dim < (uint32_t)nb) return SFB_ERR_SHAPE;
+    if (max_blocks == 0) return SFB_ERR_ARGUMENT;
+    std::vector<std::vector<sfb_work_item>> lists(lut_heads);
+    uint32_t longest = 0, heavy = 0xffffffffu, slots = 0, parts = 0;
+    for (uint32_t h = 0; h < lut_heads; ++h) {
+        uint32_t s = 0, p = 0;
+        const uint32_t hv = schedule_layout(lists[h], s, p, nn_lut + (size_t)h * lut_dim, nb, max_blocks);
+        longest = std::max<uint32_t>(longest, (uint32_t)lists[h].size());
+        heavy = std::min(heavy, hv);   // ranks that are long in every head
+        slots = std::max(slots, s);
+        parts = std::max(parts, p);
+    }
+    if (items) {
+        if (*n_items < longest) return SFB_ERR_ARGUMENT;
+        const sfb_work_item skip = {SFB_WORK_ITEM_SKIP, 0u, 0u, 1u, 0u, 0u, 0u, 0u};
+        for (uint32_t h = 0; h < lut_heads; ++h) {
+            sfb_work_item* out = items + (size_t)h * *n_items;
+            std::copy(lists[h].begin(), lists[h].end(), out);
+            std::fill(out + lists[h].size(), out + *n_items, skip);
+        }
+    } else {
+        *n_items = longest;
+    }
+    *n_heavy = heavy;
     *n_slots = slots;
     *n_parts = parts;
     return SFB_OK;

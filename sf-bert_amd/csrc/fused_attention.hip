@@ -50,6 +50,7 @@ struct FusedParams {
     uint32_t batch, heads, nb, blocks;
     uint32_t in_stride;             // elements between the rows of consecutive tokens in Q, K and V (heads * d when dense)
     uint32_t lut_stride;            // entries between heads' LUTs (0 = shared)
+    uint32_t item_stride;           // work items between heads' lists (0 = shared)
     uint32_t mask_stride;           // words between heads' masks (0 = shared)
     uint32_t groups;                // ceil(batch*heads / 8)
     uint32_t ranks;                 // work items per (batch, head)
@@ -84,7 +85,8 @@ __device__ __forceinline__ RowWork decode_row_work(const FusedParams& p) {
     w.b = __builtin_amdgcn_readfirstlane(id.bh / p.heads);
     w.h = __builtin_amdgcn_readfirstlane(id.bh % p.heads);
     if (p.items) {
-        const sfb_work_item it = p.items[id.rank];
+        const sfb_work_item it = p.items[(size_t)(id.valid ? w.h : 0u) * p.item_stride + id.rank];
+        if (it.row == SFB_WORK_ITEM_SKIP) w.valid = 0;   // filler of a head whose list is shorter than the longest
         w.row = it.row; w.first = it.first; w.count = it.count;
         w.nchunks = it.nchunks; w.slot = it.slot; w.part = it.part; w.chunk = it.chunk;
         w.lut_first = it.lut_first;
@@ -1437,6 +1439,7 @@ static void fill_common(FusedParams& p, const void* q, const void* k, const void
     p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
     p.in_stride = 0;   // set by the launcher: heads * d unless the caller gives a token stride
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
+    p.item_stride = 0;
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
     p.groups = bh_groups(batch_dim * head_dim);
     p.scale_log2e = scale * kLog2e;
@@ -1483,10 +1486,12 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
                                              uint32_t n_parts, void* workspace, size_t workspace_bytes,
                                              uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
                                              uint32_t ctx_blks, uint32_t head_dim, uint32_t state_dim,
-                                             uint32_t mask_heads, float scale, uint32_t token_stride = 0) {
+                                             uint32_t mask_heads, float scale, uint32_t token_stride = 0,
+                                             uint32_t lut_heads = 1, uint32_t lut_dim = 0) {
     using namespace sfb;
+    if (lut_heads <= 1) lut_dim = ctx_blks + blocks;
     const int rc = check_common(q, k, v, o, in_dtype, nn_lut, block_size, blocks, batch_dim, ctx_blks,
-                                head_dim, state_dim, 1, ctx_blks + blocks, mask_heads, scale);
+                                head_dim, state_dim, lut_heads, lut_dim, mask_heads, scale);
     if (rc != SFB_OK) return rc;
     if (out_dtype != SFB_F32 && out_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (!items) return SFB_ERR_NULL_POINTER;
@@ -1500,8 +1505,9 @@ static int fused_attention_scheduled(sfb_stream_t stream, const void* q, const v
         return SFB_ERR_WORKSPACE;
     FusedParams p;
     fill_common(p, q, k, v, o, out_dtype, nn_lut, mask, valid_len, block_size, blocks, batch_dim, ctx_blks, head_dim,
-                1, ctx_blks + blocks, mask_heads, scale);
+                lut_heads, lut_dim, mask_heads, scale);
     p.items = items;
+    p.item_stride = lut_heads > 1 ? n_items : 0;
     p.lse = lse;
     p.in_stride = token_stride;
     p.n_slots = n_slots; p.n_parts = n_parts; p.heavy = n_heavy;
@@ -1570,6 +1576,21 @@ extern "C" int sfb_fused_attention_scheduled_lse(sfb_stream_t stream, const void
     return fused_attention_scheduled(stream, q, k, v, o, lse, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
                                      n_items, n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
                                      batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale);
+}
+
+extern "C" int sfb_fused_attention_scheduled_heads(sfb_stream_t stream, const void* q, const void* k, const void* v,
+                                                   void* o, float* lse, int in_dtype, int out_dtype,
+                                                   const sfb_uint2* nn_lut, const void* mask, const int32_t* valid_len,
+                                                   const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                                                   uint32_t n_slots, uint32_t n_parts, void* workspace,
+                                                   size_t workspace_bytes, uint32_t block_size, uint32_t blocks,
+                                                   uint32_t batch_dim, uint32_t ctx_blks, uint32_t head_dim,
+                                                   uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim,
+                                                   uint32_t mask_heads, float scale) {
+    if (lut_heads == 0) return SFB_ERR_SHAPE;
+    return fused_attention_scheduled(stream, q, k, v, o, lse, in_dtype, out_dtype, nn_lut, mask, valid_len, items,
+                                     n_items, n_heavy, n_slots, n_parts, workspace, workspace_bytes, block_size, blocks,
+                                     batch_dim, ctx_blks, head_dim, state_dim, mask_heads, scale, 0, lut_heads, lut_dim);
 }
 
 extern "C" size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim) {

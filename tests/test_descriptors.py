@@ -176,6 +176,39 @@ def test_schedule_covers_every_block_once(max_blocks):
     assert nbytes == (4 * 12 * sched["n_slots"] * 4 + 255) // 256 * 256 + 4 * 12 * sched["n_parts"] * (64 * 64 + 256) * 4
 
 
+@pytest.mark.parametrize("max_blocks", [2, 5, 100])
+def test_schedule_per_head_is_each_heads_own_schedule(max_blocks):
+    """sfb_build_schedule_heads on the reference's per-head `fixed` pattern plus one head with emptied rows: every
+    head's list is what sfb_build_schedule makes of its table, filled up with skip items; counts are the maxima."""
+    H, nb = 4, 16
+    lay = sfb.layout_fixed(H, nb, 4, causal=True)
+    lay[2][3] = 0
+    lay[2][3][:9] = 1                      # one long row in one head only
+    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
+    width = max(len(p["nn_lut"]) for p in per_head)
+    nn = np.zeros((H, width, 2), np.uint32)
+    for h, p in enumerate(per_head):
+        nn[h, :len(p["nn_lut"])] = p["nn_lut"]
+    sched = sfb.build_schedule_heads(nn, nb, H, max_blocks)
+    singles = [sfb.build_schedule(nn[h], nb, max_blocks) for h in range(H)]
+    assert sched["lut_dim"] == width and sched["items"].shape == (H, sched["n_items"])
+    assert sched["n_items"] == max(s["n_items"] for s in singles)
+    assert sched["n_slots"] == max(s["n_slots"] for s in singles)
+    assert sched["n_parts"] == max(s["n_parts"] for s in singles)
+    assert sched["n_heavy"] == min(s["n_heavy"] for s in singles) < sched["n_items"]
+    for h, single in enumerate(singles):
+        mine = sched["items"][h]
+        assert np.array_equal(mine[:single["n_items"]], single["items"])
+        rest = mine[single["n_items"]:]
+        assert (rest["row"] == sfb.WORK_ITEM_SKIP).all() and (rest["count"] == 0).all()
+        assert (mine[:single["n_items"]]["row"] < nb).all()
+    if max_blocks == 5:
+        assert any(s["n_items"] < sched["n_items"] for s in singles), "the case has lists of different lengths"
+    # one table: the plain schedule
+    one = sfb.build_schedule_heads(nn[1], nb, 1, max_blocks)
+    assert np.array_equal(one["items"][0], singles[1]["items"])
+
+
 def check_stream(stream, luts_per_head, nb, B, H, bs):
     """Every key block of every (batch, head, row) appears exactly once, in LUT order inside its item; the flags,
     the item records, the partial records and the merge tasks are consistent."""

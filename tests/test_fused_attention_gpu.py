@@ -377,6 +377,43 @@ def test_large_scores_bf16(qmul, scale):
     assert err <= 0.75 * TOL_BF16 and err_streamed <= 0.75 * TOL_BF16
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+@pytest.mark.parametrize("bs", [32, 64])
+def test_scheduled_launch_with_per_head_tables(bf16, bs):
+    """The reference's `fixed` pattern gives every head its own layout (fixed_fusion_test.cu:38-39, 58-106): the
+    scheduled launch with one look-up table, one mask and one work-item list per head, rows cut in chunks of 2."""
+    nb, B, H, d = 16, 3, 4, 64
+    L = bs * nb
+    lay = sfb.layout_fixed(H, nb, 4, causal=True)
+    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
+    blocks = per_head[0]["blocks"]
+    assert all(p["blocks"] == blocks for p in per_head)
+    nn = np.concatenate([p["nn_lut"] for p in per_head])
+    masks = np.concatenate([sfb.pack_mask(sfb.element_mask(p["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG)) for p in per_head])
+    Q, K, V = qkv(B, L, H, d, seed=81, bf16=bf16)
+    q, k, v = (dev(x, bf16) for x in (Q, K, V))
+    tol = TOL_BF16 if bf16 else TOL_F32
+    for max_blocks in (2, 100):
+        sched = sfb.build_schedule_heads(nn, nb, H, max_blocks)
+        assert (sched["n_parts"] > 0) == (max_blocks == 2)
+        ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+        for mask in (masks, None):
+            want = orc.attention(Q, K, V, nn, bs, 0.125, mask=mask, lut_heads=H, mask_heads=H if mask is not None else 1,
+                                 blocks=blocks, nthreads=THREADS)
+            outs = []
+            for _ in range(2):   # the second launch finds the arrival counters as the first one left them
+                out = torch.full((B, L, H, d), 7.0, device="cuda")
+                sfb.fused_attention_scheduled_heads(q, k, v, sfb.to_device(nn), sfb.to_device(sched["items"]), sched, ws,
+                                                    bs, blocks, 0.125, mask=None if mask is None else sfb.to_device(mask),
+                                                    mask_heads=H if mask is not None else 1, out=out)
+                torch.cuda.synchronize()
+                outs.append(out.cpu().numpy())
+            assert np.array_equal(outs[0], outs[1])
+            diff = np.abs(outs[0].astype(np.float64) - want).max(axis=(0, 1, 3)) / np.abs(want).max()
+            print("max_blocks", max_blocks, "masked", mask is not None, "error per head", diff, flush=True)
+            assert diff.max() <= tol
+
+
 def test_argument_errors():
     q = torch.zeros((1, 64, 1, 64), device="cuda")
     lut = sfb.to_device(np.zeros((3, 2), np.uint32))
