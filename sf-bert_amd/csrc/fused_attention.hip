@@ -48,6 +48,7 @@ struct FusedParams {
     uint32_t n_slots, n_parts;
     uint32_t o_bf16;                // output element type: 0 fp32, 1 bf16 (rounded once from the fp32 result)
     uint32_t batch, heads, nb, blocks;
+    uint32_t state;                 // the tensors' head size; smaller than the kernel's (padded) one in ragged launches
     uint32_t in_stride;             // elements between the rows of consecutive tokens in Q, K and V (heads * d when dense)
     uint32_t lut_stride;            // entries between heads' LUTs (0 = shared)
     uint32_t item_stride;           // work items between heads' lists (0 = shared)
@@ -191,15 +192,32 @@ __device__ __forceinline__ float* output_row(const FusedParams& p, size_t elemen
 // L2.  (Streaming stores of the 32-byte pieces were slower than cached ones; of whole rows they are faster.)
 // o_row is this lane's own row, o_row_bytes the distance between the rows of consecutive queries; slab must hold
 // 32 * (row size + 16) bytes and be free of other users.
-template <int NO>
+// RAGGED (head sizes that are not a multiple of 32, computed by the kernel of the next multiple): only the first
+// `hd` columns exist in memory; they are stored straight from the accumulators, four at a time.
+template <int NO, bool RAGGED = false>
 __device__ __forceinline__ void store_output(float* o_row, uint32_t o_row_bytes, uint32_t as_bf16, float* lse_row,
                                              f32x16 (&o)[NO], float m_used, float m_true, float total, float c,
-                                             uint32_t lane, uint8_t* slab) {
+                                             uint32_t lane, uint8_t* slab, uint32_t hd = NO * 32) {
     constexpr int D = NO * 32;
     const uint32_t qn = lane & 31, half = lane >> 5;
     const float f = exp2_fast((m_true - m_used) * c);
     const float inv = 1.0f / (total + 1e-6f * f);
     if (lse_row != nullptr && half == 0) *lse_row = __builtin_fmaf(m_used, c, __builtin_log2f(total + 1e-6f * f));
+    if constexpr (RAGGED) {
+        for_each_out_vec<NO>([&](int mt, int ig) {
+            const uint32_t col = mt * 32 + ig * 8 + half * 4;
+            if (col >= hd) return;
+            const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
+                               o[mt][ig * 4 + 3] * inv};
+            if (as_bf16) {
+                const u32x2 packed = {pack_bf16(out.x, out.y), pack_bf16(out.z, out.w)};
+                *(u32x2*)((uint8_t*)o_row + col * 2) = packed;
+            } else {
+                *(f32x4*)(o_row + col) = out;
+            }
+        });
+        return;
+    }
     uint8_t* const wave_rows = (uint8_t*)o_row - (size_t)qn * o_row_bytes;   // row of the wave's first query
     const uint32_t pitch = as_bf16 ? D * 2 + 16 : D * 4 + 16;
     uint8_t* const mine = slab + qn * pitch;
@@ -257,28 +275,29 @@ __device__ __forceinline__ uint32_t partial_offset(int mt, int ig, uint32_t half
     return (((mt * 4 + ig) * 2 + half) * BS + q_in_block) * 4;
 }
 
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, uint32_t o_row_bytes,
                                                uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
-                                               uint32_t lane, uint8_t* slab);
+                                               uint32_t lane, uint8_t* slab, uint32_t hd = D);
 
 // End of a work item.  Unsplit rows are normalised and stored.  A chunk of a split row writes its
 // partial (unnormalised O, reference maximum, true maximum, sum) and bumps the row's counter; the
 // chunk that finds every other chunk already arrived merges all partials, stores O and resets the
 // counter for the next launch.  Nobody waits.  lds: shared memory of the work-group that nobody uses any more, at
 // least 32 * (row size + 16) bytes per wave (the output rows pass through it).
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& w, float* o_row,
                                            f32x16 (&o)[D / 32], const RowState& st, float c,
                                            uint32_t q_in_block, uint32_t half, uint32_t t, uint8_t* lds) {
-    const uint32_t lane = t & 63, o_row_bytes = p.heads * D * (p.o_bf16 ? 2u : 4u);
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t lane = t & 63, o_row_bytes = p.heads * hd * (p.o_bf16 ? 2u : 4u);
     uint8_t* const slab = lds + (t >> 6) * (32u * (D * 4 + 16));
     float* const lse_row = p.lse ? p.lse + ((size_t)w.bh * p.nb + w.row) * BS + q_in_block : nullptr;
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;   // floats per partial
     const float total = st.l + __shfl_xor(st.l, 32);
     if (w.nchunks <= 1) {
-        store_output<NO>(o_row, o_row_bytes, p.o_bf16, lse_row, o, st.m_used, st.m_true, total, c, lane, slab);
+        store_output<NO, RAGGED>(o_row, o_row_bytes, p.o_bf16, lse_row, o, st.m_used, st.m_true, total, c, lane, slab, hd);
         return;
     }
     float* base = p.partials + ((size_t)w.bh * p.n_parts + w.part) * PART;
@@ -304,15 +323,15 @@ __device__ __forceinline__ void finish_row(const FusedParams& p, const RowWork& 
     }
     __syncthreads();
     if (!last_flag) return;
-    merge_partials<BS, D>(base, w.nchunks, o_row, o_row_bytes, p.o_bf16, lse_row, c, q_in_block, lane, slab);
+    merge_partials<BS, D, RAGGED>(base, w.nchunks, o_row, o_row_bytes, p.o_bf16, lse_row, c, q_in_block, lane, slab, hd);
     if (t == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Merge of the partial records of a split row (run by the chunk that arrived last).
-template <int BS, int D>
+template <int BS, int D, bool RAGGED>
 __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchunks, float* o_row, uint32_t o_row_bytes,
                                                uint32_t as_bf16, float* lse_row, float c, uint32_t q_in_block,
-                                               uint32_t lane, uint8_t* slab) {
+                                               uint32_t lane, uint8_t* slab, uint32_t hd) {
     const uint32_t half = lane >> 5;
     constexpr int NO = D / 32;
     constexpr int PART = BS * D + 4 * BS;
@@ -343,7 +362,20 @@ __device__ __forceinline__ void merge_partials(const float* base, uint32_t nchun
             acc[mt][ig * 4 + 3] += hi.y * wgt;
         });
     }
-    store_output<NO>(o_row, o_row_bytes, as_bf16, lse_row, acc, m_used, m_true, sum, c, lane, slab);
+    store_output<NO, RAGGED>(o_row, o_row_bytes, as_bf16, lse_row, acc, m_used, m_true, sum, c, lane, slab, hd);
+}
+
+// the same for a row of hd elements (hd a multiple of 4): the two lanes of a query take alternate groups of 4
+__device__ __forceinline__ void store_zero_row_ragged(float* o_row, uint32_t as_bf16, uint32_t half, uint32_t hd) {
+    for (uint32_t col = half * 4; col < hd; col += 8) {
+        if (as_bf16) {
+            const u32x2 zero = {0u, 0u};
+            *(u32x2*)((uint8_t*)o_row + col * 2) = zero;
+        } else {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            *(f32x4*)(o_row + col) = zero;
+        }
+    }
 }
 
 template <int D>
@@ -451,7 +483,9 @@ __device__ __forceinline__ void schedule_chunks() {
 //
 // finish(o_acc, st) ends the item: it gets the unnormalised output accumulators and the row state (maxima in raw-score
 // units, this lane's part of the sum).
-template <int BS, int D, bool MASKED, bool SLIM, typename Finish>
+// RAGGED: the tensors' head size p.state is smaller than D (a multiple of 8 above D - 32): queries are padded with
+// zeros, the tiles' last slice holds filler beyond the row's features, only p.state output columns are stored.
+template <int BS, int D, bool MASKED, bool SLIM, bool RAGGED = false, typename Finish>
 __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const RowWork& w, uint8_t* smem, uint32_t* retry_flag,
                                                  sfb_uint2 first_window, Finish&& finish) {
     using T = Bf16DirectTiles<BS, D>;
@@ -459,28 +493,30 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     constexpr int TILE = T::TILE_BYTES;
     constexpr int SC = PU >= 2 ? PU / 2 : 1;   // chunks that carry a slice of the next block's scores
     static_assert(!(MASKED && SLIM), "masked launches take the general loop");
+    static_assert(!(RAGGED && SLIM), "ragged head sizes take the general loop");
 
     const uint32_t L = p.nb * BS;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
     const uint32_t row_bytes = p.in_stride * 2;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
 
     const uint32_t count = __builtin_amdgcn_readfirstlane(w.count);
-    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, hd));
 
     const __bf16* Q = (const __bf16*)p.q;
     const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)w.h * p.mask_stride * (BS / 8) : nullptr;
     const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
 
     // byte address of (b, token 0, h, 0) in K and V; key block column col starts col*BS rows further
-    const size_t bh_bytes = input_offset(p, w.b, 0, w.h, L, D) * 2;
+    const size_t bh_bytes = input_offset(p, w.b, 0, w.h, L, hd) * 2;
     const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
     const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
-    const typename T::Sources src = T::sources(lane, row_bytes);
+    const typename T::Sources src = RAGGED ? T::sources_ragged(lane, row_bytes, hd) : T::sources(lane, row_bytes);
 #if SFB_TILE_LOAD_ONCE
     // experimental form of the tile loads (one M0 write and one scalar address per tile), head size 64 only
-    constexpr bool kOnce = D == 64;
+    constexpr bool kOnce = D == 64 && !RAGGED;
     typename T::OnceSources once;
     if constexpr (kOnce) once = T::once_sources(lane, wave, row_bytes);
 #else
@@ -505,7 +541,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
             return;
         }
 #endif
-        T::load_tile_all(dst, g_tile, wave, src, row_bytes);
+        T::template load_tile_all<RAGGED>(dst, g_tile, wave, src, row_bytes);
     };
     auto load_k = [&](uint32_t j, uint32_t buf) {
         load_tile(lds0 + buf * TILE, k_base + (size_t)column_of(j) * BS * row_bytes);
@@ -525,7 +561,8 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     const float c = p.scale_log2e, slack = p.slack;
 
     bf16x8 qf[KS];
-    T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
+    if constexpr (RAGGED) T::load_q_ragged(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, hd), half, hd);
+    else T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
     const float c2 = p.scale_pow2, rest = p.scale_rest;
     if constexpr (SLIM) {
         // The score product then delivers base-2 exponents up to the factor `rest`.  Only the power-of-two part of
@@ -634,8 +671,8 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         } else {
 #pragma unroll
             for (int i = 0; i < T::LOADS; ++i) {
-                T::load_rows_all(k_dst, k_src, i, wave, src, row_bytes);
-                T::load_rows_all(v_dst, v_src, i, wave, src, row_bytes);
+                T::template load_rows_all<RAGGED>(k_dst, k_src, i, wave, src, row_bytes);
+                T::template load_rows_all<RAGGED>(v_dst, v_src, i, wave, src, row_bytes);
             }
         }
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the tile loads are issued here, not later
@@ -687,7 +724,7 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
     return true;
 }
 
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_bf16_kernel(FusedParams p) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int TILE = T::TILE_BYTES;
@@ -699,27 +736,29 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_bf16_k
     const RowWork w = decode_row_work(p);
     if (!w.valid) return;
     const uint32_t L = p.nb * BS, q_in_block = (threadIdx.x >> 6) * 32 + (lane & 31);
-    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, hd));
     if (w.count == 0) {
-        store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
+        if constexpr (RAGGED) store_zero_row_ragged(o_row, p.o_bf16, lane >> 5, hd);
+        else store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
         if (p.lse && (lane >> 5) == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
         return;
     }
     const sfb_uint2 window = lut_window(p, w, 0, lane);
     auto finish = [&](f32x16 (&o_acc)[D / 32], const RowState& st) {
-        finish_row<BS, D>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, threadIdx.x, smem);
+        finish_row<BS, D, RAGGED>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, threadIdx.x, smem);
     };
-    if constexpr (!MASKED) {
+    if constexpr (!MASKED && !RAGGED) {
         if (attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window, finish)) return;
     }
-    attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window, finish);
+    attend_item_bf16<BS, D, MASKED, false, RAGGED>(p, w, smem, &retry_flag, window, finish);
 }
 
 // ------------------------------------------------------------------------------------------------
 // fp32 inputs: v_mfma_f32_32x32x2_f32 (true fp32 products and accumulation)
 // ------------------------------------------------------------------------------------------------
 // One LDS buffer (K tile and V tile); the next block waits in registers.
-template <int BS, int D, typename Finish>
+template <int BS, int D, bool RAGGED = false, typename Finish>
 __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowWork& w, float* k_lds, float* v_lds,
                                                 Finish&& finish) {
     using T = F32Tiles<BS, D>;
@@ -731,13 +770,15 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
     const uint32_t row_stride = p.in_stride;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
 
     const sfb_uint2* lut = p.nn_lut + (size_t)w.h * p.lut_stride;
     const uint32_t lut_off = w.lut_first, count = w.count;
-    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, D));
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, L, p.heads, hd));
 
     if (count == 0) {
-        store_zero_row<D>(o_row, p.o_bf16, half);
+        if constexpr (RAGGED) store_zero_row_ragged(o_row, p.o_bf16, half, hd);
+        else store_zero_row<D>(o_row, p.o_bf16, half);
         if (p.lse && half == 0) p.lse[((size_t)w.bh * p.nb + w.row) * BS + q_in_block] = 0.f;
         return;
     }
@@ -749,7 +790,8 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
     const int valid = p.valid_len ? p.valid_len[w.b] : (int)L;
 
     f32x4 qf[QG];
-    T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
+    if constexpr (RAGGED) T::load_q_ragged(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, hd), half, hd);
+    else T::load_q(qf, Q + input_offset(p, w.b, w.row * BS + q_in_block, w.h, L, D), half);
 
     typename T::Regs gk, gv;
 
@@ -763,9 +805,14 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
 
     sfb_uint2 entry = lut[lut_off];
     {
-        const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, D);
-        T::fetch(gk, K, base, row_stride, t);
-        T::fetch(gv, V, base, row_stride, t);
+        const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, hd);
+        if constexpr (RAGGED) {
+            T::fetch_ragged(gk, K, base, row_stride, t, hd);
+            T::fetch_ragged(gv, V, base, row_stride, t, hd);
+        } else {
+            T::fetch(gk, K, base, row_stride, t);
+            T::fetch(gv, V, base, row_stride, t);
+        }
     }
 
     for (uint32_t j = 0; j < count; ++j) {
@@ -775,9 +822,14 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
         __syncthreads();
         if (j + 1 < count) {
             entry = lut[lut_off + j + 1];
-            const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, D);
-            T::fetch(gk, K, base, row_stride, t);
-            T::fetch(gv, V, base, row_stride, t);
+            const size_t base = input_offset(p, w.b, entry.y * BS, w.h, L, hd);
+            if constexpr (RAGGED) {
+                T::fetch_ragged(gk, K, base, row_stride, t, hd);
+                T::fetch_ragged(gv, V, base, row_stride, t, hd);
+            } else {
+                T::fetch(gk, K, base, row_stride, t);
+                T::fetch(gv, V, base, row_stride, t);
+            }
         }
 
         f32x16 s[KT];
@@ -817,7 +869,7 @@ __device__ __forceinline__ void attend_item_f32(const FusedParams& p, const RowW
     finish(o_acc, st);
 }
 
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_kernel(FusedParams p) {
     using T = F32Tiles<BS, D>;
     __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
@@ -826,9 +878,9 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_f32_ke
     const RowWork w = decode_row_work(p);
     if (!w.valid) return;
     const uint32_t t = threadIdx.x, lane = t & 63, q_in_block = (t >> 6) * 32 + (lane & 31);
-    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, p.nb * BS, p.heads, D));
-    attend_item_f32<BS, D>(p, w, k_lds, v_lds, [&](f32x16 (&o_acc)[D / 32], const RowState& st) {
-        finish_row<BS, D>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, t, (uint8_t*)k_lds);
+    float* o_row = output_row(p, token_offset(w.b, w.row * BS + q_in_block, w.h, p.nb * BS, p.heads, RAGGED ? p.state : (uint32_t)D));
+    attend_item_f32<BS, D, RAGGED>(p, w, k_lds, v_lds, [&](f32x16 (&o_acc)[D / 32], const RowState& st) {
+        finish_row<BS, D, RAGGED>(p, w, o_row, o_acc, st, p.scale_log2e, q_in_block, lane >> 5, t, (uint8_t*)k_lds);
     });
 }
 
@@ -1317,6 +1369,12 @@ __global__ void clear_words_kernel(uint32_t* words, uint32_t n) {
     if (i < n) words[i] = 0u;
 }
 
+// Head sizes the fused forward takes: rows of whole 16-byte vectors, at most 128 features.
+static bool head_size_supported(int in_dtype, uint32_t state_dim) {
+    const uint32_t granule = in_dtype == SFB_BF16 ? 8u : 4u;
+    return state_dim >= granule && state_dim <= 128 && state_dim % granule == 0;
+}
+
 template <int BS, int D>
 static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
     p.ranks = ranks;
@@ -1380,16 +1438,39 @@ static int stream_kernel_occupancy_any(int in_dtype, bool masked, uint32_t state
     }
 }
 
-// head sizes 32, 64, 96 and 128 for both input types
+// Head sizes that are not a multiple of 32 (the reference's kernels take any multiple of 4,
+// openai_blocksparse.h:221-222): the kernel of the next multiple of 32 with zero-padded queries, the general loop
+// only.  Plain and scheduled launches; streamed ones do not take them.
+template <int BS, int D>
+static int launch_fused_ragged(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
+    if (p.st_slots != nullptr) return SFB_ERR_HEAD_STATE;
+    p.ranks = ranks;
+    clear_stale_error();
+    const dim3 g(p.groups * 8u * ranks), b(BS * 2);
+    if (in_dtype == SFB_BF16) fused_attention_bf16_kernel<BS, D, true, true><<<g, b, 0, stream>>>(p);
+    else fused_attention_f32_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
+    return launch_status();
+}
+
+// head sizes 32, 64, 96 and 128 for both input types; other multiples of 8 (bf16) or 4 (fp32) up to 128 through
+// the padded kernels
 template <int BS>
 static int launch_fused_any(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks, uint32_t state_dim) {
     if (p.in_stride == 0) p.in_stride = p.heads * state_dim;
+    p.state = state_dim;
     switch (state_dim) {
         case 64: return launch_fused<BS, 64>(stream, p, in_dtype, ranks);
         case 32: return launch_fused<BS, 32>(stream, p, in_dtype, ranks);
         case 96: return launch_fused<BS, 96>(stream, p, in_dtype, ranks);
         case 128: return launch_fused<BS, 128>(stream, p, in_dtype, ranks);
-        default: return SFB_ERR_HEAD_STATE;
+        default: break;
+    }
+    if (!head_size_supported(in_dtype, state_dim)) return SFB_ERR_HEAD_STATE;
+    switch ((state_dim + 31) / 32) {
+        case 1: return launch_fused_ragged<BS, 32>(stream, p, in_dtype, ranks);
+        case 2: return launch_fused_ragged<BS, 64>(stream, p, in_dtype, ranks);
+        case 3: return launch_fused_ragged<BS, 96>(stream, p, in_dtype, ranks);
+        default: return launch_fused_ragged<BS, 128>(stream, p, in_dtype, ranks);
     }
 }
 
@@ -1400,7 +1481,7 @@ static int check_common(const void* q, const void* k, const void* v, const void*
     if (!q || !k || !v || !o || !nn_lut) return SFB_ERR_NULL_POINTER;
     if (in_dtype != SFB_F32 && in_dtype != SFB_BF16) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 32 && state_dim != 64 && state_dim != 96 && state_dim != 128) return SFB_ERR_HEAD_STATE;
+    if (!head_size_supported(in_dtype, state_dim)) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (batch_dim == 0 || ctx_blks == 0 || head_dim == 0 || lut_heads == 0 || mask_heads == 0)
         return SFB_ERR_SHAPE;
@@ -1474,7 +1555,8 @@ extern "C" size_t sfb_schedule_workspace_bytes(uint32_t n_slots, uint32_t n_part
                                                uint32_t state_dim) {
     const size_t bh = (size_t)batch_dim * head_dim;
     const size_t counters = (bh * n_slots * sizeof(uint32_t) + 255) / 256 * 256;
-    const size_t part = ((size_t)block_size * state_dim + 4 * (size_t)block_size) * sizeof(float);
+    const size_t padded = ((size_t)state_dim + 31) / 32 * 32;   // records have the layout of the kernel that writes them
+    const size_t part = ((size_t)block_size * padded + 4 * (size_t)block_size) * sizeof(float);
     return counters + bh * n_parts * part;
 }
 

@@ -46,6 +46,15 @@ struct TileIndex {
         const uint32_t rr = lane >> 3, pos = lane & 7u;
         return rr * row_bytes + (((pos ^ swz(8u * odd + rr)) & 3u) << 4);
     }
+    // The same for a last slice of which only the first nch chunks (1..8) exist in memory -- head sizes that are not
+    // a multiple of 32, run through the kernel of the next multiple: positions whose chunk would lie beyond the row
+    // fetch chunk (pos ^ swz) % nch instead (finite filler the readers multiply by zero queries or never store).
+    static SFB_INDEX_FN uint32_t lane_source_ragged(uint32_t lane, uint32_t odd, uint32_t row_bytes, uint32_t nch) {
+        const uint32_t rr = lane >> 3, pos = lane & 7u, x = pos ^ swz(8u * odd + rr);
+        return rr * row_bytes + ((x < nch ? x : x % nch) << 4);
+    }
+    // Chunks of the last slice that a head size of hd features (a multiple of 8, SLICES slices) has in memory.
+    static SFB_INDEX_FN uint32_t last_slice_chunks(uint32_t hd) { return (hd - 64u * (uint32_t)(SLICES - 1)) / 8u; }
     // The same for a tile whose LDS rows hold the source rows in the order that makes the 8 k-slots of a lane in
     // the second product, rows 16u + 8(j/4) + 4*half + j%4 of the tile, the 8 consecutive source rows
     // 32*half + 8u + j: LDS row 16u + 8a + 4h + c holds source row 32h + 8u + 4a + c, which is 4n + 32(rr/4) + rr%4

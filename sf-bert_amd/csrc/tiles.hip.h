@@ -76,6 +76,17 @@ struct Bf16DirectTiles {
         s.odd_part = PARTIAL ? lane_source_part(lane, 1, row_bytes) : s.odd;
         return s;
     }
+    // Sources for tensors whose head size hd (a multiple of 8, more than D - 32) is smaller than D: the last slice's
+    // lanes stay inside the hd features of their rows (TileIndex::lane_source_ragged).  Used with
+    // load_rows_all<true> / load_tile_all<true>, which treat the last slice as the partial one whatever D is.
+    static __device__ __forceinline__ Sources sources_ragged(uint32_t lane, uint32_t row_bytes, uint32_t hd) {
+        Sources s;
+        s.even = lane_source(lane, 0, row_bytes);
+        s.odd = lane_source(lane, 1, row_bytes);
+        s.even_part = I::lane_source_ragged(lane, 0, row_bytes, I::last_slice_chunks(hd));
+        s.odd_part = I::lane_source_ragged(lane, 1, row_bytes, I::last_slice_chunks(hd));
+        return s;
+    }
     // The same for a tile whose LDS rows hold the source rows in the order that makes the 8 k-slots of a lane
     // in the second product 8 consecutive source rows.  Used with load_rows<4>: the group's base advances by 4
     // source rows.
@@ -145,19 +156,21 @@ struct Bf16DirectTiles {
                      : "memory");
     }
     // Load number i of this wave's share of every slice of a tile.
+    template <bool RAGGED = false>
     static __device__ __forceinline__ void load_rows_all(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,
                                                          const Sources& src, uint32_t row_bytes) {
 #pragma unroll
         for (int f = 0; f < SLICES; ++f) {
-            const bool part = PARTIAL && f == SLICES - 1;
+            const bool part = (PARTIAL || RAGGED) && f == SLICES - 1;
             load_rows(lds_tile + f * SLICE_BYTES, g_tile + f * 128, i, wave, part ? src.even_part : src.even,
                       part ? src.odd_part : src.odd, row_bytes);
         }
     }
+    template <bool RAGGED = false>
     static __device__ __forceinline__ void load_tile_all(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
                                                          const Sources& src, uint32_t row_bytes) {
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) load_rows_all(lds_tile, g_tile, i, wave, src, row_bytes);
+        for (int i = 0; i < LOADS; ++i) load_rows_all<RAGGED>(lds_tile, g_tile, i, wave, src, row_bytes);
     }
     // with src_even / src_odd from lane_source_by_halves()
     static __device__ __forceinline__ void load_tile_by_halves(uint32_t lds_tile, const uint8_t* g_tile, uint32_t wave,
@@ -194,6 +207,16 @@ struct Bf16DirectTiles {
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) qf[ks] = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
     }
+    // a row of hd < D features: the missing ones are zeros, so whatever the K tile holds in their place drops out
+    static __device__ __forceinline__ void load_q_ragged(bf16x8 (&qf)[D / 16], const __bf16* q_row, uint32_t half,
+                                                         uint32_t hd) {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ++ks) {
+            const uint32_t first = (2 * ks + half) * 8;
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            qf[ks] = first < hd ? *(const bf16x8*)(q_row + first) : __builtin_bit_cast(bf16x8, zero);
+        }
+    }
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -223,6 +246,16 @@ struct F32Tiles {
             r.g[i] = *(const f32x4*)(X + base + (size_t)(row * row_stride + cc * 4));
         }
     }
+    // rows of hd < D floats (hd a multiple of 4): the missing chunks are zeros and nothing beyond the row is read
+    static __device__ __forceinline__ void fetch_ragged(Regs& r, const float* X, size_t base, uint32_t row_stride,
+                                                        uint32_t t, uint32_t hd) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const uint32_t cid = i * NT + t, row = cid / (D / 4), cc = cid % (D / 4);
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            r.g[i] = cc * 4 < hd ? *(const f32x4*)(X + base + (size_t)(row * row_stride + cc * 4)) : zero;
+        }
+    }
     template <int STRIDE>
     static __device__ __forceinline__ void stage(float* lds, const Regs& r, uint32_t t) {
 #pragma unroll
@@ -243,6 +276,14 @@ struct F32Tiles {
     static __device__ __forceinline__ void load_q(f32x4 (&qf)[D / 8], const float* q_row, uint32_t half) {
 #pragma unroll
         for (int g = 0; g < D / 8; ++g) qf[g] = *(const f32x4*)(q_row + 8 * g + 4 * half);
+    }
+    static __device__ __forceinline__ void load_q_ragged(f32x4 (&qf)[D / 8], const float* q_row, uint32_t half,
+                                                         uint32_t hd) {
+#pragma unroll
+        for (int g = 0; g < D / 8; ++g) {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            qf[g] = 8 * g + 4 * half < hd ? *(const f32x4*)(q_row + 8 * g + 4 * half) : zero;
+        }
     }
 };
 

@@ -227,6 +227,52 @@ def test_head_sizes_other_than_64(d, bs, bf16):
         check(out.cpu().numpy(), ref, tol)
 
 
+@pytest.mark.parametrize("d,bf16", [(16, True), (48, True), (80, True), (112, True), (40, True), (8, True), (120, True),
+                                    (16, False), (48, False), (80, False), (112, False), (36, False), (4, False),
+                                    (100, False)])
+@pytest.mark.parametrize("bs", [32, 64])
+def test_head_sizes_that_are_not_multiples_of_32(d, bs, bf16):
+    """The reference's K64 = false kernels take any head size that is a multiple of 4 (openai_blocksparse.h:221-222).
+    Here: multiples of 4 (fp32) or 8 (bf16 -- rows of whole 16-byte vectors) up to 128, through the kernel of the
+    next multiple of 32 with zero-padded queries; plain and scheduled launches, with and without mask and padding,
+    a row without blocks, split rows merged from partial records, bf16 output, log-sum-exp output."""
+    nb, B, H = 8, 2, 3
+    L = nb * bs
+    tol = TOL_BF16 if bf16 else TOL_F32
+    lay = PATTERNS["bigbird"](nb)
+    lay[5] = 0
+    luts = sfb.build_luts(lay)
+    keep = (np.random.default_rng(d).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
+    mask = sfb.pack_mask(keep)
+    valid = np.array([L, L - bs - 5], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=3 * d + bs, bf16=bf16)
+    scale = float(1.0 / np.sqrt(d))
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, mask=mask, valid_len=valid, nthreads=THREADS)
+    plain = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, nthreads=THREADS)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid), want, tol)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid, max_blocks=3), want, tol)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16), plain, tol)
+    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, max_blocks=3), plain, tol)
+    q, k, v = (dev(x, bf16) for x in (Q, K, V))
+    sched = sfb.build_schedule(luts["nn_lut"], nb, 3)
+    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+    nn, items = sfb.to_device(luts["nn_lut"]), sfb.to_device(sched["items"])
+    if d % 8 == 0:
+        o16 = sfb.fused_attention_scheduled(q, k, v, nn, items, sched, ws, bs, luts["blocks"], scale, out_dtype=sfb.BF16)
+        torch.cuda.synchronize()
+        assert rel_err(o16.float().cpu().numpy(), plain) <= max(tol, 2.0 ** -7)
+    o32, lse = sfb.fused_attention_forward_lse(q, k, v, nn, items, sched, ws, bs, luts["blocks"], scale)
+    torch.cuda.synchronize()
+    check(o32.cpu().numpy(), plain, tol)
+    assert torch.isfinite(lse).all() and float(lse[:, :, 5 * bs:6 * bs].abs().max()) == 0.0
+    # streamed launches do not take these sizes: a checked error, not a wrong result
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=16)
+    sws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    with pytest.raises(sfb.SfbError) as info:
+        sfb.fused_attention_streamed(q, k, v, nn, sfb.to_device(stream["blob"]), stream, sws, bs, luts["blocks"], scale)
+    assert info.value.status == 3
+
+
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("d", [64, 32])
 def test_token_stride_of_a_merged_projection(bf16, d):
@@ -424,6 +470,8 @@ def test_argument_errors():
         C.c_uint32(kw.get("d", 64)), C.c_uint32(1), C.c_uint32(2), C.c_uint32(1), C.c_float(0.125))
     assert call(q=None) == 1
     assert call(bs=16) == 2
-    assert call(d=48) == 3
+    assert call(d=50) == 3      # fp32 rows are whole 16-byte vectors: multiples of 4
+    assert call(d=132) == 3
+    assert call(d=44, dtype=1) == 3   # bf16: multiples of 8
     assert call(dtype=7) == 5
     assert call(q=C.c_void_p(q.data_ptr() + 4)) == 6

@@ -34,17 +34,21 @@ class Tensor:
         self.tile_base = (r0 * self.row_elems + c0) * 2
 
 
-def fill_tile(ti, tensor, lds, lds_tile=0, by_halves=False):
-    """What load_tile_all (or load_tile_by_halves) does, for all waves of the work-group."""
+def fill_tile(ti, tensor, lds, lds_tile=0, by_halves=False, ragged_hd=None):
+    """What load_tile_all (or load_tile_by_halves) does, for all waves of the work-group.  ragged_hd: the tensor's
+    head size when it is smaller than the kernel's (load_tile_all<true> with sources_ragged)."""
     group_rows = 4 if by_halves else 8
     for wave in range(ti.NW):
         for i in range(ti.LOADS):
             for f in range(ti.SLICES):
-                part = bool(ti.PARTIAL) and f == ti.SLICES - 1
+                part = (bool(ti.PARTIAL) or ragged_hd is not None) and f == ti.SLICES - 1
                 n, odd = ti.load_group(i, wave), ti.load_group_odd(i, wave)
                 assert odd == n % 2
                 if by_halves:
                     source = ti.lane_source_by_halves
+                elif part and ragged_hd is not None:
+                    nch = ti.last_slice_chunks(ragged_hd)
+                    source = lambda lane, odd, row_bytes: ti.lane_source_ragged(lane, odd, row_bytes, nch)
                 else:
                     source = ti.lane_source_part if part else ti.lane_source
                 offsets = [source(lane, odd, tensor.row_bytes) for lane in range(64)]
@@ -148,6 +152,62 @@ def test_one_lds_base_per_tile_fills_the_same_tile(bs, heads):
     fill_tile_once(ti, tensor, b, lds_tile=2 * ti.TILE_BYTES)
     assert np.array_equal(a.mem, b.mem) and np.array_equal(a.writes, b.writes)
     check_score_fragments(ti, b, lds_tile=2 * ti.TILE_BYTES)
+
+
+@pytest.mark.parametrize("bs", [32, 64])
+@pytest.mark.parametrize("hd", [8, 16, 24, 40, 48, 56, 72, 80, 88, 104, 112, 120])
+def test_head_sizes_between_the_kernels(bs, hd):
+    """A head size that is not a multiple of 32 runs through the kernel of the next multiple: the loaders must stay
+    inside the hd features of their rows (the neighbouring head's features, or the end of the allocation, lie right
+    behind them), every LDS byte the readers touch must have been written, the features that exist must be where
+    the readers expect them, and with zero-padded queries the score product must come out exact."""
+    D = (hd + 31) // 32 * 32
+    ti = TileIndex(bs, D)
+    tensor = Tensor(bs, hd, heads=3, head=2, blocks=2, block=1)      # the last head of the last block: the
+    lds = Lds(ti.TILE_BYTES)                                         # allocation ends with the tile's last row
+    assert ti.last_slice_chunks(hd) == (hd - 64 * (ti.SLICES - 1)) // 8 >= 1
+    fill_tile(ti, tensor, lds, ragged_hd=hd)
+    check_fill(ti, lds)
+    rng = np.random.default_rng(hd)
+    K = rng.integers(-3, 4, (bs, hd)).astype(np.float64)
+    Q = rng.integers(-3, 4, (bs, hd)).astype(np.float64)
+    S = K @ Q.T
+    for wave in range(bs // 32):
+        acc = [np.zeros((64, 16)) for _ in range(bs // 32)]
+        for ks in range(D // 16):
+            q_regs = np.zeros((64, 8))
+            for lane in range(64):
+                first = 16 * ks + 8 * (lane // 32)
+                if first < hd:                                       # load_q_ragged: zeros beyond the row
+                    q_regs[lane] = Q[32 * wave + lane % 32, first:first + 8]
+            for kt in range(bs // 32):
+                addresses = [ti.k_frag_offset(ti.k_lane_base(lane % 32, lane // 32), kt, ks) for lane in range(64)]
+                ids = lds.ds_read_b128(addresses)
+                assert (ids != POISON).all(), "filler must come from the tile's own rows"
+                k_regs = np.zeros((64, 8))
+                for lane in range(64):
+                    first = 16 * ks + 8 * (lane // 32)
+                    if first < hd:
+                        want = [element_id(32 * kt + lane % 32, first + e) for e in range(8)]
+                        assert ids[lane].tolist() == want, (kt, ks, lane)
+                        k_regs[lane] = K[ids[lane] >> 8, ids[lane] & 0xFF]
+                    else:
+                        k_regs[lane] = 99.0                          # whatever the filler is, it meets zeros
+                acc[kt] = mfma_32x32x16(k_regs, q_regs, acc[kt])
+        for kt in range(bs // 32):
+            for lane in range(64):
+                for i in range(16):
+                    assert acc[kt][lane, i] == S[32 * kt + accumulator_row(i, lane // 32), 32 * wave + lane % 32]
+    # the second product reads columns: those below hd are the tile's own
+    for mt in range(D // 32):
+        for u in range(bs // 16):
+            got = read_transposed(ti, lds, mt, u)
+            assert (got != POISON).all()
+            for lane in range(64):
+                m, half = lane % 32, lane // 32
+                if 32 * mt + m < hd:
+                    want = [element_id(16 * u + 8 * a + 4 * half + c, 32 * mt + m) for a in range(2) for c in range(4)]
+                    assert got[lane].tolist() == want, (mt, u, lane)
 
 
 def test_row_order_of_the_dsd_tile():

@@ -48,6 +48,7 @@ class _Names:
     ti_slab_passes = ti_sdd_wait_count = ti_sdd_wait_loads = ti_dsd_wait_count = ti_dsd_depth = None
     ti_dsd_p_loads = ti_dsd_v_loads = None
     ti_once_inst_offset = ti_once_lane_offset = ti_once_base = ti_once_m0 = None
+    ti_lane_source_ragged = ti_last_slice_chunks = None
 
 
 class TileIndex:
@@ -72,6 +73,12 @@ class TileIndex:
 
     def lane_source_by_halves(self, lane, odd, row_bytes):
         return int(self._l.ti_lane_source_by_halves(self.bs, self.d, lane, odd, row_bytes))
+
+    def lane_source_ragged(self, lane, odd, row_bytes, nch):
+        return int(self._l.ti_lane_source_ragged(self.bs, self.d, lane, odd, row_bytes, nch))
+
+    def last_slice_chunks(self, hd):
+        return int(self._l.ti_last_slice_chunks(self.bs, self.d, hd))
 
     def load_group(self, i, wave):
         return int(self._l.ti_load_group(self.bs, self.d, i, wave))

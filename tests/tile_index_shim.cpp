@@ -35,6 +35,10 @@ uint32_t ti_lane_source_part(int bs, int d, uint32_t lane, uint32_t odd, uint32_
 uint32_t ti_lane_source_by_halves(int bs, int d, uint32_t lane, uint32_t odd, uint32_t row_bytes) {
     DISPATCH(bs, d, I::lane_source_by_halves(lane, odd, row_bytes));
 }
+uint32_t ti_lane_source_ragged(int bs, int d, uint32_t lane, uint32_t odd, uint32_t row_bytes, uint32_t nch) {
+    DISPATCH(bs, d, I::lane_source_ragged(lane, odd, row_bytes, nch));
+}
+uint32_t ti_last_slice_chunks(int bs, int d, uint32_t hd) { DISPATCH(bs, d, I::last_slice_chunks(hd)); }
 uint32_t ti_load_group(int bs, int d, int i, uint32_t wave) { DISPATCH(bs, d, I::load_group(i, wave)); }
 uint32_t ti_load_group_odd(int bs, int d, int i, uint32_t wave) { DISPATCH(bs, d, I::load_group_odd(i, wave)); }
 int ti_once_inst_offset(int bs, int d, int i) { DISPATCH(bs, d, I::once_inst_offset(i)); }
