@@ -252,7 +252,8 @@ uint32_t sfb_resident_work_groups(void);
  * launches return SFB_ERR_HEAD_STATE for those); the products of the unfused path
  * (sfb_sdd_nt, sfb_dsd_xn and the kernels made of them) take 64 with either type and 32, 96, 128 with fp32
  * Q / K / V (the dense operand of a product) -- the reference's K64 = false paths,
- * openai_blocksparse.h:221-222; the fused backward takes 64.  Anything else returns SFB_ERR_HEAD_STATE. */
+ * openai_blocksparse.h:221-222; the fused backward takes 32, 64, 96 and 128 (bf16).  Anything else returns
+ * SFB_ERR_HEAD_STATE. */
 
 /* Fully fused attention: O = softmax_rows(scale * Q K^T restricted to layout & mask & key<valid_len) V,
  * one work-group per (batch, head, block-row), no S/P in memory.  Replaces the sequence

@@ -146,7 +146,7 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
         const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
         const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
         const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
-        const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+        const typename T::Sources src = T::sources(lane, row_bytes);
         const uint32_t lds0 = T::lds_address(smem);
         const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
         const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
@@ -164,8 +164,8 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
             return u;
         };
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
-            T::load_tile(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
-            T::load_tile(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+            T::load_tile_all(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::load_tile_all(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
         };
         const sfb_uint2* const nn_lut = p.nn_lut + (size_t)h * p.lut_stride;
         sfb_uint2 e = uniform(nn_lut[off]);
@@ -255,7 +255,7 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
         const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
         const uint8_t* const q_base = (const uint8_t*)p.q + bh_bytes;
         const uint8_t* const do_base = (const uint8_t*)p.d_out + bh_bytes;
-        const uint32_t src_even = T::lane_source(lane, 0, row_bytes), src_odd = T::lane_source(lane, 1, row_bytes);
+        const typename T::Sources src = T::sources(lane, row_bytes);
         const uint32_t lds0 = T::lds_address(smem);
         const uint32_t k_lane = T::k_lane_base(kn, half), v_lane = T::v_lane_base(lane);
         const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
@@ -274,8 +274,8 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
             return u;
         };
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {   // e = {block id, row block}
-            T::load_tile(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
-            T::load_tile(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src_even, src_odd, row_bytes);
+            T::load_tile_all(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::load_tile_all(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
         };
         const sfb_uint2* const tn_lut = p.tn_lut + (size_t)h * p.lut_stride;
         sfb_uint2 e = uniform(tn_lut[off]);
@@ -365,7 +365,7 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
 // work-group of the first is done; as one, its work-groups fill the slots as the first's drain.  col_wgs is a
 // multiple of 8, so both halves see the same work-group -> XCD assignment as a launch of their own.
 template <int BS, int D, bool MASKED>
-__global__ __launch_bounds__(BS * 2, 2) void attention_backward_kernel(BackwardParams cols, BackwardParams rows,
+__global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void attention_backward_kernel(BackwardParams cols, BackwardParams rows,
                                                                        uint32_t col_wgs) {
     __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * Bf16DirectTiles<BS, D>::TILE_BYTES];
     if (blockIdx.x < col_wgs) attention_dkdv<BS, D, MASKED>(cols, blockIdx.x, smem);
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(float* dk, float* 
     else reduce_line<BS, D, 1>(dq, nullptr, row_partials, it, n_row_parts, blockIdx.y, heads, ctx);
 }
 
-template <int BS>
+template <int BS, int D>
 static int launch_backward(hipStream_t stream, const BackwardParams& p, const sfb_work_item* row_items,
                            uint32_t n_row_items, uint32_t n_row_heavy, uint32_t n_row_parts,
                            const sfb_work_item* col_items, uint32_t n_col_items, uint32_t n_col_heavy,
@@ -421,13 +421,13 @@ static int launch_backward(hipStream_t stream, const BackwardParams& p, const sf
     clear_stale_error();
     const uint32_t col_wgs = groups * 8u * cols.ranks, row_wgs = groups * 8u * rows.ranks;
     if (masked)
-        attention_backward_kernel<BS, 64, true><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
+        attention_backward_kernel<BS, D, true><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
     else
-        attention_backward_kernel<BS, 64, false><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
+        attention_backward_kernel<BS, D, false><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
     const uint32_t reduce_cols = (col_items && n_col_parts) ? n_col_items : 0u;
     const uint32_t reduce_rows = (row_items && n_row_parts) ? n_row_items : 0u;
     if (reduce_cols + reduce_rows)
-        reduce_partials_kernel<BS, 64><<<dim3(reduce_cols + reduce_rows, p.batch * p.heads), dim3(256), 0, stream>>>(
+        reduce_partials_kernel<BS, D><<<dim3(reduce_cols + reduce_rows, p.batch * p.heads), dim3(256), 0, stream>>>(
             p.dk, p.dv, p.dq, col_partials, row_partials, col_items, row_items, reduce_cols, n_col_parts, n_row_parts,
             p.heads, p.nb * BS);
     return launch_status();
@@ -458,7 +458,7 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
         return SFB_ERR_NULL_POINTER;
     if (dtype != SFB_BF16) return SFB_ERR_DTYPE;   // fp32 tensors take the unfused sequence
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 64) return SFB_ERR_HEAD_STATE;
+    if (state_dim != 32 && state_dim != 64 && state_dim != 96 && state_dim != 128) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (!batch_dim || !ctx_blks || !head_dim || !mask_heads || !lut_heads) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
@@ -490,9 +490,18 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     float* row_partials = (float*)workspace;
     float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * state_dim;
     hipStream_t s = (hipStream_t)stream;
-    if (block_size == 64)
-        return launch_backward<64>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items,
-                                   n_col_heavy, n_col_parts, row_partials, col_partials);
-    return launch_backward<32>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items,
-                               n_col_heavy, n_col_parts, row_partials, col_partials);
+#define SFB_CALL(BSV, DV)                                                                                        \
+    return launch_backward<BSV, DV>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items, \
+                                    n_col_heavy, n_col_parts, row_partials, col_partials)
+    if (block_size == 64) {
+        if (state_dim == 64) SFB_CALL(64, 64);
+        if (state_dim == 32) SFB_CALL(64, 32);
+        if (state_dim == 96) SFB_CALL(64, 96);
+        SFB_CALL(64, 128);
+    }
+    if (state_dim == 64) SFB_CALL(32, 64);
+    if (state_dim == 32) SFB_CALL(32, 32);
+    if (state_dim == 96) SFB_CALL(32, 96);
+    SFB_CALL(32, 128);
+#undef SFB_CALL
 }
