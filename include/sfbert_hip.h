@@ -250,8 +250,8 @@ uint32_t sfb_resident_work_groups(void);
  * launches also take every other multiple of 4 (fp32) or 8 (bf16: rows are whole 16-byte vectors) up to 128 -- the
  * reference's `d % 4 == 0` -- through the kernel of the next multiple of 32 with zero-padded queries (streamed
  * launches return SFB_ERR_HEAD_STATE for those); the products of the unfused path
- * (sfb_sdd_nt, sfb_dsd_xn and the kernels made of them) take 64 with either type and 32, 96, 128 with fp32
- * Q / K / V (the dense operand of a product) -- the reference's K64 = false paths,
+ * (sfb_sdd_nt, sfb_dsd_xn and the kernels made of them) take 32, 64, 96 and 128 with either type -- the
+ * reference's K64 = false paths,
  * openai_blocksparse.h:221-222; the fused backward takes 32, 64, 96 and 128 (bf16).  Anything else returns
  * SFB_ERR_HEAD_STATE. */
 

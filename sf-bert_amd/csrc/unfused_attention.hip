@@ -1145,7 +1145,7 @@ struct DsdParams {
 };
 
 template <int BS, int D, typename TA, typename TB>
-__global__ __launch_bounds__(BS * 2, 2) void dsd_tn_kernel(DsdParams p) {
+__global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && sizeof(TB) == 2) ? 1 : 2) void dsd_tn_kernel(DsdParams p) {
     constexpr int NO = D / 32;
     constexpr bool kFast = sizeof(TA) == 2 && sizeof(TB) == 2 && BS == 64;
     using TD = Bf16DirectTiles<BS, D>;
@@ -1179,13 +1179,13 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_tn_kernel(DsdParams p) {
     if constexpr (kFast) {
         // tiles 0, 1: X row blocks [q][D]; tiles 2, 3: sparse blocks [q][key]; LDS-direct loads, double-buffered
         const uint32_t row_bytes = row_stride * 2;
-        const uint32_t x_even = TD::lane_source(lane, 0, row_bytes), x_odd = TD::lane_source(lane, 1, row_bytes);
+        const typename TD::Sources x_src = TD::sources(lane, row_bytes);
         const uint32_t a_even = TD::lane_source(lane, 0, BS * 2), a_odd = TD::lane_source(lane, 1, BS * 2);
         const uint32_t lds0 = TD::lds_address(smem);
         const uint32_t x_lane = TD::v_lane_base(lane);
         const uint8_t* const x_base = (const uint8_t*)X + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
-            TD::load_tile(lds0 + buf * TILE, x_base + (size_t)e.y * BS * row_bytes, wave, x_even, x_odd, row_bytes);
+            TD::load_tile_all(lds0 + buf * TILE, x_base + (size_t)e.y * BS * row_bytes, wave, x_src, row_bytes);
             TD::load_tile(lds0 + (2 + buf) * TILE, (const uint8_t*)A + (size_t)e.x * BS * BS * 2, wave, a_even, a_odd,
                           BS * 2);
         };
@@ -1271,7 +1271,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr bool kBf16 = sizeof(TV) == 2;
     using TD = Bf16DirectTiles<BS, D>;
     using TF = F32Tiles<BS, D>;
-    constexpr int LDS_BYTES = kBf16 ? (sizeof(TP) == 2 && BS == 64 ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
+    constexpr bool kRing = kBf16 && sizeof(TP) == 2 && BS == 64 && D == 64;   // the streaming form below
+    constexpr int LDS_BYTES = kBf16 ? (kRing ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
     // Block-rows are taken from both ends of the context inwards, the last and the first one of every head before
@@ -1297,7 +1298,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[n][i] = 0.f;
 
-    if constexpr (kBf16 && sizeof(TP) == 2 && BS == 64) {
+    if constexpr (kRing) {
         // bf16 P and V.  P is the stream from memory: it is read once, straight into registers in operand layout,
         // kDepth key blocks ahead, so that a work-group keeps several tiles in flight without spending LDS on
         // them (LDS would bound the work-groups per CU, and with them the bytes in flight).  For that a lane's 8
@@ -1396,7 +1397,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         // multiplied.  One barrier per key block.
         constexpr int PU = BS / 16;
         const uint32_t row_bytes = row_stride * 2;
-        const uint32_t src_even = TD::lane_source(lane, 0, row_bytes), src_odd = TD::lane_source(lane, 1, row_bytes);
+        const typename TD::Sources src = TD::sources(lane, row_bytes);
         const uint32_t lds0 = TD::lds_address(smem), v_lane = TD::v_lane_base(lane);
         const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
         // slots j of product step u: keys 16u + 8(j/4) + 4*half + j%4
@@ -1410,8 +1411,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
             }
         };
         auto fetch_v = [&](uint32_t col, uint32_t buf) {
-            TD::load_tile(lds0 + buf * TD::TILE_BYTES, v_base + (size_t)col * BS * row_bytes, wave, src_even, src_odd,
-                          row_bytes);
+            TD::load_tile_all(lds0 + buf * TD::TILE_BYTES, v_base + (size_t)col * BS * row_bytes, wave, src, row_bytes);
         };
         if (count > 0) {
             const sfb_uint2 e0 = lut[off];
@@ -1826,22 +1826,26 @@ static int check_dtype(int d) { return (d == SFB_F32 || d == SFB_BF16) ? SFB_OK 
 
 using namespace sfb;
 
-// Head sizes: 64 with every type combination; 32, 96 and 128 with fp32 dense tensors (Q, K, V and the like).
+// Head sizes: 32, 64, 96 and 128 with every type combination (the reference's K64 = false paths,
+// openai_blocksparse.h:221-222, for the sizes the MFMA tiles divide).
 static int check_head_state(uint32_t state_dim, int dense_dtype) {
-    if (state_dim == 64) return SFB_OK;
-    if (dense_dtype == SFB_F32 && (state_dim == 32 || state_dim == 96 || state_dim == 128)) return SFB_OK;
-    return SFB_ERR_HEAD_STATE;
+    (void)dense_dtype;
+    return state_dim == 32 || state_dim == 64 || state_dim == 96 || state_dim == 128 ? SFB_OK : SFB_ERR_HEAD_STATE;
 }
-// CALL(D, T) for a head size other than 64: dense type float, T = the sparse tensor's type
-#define SFB_DISPATCH_D(DV, TS, CALL)                                      \
-    do {                                                                  \
-        if ((TS) == SFB_F32) { CALL(DV, float); } else { CALL(DV, __bf16); } \
+// CALL(D, TD, TS) for a head size other than 64: TD = the dense tensors' type, TS = the sparse tensor's
+#define SFB_DISPATCH_D(DV, TDN, TS, CALL)                                            \
+    do {                                                                             \
+        if ((TDN) == SFB_F32) {                                                      \
+            if ((TS) == SFB_F32) { CALL(DV, float, float); } else { CALL(DV, float, __bf16); }   \
+        } else {                                                                     \
+            if ((TS) == SFB_F32) { CALL(DV, __bf16, float); } else { CALL(DV, __bf16, __bf16); } \
+        }                                                                            \
     } while (0)
-#define SFB_DISPATCH_OTHER_D(STATE, TS, CALL)                              \
+#define SFB_DISPATCH_OTHER_D(STATE, TDN, TS, CALL)                         \
     do {                                                                  \
-        if ((STATE) == 32) SFB_DISPATCH_D(32, TS, CALL);                   \
-        else if ((STATE) == 96) SFB_DISPATCH_D(96, TS, CALL);              \
-        else SFB_DISPATCH_D(128, TS, CALL);                                \
+        if ((STATE) == 32) SFB_DISPATCH_D(32, TDN, TS, CALL);              \
+        else if ((STATE) == 96) SFB_DISPATCH_D(96, TDN, TS, CALL);         \
+        else SFB_DISPATCH_D(128, TDN, TS, CALL);                           \
     } while (0)
 
 #define SFB_DISPATCH_2(BSV, T0, T1, CALL)                                                  \
@@ -1870,10 +1874,10 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (state_dim != 64) {
-#define SFB_CALL64(DV, TO) sdd_nt_kernel<64, DV, float, TO><<<grid, dim3(128), 0, s>>>(p)
-#define SFB_CALL32(DV, TO) sdd_nt_kernel<32, DV, float, TO><<<grid, dim3(64), 0, s>>>(p)
-        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, out_dtype, SFB_CALL64);
-        else SFB_DISPATCH_OTHER_D(state_dim, out_dtype, SFB_CALL32);
+#define SFB_CALL64(DV, TI, TO) sdd_nt_kernel<64, DV, TI, TO><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_CALL32(DV, TI, TO) sdd_nt_kernel<32, DV, TI, TO><<<grid, dim3(64), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, in_dtype, out_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, in_dtype, out_dtype, SFB_CALL32);
 #undef SFB_CALL64
 #undef SFB_CALL32
         return launch_status();
@@ -1953,16 +1957,16 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (state_dim != 64) {
-#define SFB_TN64(DV, TA) dsd_tn_kernel<64, DV, TA, float><<<grid, dim3(128), 0, s>>>(p)
-#define SFB_TN32(DV, TA) dsd_tn_kernel<32, DV, TA, float><<<grid, dim3(64), 0, s>>>(p)
-#define SFB_NN64(DV, TA) dsd_nn_kernel<64, DV, TA, float><<<grid, dim3(128), 0, s>>>(p)
-#define SFB_NN32(DV, TA) dsd_nn_kernel<32, DV, TA, float><<<grid, dim3(64), 0, s>>>(p)
+#define SFB_TN64(DV, TB, TA) dsd_tn_kernel<64, DV, TA, TB><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_TN32(DV, TB, TA) dsd_tn_kernel<32, DV, TA, TB><<<grid, dim3(64), 0, s>>>(p)
+#define SFB_NN64(DV, TB, TA) dsd_nn_kernel<64, DV, TA, TB><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_NN32(DV, TB, TA) dsd_nn_kernel<32, DV, TA, TB><<<grid, dim3(64), 0, s>>>(p)
         if (op == SFB_TN_OP) {
-            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_TN64);
-            else SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_TN32);
+            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, b_dtype, a_dtype, SFB_TN64);
+            else SFB_DISPATCH_OTHER_D(state_dim, b_dtype, a_dtype, SFB_TN32);
         } else {
-            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_NN64);
-            else SFB_DISPATCH_OTHER_D(state_dim, a_dtype, SFB_NN32);
+            if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, b_dtype, a_dtype, SFB_NN64);
+            else SFB_DISPATCH_OTHER_D(state_dim, b_dtype, a_dtype, SFB_NN32);
         }
 #undef SFB_TN64
 #undef SFB_TN32
@@ -2037,10 +2041,10 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (state_dim != 64) {
-#define SFB_CALL64(DV, TO) sdd_softmax_kernel<64, DV, float, TO><<<grid, dim3(128 * kSddSoftmaxKeyGroups), 0, s>>>(p)
-#define SFB_CALL32(DV, TO) sdd_softmax_kernel<32, DV, float, TO><<<grid, dim3(64 * kSddSoftmaxKeyGroups), 0, s>>>(p)
-        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, y_dtype, SFB_CALL64);
-        else SFB_DISPATCH_OTHER_D(state_dim, y_dtype, SFB_CALL32);
+#define SFB_CALL64(DV, TI, TO) sdd_softmax_kernel<64, DV, TI, TO><<<grid, dim3(128 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+#define SFB_CALL32(DV, TI, TO) sdd_softmax_kernel<32, DV, TI, TO><<<grid, dim3(64 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, in_dtype, y_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, in_dtype, y_dtype, SFB_CALL32);
 #undef SFB_CALL64
 #undef SFB_CALL32
         return launch_status();
@@ -2148,10 +2152,10 @@ extern "C" int sfb_sdd_softmax_grad(sfb_stream_t stream, const sfb_uint2* nt_lut
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
     if (state_dim != 64) {
-#define SFB_CALL64(DV, TS) sdd_softmax_grad_kernel<64, DV, float, TS><<<grid, dim3(128), 0, s>>>(g)
-#define SFB_CALL32(DV, TS) sdd_softmax_grad_kernel<32, DV, float, TS><<<grid, dim3(64), 0, s>>>(g)
-        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, sparse_dtype, SFB_CALL64);
-        else SFB_DISPATCH_OTHER_D(state_dim, sparse_dtype, SFB_CALL32);
+#define SFB_CALL64(DV, TI, TS) sdd_softmax_grad_kernel<64, DV, TI, TS><<<grid, dim3(128), 0, s>>>(g)
+#define SFB_CALL32(DV, TI, TS) sdd_softmax_grad_kernel<32, DV, TI, TS><<<grid, dim3(64), 0, s>>>(g)
+        if (block_size == 64) SFB_DISPATCH_OTHER_D(state_dim, in_dtype, sparse_dtype, SFB_CALL64);
+        else SFB_DISPATCH_OTHER_D(state_dim, in_dtype, sparse_dtype, SFB_CALL32);
 #undef SFB_CALL64
 #undef SFB_CALL32
         return launch_status();
