@@ -123,6 +123,47 @@ def test_error_codes():
                    u32(0), None, C.c_size_t(0), *args_tail, u32(64), u32(1), C.c_float(0.125)) == 1   # NULL tensors
 
 
+def test_argument_checks_of_the_newer_entry_points():
+    """Checked before anything touches the device, so they can be exercised without one."""
+    u32, ptr = C.c_uint32, C.c_void_p
+    buf = np.zeros(4096, np.uint8)
+    p = ptr(buf.ctypes.data)          # 16-byte aligned host memory standing in for tensors: never dereferenced here
+    heads = sfb.lib.sfb_fused_attention_scheduled_heads
+
+    def call(q=p, dtype=sfb.BF16, d=64, lut_heads=4, lut_dim=10, head_dim=4, items=p, n_items=3, n_heavy=0):
+        return heads(None, q, p, p, p, None, dtype, sfb.F32, p, None, None, items, u32(n_items), u32(n_heavy), u32(0),
+                     u32(0), None, C.c_size_t(0), u32(64), u32(6), u32(1), u32(4), u32(head_dim), u32(d), u32(lut_heads),
+                     u32(lut_dim), u32(1), C.c_float(0.125))
+    assert call(q=None) == 1
+    assert call(items=None) == 1
+    assert call(lut_heads=3) == 4           # one table per head or one for all
+    assert call(lut_dim=11) == 4            # lut_dim = ctx_blks + blocks
+    assert call(lut_heads=0) == 4
+    assert call(n_heavy=3) == 4
+    assert call(d=44) == 3 and call(d=136) == 3 and call(d=0) == 3      # bf16 rows: multiples of 8 up to 128
+    assert call(d=44, dtype=sfb.F32, q=None) == 1                       # fp32: multiples of 4 (passes the size check)
+    assert call(d=42, dtype=sfb.F32) == 3
+    assert sfb.lib.sfb_stream_reset(None, None, u32(64), p) == 1
+    assert sfb.lib.sfb_resident_work_groups_for(7, u32(64), u32(64), 0) == 0
+    assert sfb.lib.sfb_resident_work_groups_for(sfb.BF16, u32(48), u32(64), 0) == 0
+    n = u32(0)
+    assert sfb.lib.sfb_build_schedule_heads(None, C.byref(n), C.byref(n), C.byref(n), C.byref(n), None, 4, u32(1), u32(8),
+                                            u32(4)) == 1
+    assert sfb.lib.sfb_build_schedule_heads(None, C.byref(n), C.byref(n), C.byref(n), C.byref(n), p, 4, u32(2), u32(3),
+                                            u32(4)) == 4    # a table shorter than its header
+    assert sfb.lib.sfb_build_schedule_heads(None, C.byref(n), C.byref(n), C.byref(n), C.byref(n), p, 4, u32(1), u32(8),
+                                            u32(0)) == 8    # max_blocks
+    # the fused backward takes head sizes 32, 64, 96, 128
+    bwd = sfb.lib.sfb_fused_attention_backward
+
+    def backward(d, dtype=sfb.BF16):
+        return bwd(None, p, p, p, p, p, p, p, p, p, p, dtype, p, p, None, None, None, u32(0), u32(0), u32(0), None, u32(0),
+                   u32(0), u32(0), None, C.c_size_t(0), u32(64), u32(6), u32(1), u32(4), u32(4), u32(d), u32(1), u32(10),
+                   u32(1), C.c_float(-1.0))
+    assert backward(48) == 3 and backward(64, sfb.F32) == 5
+    assert backward(96) == 8 and backward(32) == 8 and backward(128) == 8   # size accepted; the scale is what is wrong
+
+
 def test_suggested_chunk_length():
     """1.25 x (key blocks of one head x batch x heads / 1024 resident work-groups), rounded up, at least 16."""
     lay = orc.layout_bigbird(64, 1, 2, True, orc.bigbird_draw(64, 1, 2, True, 3, 1234))
