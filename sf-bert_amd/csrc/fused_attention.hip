@@ -22,6 +22,9 @@
 #ifndef SFB_TILE_LOAD_ONCE
 #define SFB_TILE_LOAD_ONCE 0   // 1: the fused bf16 kernel for head size 64 issues a tile's loads as one group (load_tile_once)
 #endif
+#ifndef SFB_TILE_LOAD_STAGED
+#define SFB_TILE_LOAD_STAGED 0   // 1: ... brings the tiles of its loop in through registers (staged_fetch / staged_commit)
+#endif
 #include <type_traits>
 
 namespace sfb {
@@ -522,6 +525,14 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
 #else
     constexpr bool kOnce = false;
 #endif
+#if SFB_TILE_LOAD_STAGED
+    // experimental: the loop's tiles go through registers; the prologue keeps the LDS-direct loads
+    constexpr bool kStaged = D == 64 && !RAGGED;
+    const uint32_t staged_src = T::I::staged_source(lane, row_bytes);
+    const uint32_t staged_even = T::I::staged_lds_offset(lane, 0), staged_odd = T::I::staged_lds_offset(lane, 1);
+#else
+    constexpr bool kStaged = false;
+#endif
     const uint32_t lds0 = T::lds_address(smem);
     // LUT entries of key blocks [win, win + 64) of this item, one per lane (clamped to the last one)
     uint32_t win = 0;
@@ -665,6 +676,13 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         };
         fragments(0);
         exps(0);
+#if SFB_TILE_LOAD_STAGED
+        typename T::Staged k_staged, v_staged;
+        if constexpr (kStaged) {
+            T::staged_fetch(k_staged, k_src, wave, staged_src, row_bytes);
+            T::staged_fetch(v_staged, v_src, wave, staged_src, row_bytes);
+        } else
+#endif
         if constexpr (kOnce) {
             load_tile(k_dst, k_src);
             load_tile(v_dst, v_src);
@@ -706,6 +724,13 @@ __device__ __forceinline__ bool attend_item_bf16(const FusedParams& p, const Row
         }
         st.l += sum0 + sum1;
         if constexpr (SLIM) __builtin_amdgcn_sched_barrier(0);   // the wait for the tiles comes last
+#if SFB_TILE_LOAD_STAGED
+        if constexpr (kStaged) {
+            // K(j) and V(j-1), whose buffers these tiles take, were last read in iteration j-1, before its barrier
+            T::staged_commit(k_staged, smem + par * TILE, wave, staged_even, staged_odd);
+            T::staged_commit(v_staged, smem + (2 + (par ^ 1)) * TILE, wave, staged_even, staged_odd);
+        }
+#endif
         loads_landed();
     };
 

@@ -90,6 +90,17 @@ struct TileIndex {
     static_assert(LOADS == 4 && (LOADS - 1) * NW * 1024 - ONCE_CENTER <= 4095 && -ONCE_CENTER >= -4096,
                   "four loads per wave and slice, offsets of 13 signed bits");
 
+    // The same tile filled through registers (ordinary 16-byte loads, then ds_write_b128): the lanes read whole rows
+    // in order -- lane l the chunk l % 8 of row l / 8 of an 8-row group -- and apply the swizzle on the LDS side.
+    // Both offsets are relative to the group's first source row / its 1 KiB of LDS.
+    static SFB_INDEX_FN uint32_t staged_source(uint32_t lane, uint32_t row_bytes) {
+        return (lane >> 3) * row_bytes + ((lane & 7u) << 4);
+    }
+    static SFB_INDEX_FN uint32_t staged_lds_offset(uint32_t lane, uint32_t odd) {
+        const uint32_t rr = lane >> 3, c = lane & 7u;
+        return rr * 128u + ((c ^ swz(8u * odd + rr)) << 4);
+    }
+
     // Per-lane byte offset of the score fragment (16 bytes: 8 features of one row) of k-step 0 in row tile 0;
     // k-step ks (features 16 ks + 8 half ..) is at (base ^ (ks % 4) * 32) in slice ks / 4, row tile kt 4096 bytes on.
     static SFB_INDEX_FN uint32_t k_lane_base(uint32_t qn, uint32_t half) {

@@ -155,6 +155,26 @@ struct Bf16DirectTiles {
                        "n"(I::once_inst_offset(3))
                      : "memory");
     }
+    // A wave's share of a one-slice tile on its way through registers: fetch() issues ordinary 16-byte loads of whole
+    // rows (the wave is free again as soon as they are issued), commit() writes them to LDS with the swizzle applied
+    // on that side (TileIndex::staged_*).  Against the LDS-direct form this costs 16 registers per tile in flight
+    // and four ds_write_b128 per wave and tile.
+    struct Staged {
+        u32x4 r[I::LOADS];
+    };
+    static __device__ __forceinline__ void staged_fetch(Staged& st, const uint8_t* g_tile, uint32_t wave, uint32_t lane_src,
+                                                        uint32_t row_bytes) {
+        static_assert(SLICES == 1 && !PARTIAL, "whole one-slice tiles");
+#pragma unroll
+        for (int i = 0; i < I::LOADS; ++i)
+            st.r[i] = *(const u32x4*)(g_tile + (size_t)I::load_group(i, wave) * 8u * row_bytes + lane_src);
+    }
+    static __device__ __forceinline__ void staged_commit(const Staged& st, uint8_t* lds_tile, uint32_t wave,
+                                                         uint32_t dst_even, uint32_t dst_odd) {
+#pragma unroll
+        for (int i = 0; i < I::LOADS; ++i)
+            *(u32x4*)(lds_tile + I::load_group(i, wave) * 1024u + (I::load_group_odd(i, wave) ? dst_odd : dst_even)) = st.r[i];
+    }
     // Load number i of this wave's share of every slice of a tile.
     template <bool RAGGED = false>
     static __device__ __forceinline__ void load_rows_all(uint32_t lds_tile, const uint8_t* g_tile, int i, uint32_t wave,

@@ -68,6 +68,22 @@ def fill_tile_once(ti, tensor, lds, lds_tile=0):
                                         tensor.allowed, inst_offset=ti.once_inst_offset(i))
 
 
+def fill_tile_staged(ti, tensor, lds, lds_tile=0):
+    """What the register-staged form does: 16-byte loads of whole rows, then ds_write_b128 to the swizzled places."""
+    assert ti.SLICES == 1 and not ti.PARTIAL
+    for wave in range(ti.NW):
+        for i in range(ti.LOADS):
+            n, odd = ti.load_group(i, wave), ti.load_group_odd(i, wave)
+            base = tensor.tile_base + n * 8 * tensor.row_bytes
+            data, addresses = [], []
+            for lane in range(64):
+                src = base + ti.staged_source(lane, tensor.row_bytes)
+                assert tensor.allowed[src:src + 16].all(), "lane %d reads bytes outside its row" % lane
+                data.append(tensor.bytes[src:src + 16])
+                addresses.append(lds_tile + n * 1024 + ti.staged_lds_offset(lane, odd))
+            lds.ds_write_b128(addresses, data)
+
+
 def check_fill(ti, lds, lds_tile=0):
     written = lds.writes[lds_tile:lds_tile + ti.TILE_BYTES]
     assert (written == 1).all(), "every byte of the tile is written exactly once"
@@ -152,6 +168,10 @@ def test_one_lds_base_per_tile_fills_the_same_tile(bs, heads):
     fill_tile_once(ti, tensor, b, lds_tile=2 * ti.TILE_BYTES)
     assert np.array_equal(a.mem, b.mem) and np.array_equal(a.writes, b.writes)
     check_score_fragments(ti, b, lds_tile=2 * ti.TILE_BYTES)
+    # and so does the form that goes through registers and applies the swizzle on the LDS write
+    c = Lds(3 * ti.TILE_BYTES)
+    fill_tile_staged(ti, tensor, c, lds_tile=2 * ti.TILE_BYTES)
+    assert np.array_equal(a.mem, c.mem) and np.array_equal(a.writes, c.writes)
 
 
 @pytest.mark.parametrize("bs", [32, 64])

@@ -48,7 +48,7 @@ class _Names:
     ti_slab_passes = ti_sdd_wait_count = ti_sdd_wait_loads = ti_dsd_wait_count = ti_dsd_depth = None
     ti_dsd_p_loads = ti_dsd_v_loads = None
     ti_once_inst_offset = ti_once_lane_offset = ti_once_base = ti_once_m0 = None
-    ti_lane_source_ragged = ti_last_slice_chunks = None
+    ti_lane_source_ragged = ti_last_slice_chunks = ti_staged_source = ti_staged_lds_offset = None
 
 
 class TileIndex:
@@ -98,6 +98,12 @@ class TileIndex:
     def once_m0(self, wave):
         return int(self._l.ti_once_m0(self.bs, self.d, wave))
 
+    def staged_source(self, lane, row_bytes):
+        return int(self._l.ti_staged_source(self.bs, self.d, lane, row_bytes))
+
+    def staged_lds_offset(self, lane, odd):
+        return int(self._l.ti_staged_lds_offset(self.bs, self.d, lane, odd))
+
     def k_lane_base(self, qn, half):
         return int(self._l.ti_k_lane_base(self.bs, self.d, qn, half))
 
@@ -133,6 +139,13 @@ class Lds:
             assert 0 <= dst and dst + 16 <= self.mem.size, "LDS destination outside the tile"
             self.mem[dst:dst + 16] = glob[src:src + 16]
             self.writes[dst:dst + 16] += 1
+
+    def ds_write_b128(self, addresses, data):
+        """data: [64][16] bytes, lane l's 16 bytes go to its own address."""
+        for lane, a in enumerate(addresses):
+            assert a % 16 == 0 and 0 <= a and a + 16 <= self.mem.size, "b128 write misaligned or outside the tile"
+            self.mem[a:a + 16] = data[lane]
+            self.writes[a:a + 16] += 1
 
     def ds_read_b128(self, addresses):
         out = np.zeros((64, 8), np.uint16)

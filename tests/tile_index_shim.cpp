@@ -47,6 +47,8 @@ uint32_t ti_once_lane_offset(int bs, int d, uint32_t lane, int i, uint32_t wave,
 }
 uint32_t ti_once_base(int bs, int d, uint32_t wave, uint32_t row_bytes) { DISPATCH(bs, d, I::once_base(wave, row_bytes)); }
 uint32_t ti_once_m0(int bs, int d, uint32_t wave) { DISPATCH(bs, d, I::once_m0(wave)); }
+uint32_t ti_staged_source(int bs, int d, uint32_t lane, uint32_t row_bytes) { DISPATCH(bs, d, I::staged_source(lane, row_bytes)); }
+uint32_t ti_staged_lds_offset(int bs, int d, uint32_t lane, uint32_t odd) { DISPATCH(bs, d, I::staged_lds_offset(lane, odd)); }
 uint32_t ti_k_lane_base(int bs, int d, uint32_t qn, uint32_t half) { DISPATCH(bs, d, I::k_lane_base(qn, half)); }
 uint32_t ti_k_frag_offset(int bs, int d, uint32_t lane_base, int kt, int ks) {
     DISPATCH(bs, d, I::k_frag_offset(lane_base, kt, ks));
