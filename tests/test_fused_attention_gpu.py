@@ -227,52 +227,6 @@ def test_head_sizes_other_than_64(d, bs, bf16):
         check(out.cpu().numpy(), ref, tol)
 
 
-@pytest.mark.parametrize("d,bf16", [(16, True), (48, True), (80, True), (112, True), (40, True), (8, True), (120, True),
-                                    (16, False), (48, False), (80, False), (112, False), (36, False), (4, False),
-                                    (100, False)])
-@pytest.mark.parametrize("bs", [32, 64])
-def test_head_sizes_that_are_not_multiples_of_32(d, bs, bf16):
-    """The reference's K64 = false kernels take any head size that is a multiple of 4 (openai_blocksparse.h:221-222).
-    Here: multiples of 4 (fp32) or 8 (bf16 -- rows of whole 16-byte vectors) up to 128, through the kernel of the
-    next multiple of 32 with zero-padded queries; plain and scheduled launches, with and without mask and padding,
-    a row without blocks, split rows merged from partial records, bf16 output, log-sum-exp output."""
-    nb, B, H = 8, 2, 3
-    L = nb * bs
-    tol = TOL_BF16 if bf16 else TOL_F32
-    lay = PATTERNS["bigbird"](nb)
-    lay[5] = 0
-    luts = sfb.build_luts(lay)
-    keep = (np.random.default_rng(d).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
-    mask = sfb.pack_mask(keep)
-    valid = np.array([L, L - bs - 5], np.int32)
-    Q, K, V = qkv(B, L, H, d, seed=3 * d + bs, bf16=bf16)
-    scale = float(1.0 / np.sqrt(d))
-    want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, mask=mask, valid_len=valid, nthreads=THREADS)
-    plain = orc.attention(Q, K, V, luts["nn_lut"], bs, scale, nthreads=THREADS)
-    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid), want, tol)
-    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, mask=mask, valid_len=valid, max_blocks=3), want, tol)
-    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16), plain, tol)
-    check(run_fused(Q, K, V, luts, bs, scale, bf16=bf16, max_blocks=3), plain, tol)
-    q, k, v = (dev(x, bf16) for x in (Q, K, V))
-    sched = sfb.build_schedule(luts["nn_lut"], nb, 3)
-    ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
-    nn, items = sfb.to_device(luts["nn_lut"]), sfb.to_device(sched["items"])
-    if d % 8 == 0:
-        o16 = sfb.fused_attention_scheduled(q, k, v, nn, items, sched, ws, bs, luts["blocks"], scale, out_dtype=sfb.BF16)
-        torch.cuda.synchronize()
-        assert rel_err(o16.float().cpu().numpy(), plain) <= max(tol, 2.0 ** -7)
-    o32, lse = sfb.fused_attention_forward_lse(q, k, v, nn, items, sched, ws, bs, luts["blocks"], scale)
-    torch.cuda.synchronize()
-    check(o32.cpu().numpy(), plain, tol)
-    assert torch.isfinite(lse).all() and float(lse[:, :, 5 * bs:6 * bs].abs().max()) == 0.0
-    # streamed launches do not take these sizes: a checked error, not a wrong result
-    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=16)
-    sws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
-    with pytest.raises(sfb.SfbError) as info:
-        sfb.fused_attention_streamed(q, k, v, nn, sfb.to_device(stream["blob"]), stream, sws, bs, luts["blocks"], scale)
-    assert info.value.status == 3
-
-
 @pytest.mark.parametrize("bf16", [False, True])
 @pytest.mark.parametrize("d", [64, 32])
 def test_token_stride_of_a_merged_projection(bf16, d):
@@ -395,69 +349,6 @@ def test_scale_and_large_scores():
     for scale in (0.125, 1.0, 0.01):
         want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale)
         check(run_fused(Q, K, V, luts, bs, scale), want, TOL_F32)
-
-
-@pytest.mark.parametrize("qmul,scale", [(6.0, 0.125), (1.0, 1.0), (2.0, 1.0), (6.0, 1.0)])
-def test_large_scores_bf16(qmul, scale):
-    """Peaked rows with bf16 tensors, through the scheduled and the streamed launch without mask: |score * scale| of
-    30 to 90, exponents up to 2^85 above the offset of the row's first block, so the loop with the fixed offset is
-    what runs (the last case passes 2^100 and is redone by the loop that follows the maximum).  The error must not
-    grow with the scores: the scale's power-of-two part on the queries is exact and the rest is applied in fp32."""
-    bs, nb, B, H, d = 64, 8, 2, 3, 64
-    L = bs * nb
-    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
-    Q, K, V = qkv(B, L, H, d, seed=91)
-    Q, K, V = orc.round_bf16(Q * qmul), orc.round_bf16(K), orc.round_bf16(V)
-    want = orc.attention(Q, K, V, luts["nn_lut"], bs, scale)
-    got = run_fused(Q, K, V, luts, bs, scale, bf16=True, max_blocks=4)
-    err = rel_err(got, want)
-    q, k, v = (dev(x, True) for x in (Q, K, V))
-    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=16)
-    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
-    streamed = sfb.fused_attention_streamed(q, k, v, sfb.to_device(luts["nn_lut"]), sfb.to_device(stream["blob"]), stream,
-                                            ws, bs, luts["blocks"], scale)
-    torch.cuda.synchronize()
-    err_streamed = rel_err(streamed.cpu().numpy(), want)
-    print("scheduled %.3e, streamed %.3e" % (err, err_streamed), flush=True)
-    assert sfb.stream_status(stream, d, ws) == 0
-    assert err <= 0.75 * TOL_BF16 and err_streamed <= 0.75 * TOL_BF16
-
-
-@pytest.mark.parametrize("bf16", [True, False])
-@pytest.mark.parametrize("bs", [32, 64])
-def test_scheduled_launch_with_per_head_tables(bf16, bs):
-    """The reference's `fixed` pattern gives every head its own layout (fixed_fusion_test.cu:38-39, 58-106): the
-    scheduled launch with one look-up table, one mask and one work-item list per head, rows cut in chunks of 2."""
-    nb, B, H, d = 16, 3, 4, 64
-    L = bs * nb
-    lay = sfb.layout_fixed(H, nb, 4, causal=True)
-    per_head = [sfb.build_luts(lay[h]) for h in range(H)]
-    blocks = per_head[0]["blocks"]
-    assert all(p["blocks"] == blocks for p in per_head)
-    nn = np.concatenate([p["nn_lut"] for p in per_head])
-    masks = np.concatenate([sfb.pack_mask(sfb.element_mask(p["nt_lut"], bs, sfb.MASK_CAUSAL_DIAG)) for p in per_head])
-    Q, K, V = qkv(B, L, H, d, seed=81, bf16=bf16)
-    q, k, v = (dev(x, bf16) for x in (Q, K, V))
-    tol = TOL_BF16 if bf16 else TOL_F32
-    for max_blocks in (2, 100):
-        sched = sfb.build_schedule_heads(nn, nb, H, max_blocks)
-        assert (sched["n_parts"] > 0) == (max_blocks == 2)
-        ws = torch.zeros(max(sfb.schedule_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
-        for mask in (masks, None):
-            want = orc.attention(Q, K, V, nn, bs, 0.125, mask=mask, lut_heads=H, mask_heads=H if mask is not None else 1,
-                                 blocks=blocks, nthreads=THREADS)
-            outs = []
-            for _ in range(2):   # the second launch finds the arrival counters as the first one left them
-                out = torch.full((B, L, H, d), 7.0, device="cuda")
-                sfb.fused_attention_scheduled_heads(q, k, v, sfb.to_device(nn), sfb.to_device(sched["items"]), sched, ws,
-                                                    bs, blocks, 0.125, mask=None if mask is None else sfb.to_device(mask),
-                                                    mask_heads=H if mask is not None else 1, out=out)
-                torch.cuda.synchronize()
-                outs.append(out.cpu().numpy())
-            assert np.array_equal(outs[0], outs[1])
-            diff = np.abs(outs[0].astype(np.float64) - want).max(axis=(0, 1, 3)) / np.abs(want).max()
-            print("max_blocks", max_blocks, "masked", mask is not None, "error per head", diff, flush=True)
-            assert diff.max() <= tol
 
 
 def test_argument_errors():
