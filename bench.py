@@ -245,6 +245,9 @@ def time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, max_blocks
             "backward_TFLOPs": 2.5 * flops_forward / (ms_b * 1e-3) / 1e12}
 
 
+GEMM_TUNING = 0   # what --gemm-tuning asked for (reported with the layer's numbers)
+
+
 def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), steps=20):
     """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
     B, L, ffn = 8, 4096, 3072
@@ -264,6 +267,7 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), s
     pos = torch.randn((L, n), device="cuda") * 0.02
     x = sfb.embedding_lookup(tok, ids, pos).reshape(B * L, n)
     out = {"shape": "B8 L4096 hidden 768 heads 12 ffn 3072, BigBird block 64", "gemm_flops": 2.0 * B * L * (4 * n * n + 2 * n * ffn)}
+    out["gemm_tuning"] = GEMM_TUNING
     y = torch.empty_like(x)
     attn_flops = luts["blocks"] * B * H * 4.0 * bs * bs * d
     for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
@@ -333,6 +337,9 @@ def main():
                     help="only the bf16 encoder layer at B8 L4096, 200 timed calls (for a kernel trace of the layer)")
     ap.add_argument("--skip-extras", action="store_true",
                     help="only the fused-attention line: no unfused comparison, no encoder-layer timing")
+    ap.add_argument("--gemm-tuning", type=int, default=0, choices=[0, 1],
+                    help="how the GEMM seam picks its kernels (sfb_gemm_tuning): 0 = the library's short list, "
+                         "1 = every kernel of the library that supports the problem (seconds per shape, once)")
     ap.add_argument("--heavy", type=int, default=-1,
                     help="override the schedule's number of leading items launched for all heads first")
     ap.add_argument("--max-blocks", type=int, default=-1,
@@ -350,6 +357,9 @@ def main():
         print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
         sys.exit(1)
 
+    global GEMM_TUNING
+    GEMM_TUNING = args.gemm_tuning
+    sfb.gemm_tuning(args.gemm_tuning)
     pattern, B, H, L, d, bs, default_dtype = WORKLOADS[args.workload]
     dtype = args.dtype or default_dtype
     bf16 = dtype == "bf16"

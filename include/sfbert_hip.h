@@ -520,6 +520,11 @@ int sfb_cast_f32_bf16(sfb_stream_t stream, void* out, const float* in, uint64_t 
 /* Destroys the GEMM plans and the rocBLAS / hipBLASLt handles the GEMM entry points made (they are made again on
  * the next use).  Call it when no GEMM of this library is in flight. */
 void sfb_gemm_release(void);
+/* How a GEMM plan picks its kernel when it is made (first call of a shape): level 0 (default) times the library's
+ * short list of candidates for the problem, level 1 times every kernel of the library that supports the problem
+ * (a second or two per shape, once).  Plans already made keep their kernel until sfb_gemm_release().  Returns
+ * SFB_ERR_ARGUMENT for other levels. */
+int sfb_gemm_tuning(int level);
 
 /* cblas_sgemm(RowMajor, NoTrans, NoTrans, m, n, k, 1, A, k, W, n, 0, C, n) (transformer.cpp:516-522, 547,
  * 562, 571; cublasSgemm twins transformer_attention_optimize.cu:693-716): C[m][n] = A[m][k] W[k][n],

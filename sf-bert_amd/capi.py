@@ -67,7 +67,7 @@ EXPORTED = [
     "sfb_pack_mask", "sfb_transpose_mask", "sfb_build_row_order",
     "sfb_build_schedule", "sfb_build_schedule_heads", "sfb_suggest_max_blocks", "sfb_schedule_workspace_bytes",
     "sfb_build_stream", "sfb_stream_workspace_bytes", "sfb_stream_status", "sfb_stream_reset", "sfb_resident_work_groups",
-    "sfb_resident_work_groups_for", "sfb_scale_parts",
+    "sfb_resident_work_groups_for", "sfb_scale_parts", "sfb_gemm_tuning",
     "sfb_fused_attention_streamed",
     "sfb_static_scratch_bytes", "sfb_fused_attention_scheduled_noalloc",
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
@@ -311,6 +311,11 @@ def build_stream(nn_lut, nb, batch, heads, block_size, lut_heads=1, wg_slots=Non
                 blocks=view(plan.blocks_offset, plan.n_blocks, STREAM_BLOCK_DTYPE),
                 items=view(plan.items_offset, plan.n_items, STREAM_ITEM_DTYPE),
                 merges=view(plan.merges_offset, plan.n_merges, STREAM_MERGE_DTYPE))
+
+
+def gemm_tuning(level):
+    """sfb_gemm_tuning: 0 = time the library's short list of GEMM kernels per problem, 1 = all that support it."""
+    _check(lib.sfb_gemm_tuning(C.c_int(level)), "sfb_gemm_tuning")
 
 
 def scale_parts(scale):

@@ -8,12 +8,14 @@
 // C, n), transformer.cpp:516); the GEMM is issued column-major as C^T = W^T A^T, the same trick as the
 // reference's cuBLAS calls (transformer_attention_optimize.cu:693-716).
 #include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt-ext.hpp>
 #include <hipblaslt/hipblaslt.h>
 #include <rocblas/rocblas.h>
 
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "../../include/sfbert_hip.h"
 
@@ -53,6 +55,11 @@ typedef std::tuple<uint32_t, uint32_t, uint32_t, int, int, int, int, int> PlanKe
 std::map<PlanKey, LtPlan> g_plans;
 constexpr float kGeluSigmoidSlope = 1.702f;
 constexpr int kCandidates = 16;
+// sfb_gemm_tuning(): 0 = time the library's own short list of candidates, 1 = time every kernel of the library that
+// supports the problem (the short list is what a heuristic expects to be fast; at the layer's shapes its best entry
+// runs at about a third of the matrix peak, so the long list is worth a second or two per problem at first use)
+int g_tuning_level = 0;
+constexpr size_t kMostCandidates = 1024;
 
 void destroy_plan(LtPlan& p) {
     if (p.w) hipblasLtMatrixLayoutDestroy(p.w);
@@ -119,14 +126,35 @@ LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, in
     if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
     const uint64_t max_ws = with_ws ? ops.workspace_bytes : 0;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-    hipblasLtMatmulHeuristicResult_t results[kCandidates];
+    std::vector<hipblasLtMatmulHeuristicResult_t> results(kCandidates);
     int found = 0;
-    const bool got = hipblasLtMatmulAlgoGetHeuristic(g_lt, p.desc, p.w, p.a, p.c, p.c, pref, kCandidates, results, &found) ==
-                     HIPBLAS_STATUS_SUCCESS;
+    const bool got = hipblasLtMatmulAlgoGetHeuristic(g_lt, p.desc, p.w, p.a, p.c, p.c, pref, kCandidates, results.data(),
+                                                     &found) == HIPBLAS_STATUS_SUCCESS;
     hipblasLtMatmulPreferenceDestroy(pref);
     if (!got || found <= 0) return p;
+    results.resize((size_t)found);
+    const bool can_time = !stream_is_capturing(ops.stream) && ops.c && ops.a && ops.w;
+    if (g_tuning_level >= 1 && can_time) {
+        // every kernel the library has for these types, kept if it supports this problem within the workspace
+        std::vector<hipblasLtMatmulHeuristicResult_t> all;
+        if (hipblaslt_ext::getAllAlgos(g_lt, hipblaslt_ext::GemmType::HIPBLASLT_GEMM, none, none, in, in, out, out,
+                                       HIPBLAS_COMPUTE_32F, all) == HIPBLAS_STATUS_SUCCESS) {
+            const float one = 1.0f, zero = 0.0f;
+            for (auto& r : all) {
+                if (results.size() >= kMostCandidates) break;
+                size_t need = 0;
+                if (hipblaslt_ext::matmulIsAlgoSupported(g_lt, p.desc, &one, p.w, p.a, &zero, p.c, p.c, r.algo, need) !=
+                        HIPBLAS_STATUS_SUCCESS || need > max_ws)
+                    continue;
+                r.workspaceSize = need;
+                r.state = HIPBLAS_STATUS_SUCCESS;
+                results.push_back(r);
+            }
+        }
+        found = (int)results.size();
+    }
     int best = -1;
-    if (!stream_is_capturing(ops.stream) && ops.c && ops.a && ops.w) {
+    if (can_time) {
         // time every candidate on the caller's operands: 1 untimed + 3 timed launches each
         hipEvent_t e0 = nullptr, e1 = nullptr;
         if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
@@ -149,8 +177,8 @@ LtPlan& lt_plan(uint32_t m, uint32_t n, uint32_t k, int dtype, int out_dtype, in
             }
             p.tuned = best >= 0;
         }
-        if (e0) hipEventDestroy(e0);
-        if (e1) hipEventDestroy(e1);
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
     }
     if (best < 0)
         for (int i = 0; i < found && best < 0; ++i)
@@ -206,6 +234,13 @@ static int lt_gemm(sfb_stream_t stream, void* c, int out_dtype, const void* a, c
         return SFB_OK;
     p.usable = false;   // do not try this plan again
     return SFB_ERR_LAUNCH;
+}
+
+extern "C" int sfb_gemm_tuning(int level) {
+    if (level < 0 || level > 1) return SFB_ERR_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_tuning_level = level;   // plans already made keep their kernel until sfb_gemm_release()
+    return SFB_OK;
 }
 
 extern "C" void sfb_gemm_release(void) {
