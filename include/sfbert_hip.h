@@ -367,7 +367,8 @@ int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const voi
  * arithmetic as the reference's sequence TN, NT, softmax gradient, TN, NN (transformer_attention_optimize.cu:
  * 924-965; ewops.h:101-124; matmul.h:81-99): P = exp2(S scale log2e - lse), dV = P^T dO, dS = P (dO V^T - delta)
  * scale, dK = dS^T Q, dQ = dS K, where delta = rowsum(dO * O) (computed here into the caller's buffer) stands for
- * the gradient's sum over the sparse row.  q, k, v, d_out [dev] bf16 [batch, ctx, heads, 64]; o [dev] fp32, the
+ * the gradient's sum over the sparse row.  q, k, v, d_out [dev] bf16 or fp32 (dtype; fp32 tensors get true fp32
+ * products) [batch, ctx, heads, state_dim], state_dim 32, 64, 96 or 128; o [dev] fp32, the
  * forward output; lse [dev] from sfb_fused_attention_scheduled_lse; delta [dev] fp32 [batch][heads][ctx]
  * (scratch, overwritten); dq, dk, dv [dev] fp32; nn_lut, tn_lut [dev]: one layout for all heads (lut_heads 1), or
  * one table per head, lut_dim = ctx_blks + blocks entries apart, every head with the same number of blocks
@@ -376,8 +377,7 @@ int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const voi
  * order): work items of sfb_build_schedule over nn_lut / over tn_lut, longest first, with lines of more than
  * max_blocks blocks cut into chunks; the chunks of a split line write partial records into workspace ([dev],
  * 256-byte aligned, sfb_backward_workspace_bytes() bytes; n_*_parts as returned by sfb_build_schedule) and a
- * follow-up kernel adds them in chunk order, so results do not depend on timing.  dtype must be SFB_BF16 (fp32
- * tensors: use the unfused sequence). */
+ * follow-up kernel adds them in chunk order, so results do not depend on timing. */
 size_t sfb_backward_workspace_bytes(uint32_t n_row_parts, uint32_t n_col_parts, uint32_t batch_dim,
                                     uint32_t head_dim, uint32_t block_size, uint32_t state_dim);
 int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, const void* k, const void* v, const float* o,

@@ -14,7 +14,8 @@
 //   * dkdv kernel, one work-group per (batch, head, key-block column), a lane owns one key: per query block
 //         S = Q K^T, dP = dO V^T (row-wise reads of the Q and dO tiles; lse and delta per accumulator element),
 //         dV^T += dO^T P, dK^T += Q^T dS (transposed reads of the dO and Q tiles).
-// bf16 tensors, head size 64, block size 32 or 64; fp32 accumulation and fp32 gradients.
+// bf16 or fp32 tensors (the latter with true fp32 products, further down), head sizes 32 / 64 / 96 / 128, block
+// size 32 or 64; fp32 accumulation and fp32 gradients.
 #include "tiles.hip.h"
 
 namespace sfb {
@@ -372,6 +373,250 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void attention_backward_ker
     else attention_dq<BS, D, MASKED>(rows, blockIdx.x - col_wgs, smem);
 }
 
+// ------------------------------------------------------------------------------------------------
+// fp32 tensors: the same two halves on v_mfma_f32_32x32x2_f32 (true fp32 products), tiles staged through registers
+// into one LDS buffer each as in the fp32 forward kernel (F32Tiles; rows of D + 4 floats, read row-wise as 128-bit
+// fragments for the score-like products and element-wise down a column for the transposed ones)
+// ------------------------------------------------------------------------------------------------
+// element (row 32 kt + (i/4) 8 + 4 half + i%4, column 32 mt + qn) of a tile in the K layout of F32Tiles: the A operand
+// of a transposed product step, as F32Tiles::v_elem is for the V layout
+template <int BS, int D>
+__device__ __forceinline__ float tile_column_elem(const float* lds, int kt, int i, int mt, uint32_t qn, uint32_t half) {
+    const uint32_t row = kt * 32 + (i / 4) * 8 + half * 4 + (i % 4);
+    return lds[row * F32Tiles<BS, D>::K_STRIDE + mt * 32 + qn];
+}
+
+template <int BS, int D, bool MASKED>
+__device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32_t wg, float* k_lds, float* v_lds) {
+    using T = F32Tiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, QG = D / 8;
+
+    const LineWork work = decode_line_work(p, p.nn_lut, wg);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t r = work.line;
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t qn = lane & 31, half = lane >> 5;
+    const uint32_t q_in_block = wave * 32 + qn;
+    const uint32_t row_stride = p.heads * D;
+    const uint32_t off = work.first, count = work.count;
+    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+
+    f32x16 dq_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dq_acc[n][i] = 0.f;
+
+    if (count > 0) {
+        const float* K = (const float*)p.k;
+        const float* V = (const float*)p.v;
+        const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+        const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+        const float c = p.scale_log2e;
+
+        f32x4 qf[QG], dof[QG];
+        T::load_q(qf, (const float*)p.q + my_row, half);
+        T::load_q(dof, (const float*)p.d_out + my_row, half);
+        const size_t stat = ((size_t)work.bh * p.nb + r) * BS + q_in_block;
+        const float lse = p.lse[stat], delta = p.delta[stat];
+
+        const sfb_uint2* const nn_lut = p.nn_lut + (size_t)h * p.lut_stride;
+        typename T::Regs gk, gv;
+        sfb_uint2 entry = nn_lut[off];
+        {
+            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
+            T::fetch(gk, K, base, row_stride, t);
+            T::fetch(gv, V, base, row_stride, t);
+        }
+        for (uint32_t j = 0; j < count; ++j) {
+            const sfb_uint2 e = entry;
+            T::template stage<T::K_STRIDE>(k_lds, gk, t);
+            T::template stage<T::K_STRIDE>(v_lds, gv, t);
+            __syncthreads();
+            if (j + 1 < count) {
+                entry = nn_lut[off + j + 1];
+                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
+                T::fetch(gk, K, base, row_stride, t);
+                T::fetch(gv, V, base, row_stride, t);
+            }
+            f32x16 s[KT], dp[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { s[kt][i] = 0.f; dp[kt][i] = 0.f; }
+#pragma unroll
+            for (int g = 0; g < QG; ++g)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    const f32x4 ka = T::k_frag(k_lds, kt, g, qn, half), va = T::k_frag(v_lds, kt, g, qn, half);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[x], qf[g][x], s[kt], 0, 0, 0);
+                        dp[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va[x], dof[g][x], dp[kt], 0, 0, 0);
+                    }
+                }
+            if (MASKED) {
+                const int limit = valid - (int)(e.y * BS);
+                if ((mask != nullptr) || (limit < BS))
+                    apply_keep<KT>(s, load_keep_word<BS>(mask, (size_t)e.x * BS + q_in_block, limit), half);
+            }
+            // dS^T for this lane's query: P (dP - delta) scale; a masked score is -3e38, its probability an exact 0
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float prob = exp2_fast(__builtin_fmaf(s[kt][i], c, -lse));
+                    s[kt][i] = prob * (dp[kt][i] - delta) * p.scale;
+                }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+#pragma unroll
+                    for (int mt = 0; mt < NO; ++mt)
+                        dq_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tile_column_elem<BS, D>(k_lds, kt, i, mt, qn, half),
+                                                                          s[kt][i], dq_acc[mt], 0, 0, 0);
+            __syncthreads();   // every wave is done with the tiles before the next block is staged
+        }
+    }
+    if (work.slot < 0) store_rows_f32<NO>(p.dq + my_row, dq_acc, half);
+    else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
+}
+
+template <int BS, int D, bool MASKED>
+__device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint32_t wg, float* q_lds, float* do_lds) {
+    using T = F32Tiles<BS, D>;
+    constexpr int KT = BS / 32, NO = D / 32, QG = D / 8;
+
+    const LineWork work = decode_line_work(p, p.tn_lut, wg);
+    if (!work.valid) return;
+    const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
+    const uint32_t col = work.line;
+    const uint32_t L = p.nb * BS;
+    const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const uint32_t kn = lane & 31, half = lane >> 5;
+    const uint32_t key_in_block = wave * 32 + kn;
+    const uint32_t row_stride = p.heads * D;
+    const uint32_t off = work.first, count = work.count;
+    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, D);
+
+    f32x16 dk_acc[NO], dv_acc[NO];
+#pragma unroll
+    for (int n = 0; n < NO; ++n)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { dk_acc[n][i] = 0.f; dv_acc[n][i] = 0.f; }
+
+    if (count > 0) {
+        const float* Q = (const float*)p.q;
+        const float* DO = (const float*)p.d_out;
+        const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
+        const int valid = p.valid_len ? p.valid_len[b] : (int)L;
+        const bool key_valid = (int)(col * BS + key_in_block) < valid;
+        const float c = p.scale_log2e;
+        const float* lse_bh = p.lse + (size_t)work.bh * L;
+        const float* delta_bh = p.delta + (size_t)work.bh * L;
+
+        f32x4 kf[QG], vf[QG];   // this lane's key as the B operand of both score-like products
+        T::load_q(kf, (const float*)p.k + my_row, half);
+        T::load_q(vf, (const float*)p.v + my_row, half);
+
+        const sfb_uint2* const tn_lut = p.tn_lut + (size_t)h * p.lut_stride;
+        typename T::Regs gq, gd;
+        sfb_uint2 entry = tn_lut[off];   // {block id, row block}
+        {
+            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
+            T::fetch(gq, Q, base, row_stride, t);
+            T::fetch(gd, DO, base, row_stride, t);
+        }
+        for (uint32_t j = 0; j < count; ++j) {
+            const sfb_uint2 e = entry;
+            T::template stage<T::K_STRIDE>(q_lds, gq, t);
+            T::template stage<T::K_STRIDE>(do_lds, gd, t);
+            __syncthreads();
+            if (j + 1 < count) {
+                entry = tn_lut[off + j + 1];
+                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
+                T::fetch(gq, Q, base, row_stride, t);
+                T::fetch(gd, DO, base, row_stride, t);
+            }
+            // S[query][key], dP[query][key]: element i of tile kt is query kt*32 + (i/4)*8 + half*4 + i%4, key = lane's
+            f32x16 s[KT], dp[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { s[kt][i] = 0.f; dp[kt][i] = 0.f; }
+#pragma unroll
+            for (int g = 0; g < QG; ++g)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    const f32x4 qa = T::k_frag(q_lds, kt, g, kn, half), da = T::k_frag(do_lds, kt, g, kn, half);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[x], kf[g][x], s[kt], 0, 0, 0);
+                        dp[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(da[x], vf[g][x], dp[kt], 0, 0, 0);
+                    }
+                }
+            const float* lse_blk = lse_bh + (size_t)e.y * BS;
+            const float* delta_blk = delta_bh + (size_t)e.y * BS;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ig = 0; ig < 4; ++ig) {
+                    const uint32_t q0 = kt * 32 + ig * 8 + half * 4;
+                    const f32x4 lse4 = *(const f32x4*)(lse_blk + q0), delta4 = *(const f32x4*)(delta_blk + q0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int i = ig * 4 + x;
+                        float prob = exp2_fast(__builtin_fmaf(s[kt][i], c, -lse4[x]));
+                        if (MASKED) {
+                            bool keep = key_valid;
+                            if (mask != nullptr) {
+                                const size_t word = (size_t)e.x * BS + q0 + x;
+                                const uint64_t bits = (BS == 64) ? ((const uint64_t*)mask)[word] : ((const uint32_t*)mask)[word];
+                                keep = keep && ((bits >> key_in_block) & 1u);
+                            }
+                            prob = keep ? prob : 0.f;
+                        }
+                        s[kt][i] = prob;
+                        dp[kt][i] = prob * (dp[kt][i] - delta4[x]) * p.scale;
+                    }
+                }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+#pragma unroll
+                    for (int mt = 0; mt < NO; ++mt) {
+                        dv_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tile_column_elem<BS, D>(do_lds, kt, i, mt, kn, half),
+                                                                          s[kt][i], dv_acc[mt], 0, 0, 0);
+                        dk_acc[mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(tile_column_elem<BS, D>(q_lds, kt, i, mt, kn, half),
+                                                                          dp[kt][i], dk_acc[mt], 0, 0, 0);
+                    }
+            __syncthreads();
+        }
+    }
+    if (work.slot < 0) {
+        store_rows_f32<NO>(p.dk + my_row, dk_acc, half);
+        store_rows_f32<NO>(p.dv + my_row, dv_acc, half);
+    } else {   // partial record of a split column: dK rows, then dV rows
+        float* part = p.partials + (((size_t)work.bh * p.n_parts + work.slot) * 2 * BS + key_in_block) * D;
+        store_rows_f32<NO>(part, dk_acc, half);
+        store_rows_f32<NO>(part + (size_t)BS * D, dv_acc, half);
+    }
+}
+
+template <int BS, int D, bool MASKED>
+__global__ __launch_bounds__(BS * 2, 1) void attention_backward_f32_kernel(BackwardParams cols, BackwardParams rows,
+                                                                           uint32_t col_wgs) {
+    using T = F32Tiles<BS, D>;
+    __shared__ __attribute__((aligned(16))) float a_lds[T::K_FLOATS];
+    __shared__ __attribute__((aligned(16))) float b_lds[T::K_FLOATS];
+    if (blockIdx.x < col_wgs) attention_dkdv_f32<BS, D, MASKED>(cols, blockIdx.x, a_lds, b_lds);
+    else attention_dq_f32<BS, D, MASKED>(rows, blockIdx.x - col_wgs, a_lds, b_lds);
+}
+
 // Sum of the partial records of one split line, in chunk order (so the result does not depend on which chunk
 // finished when), written to the line's rows of the output tensors.
 template <int BS, int D, int TENSORS>
@@ -407,7 +652,7 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(float* dk, float* 
 }
 
 template <int BS, int D>
-static int launch_backward(hipStream_t stream, const BackwardParams& p, const sfb_work_item* row_items,
+static int launch_backward(hipStream_t stream, int dtype, const BackwardParams& p, const sfb_work_item* row_items,
                            uint32_t n_row_items, uint32_t n_row_heavy, uint32_t n_row_parts,
                            const sfb_work_item* col_items, uint32_t n_col_items, uint32_t n_col_heavy,
                            uint32_t n_col_parts, float* row_partials, float* col_partials) {
@@ -420,10 +665,15 @@ static int launch_backward(hipStream_t stream, const BackwardParams& p, const sf
     cols.n_parts = n_col_parts; cols.partials = col_partials;
     clear_stale_error();
     const uint32_t col_wgs = groups * 8u * cols.ranks, row_wgs = groups * 8u * rows.ranks;
-    if (masked)
-        attention_backward_kernel<BS, D, true><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
-    else
-        attention_backward_kernel<BS, D, false><<<dim3(col_wgs + row_wgs), dim3(BS * 2), 0, stream>>>(cols, rows, col_wgs);
+    const dim3 grid(col_wgs + row_wgs), block(BS * 2);
+    if (dtype == SFB_F32) {
+        if (masked) attention_backward_f32_kernel<BS, D, true><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+        else attention_backward_f32_kernel<BS, D, false><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+    } else if (masked) {
+        attention_backward_kernel<BS, D, true><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+    } else {
+        attention_backward_kernel<BS, D, false><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+    }
     const uint32_t reduce_cols = (col_items && n_col_parts) ? n_col_items : 0u;
     const uint32_t reduce_rows = (row_items && n_row_parts) ? n_row_items : 0u;
     if (reduce_cols + reduce_rows)
@@ -456,7 +706,7 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     using namespace sfb;
     if (!q || !k || !v || !o || !d_out || !lse || !delta || !dq || !dk || !dv || !nn_lut || !tn_lut)
         return SFB_ERR_NULL_POINTER;
-    if (dtype != SFB_BF16) return SFB_ERR_DTYPE;   // fp32 tensors take the unfused sequence
+    if (dtype != SFB_BF16 && dtype != SFB_F32) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
     if (state_dim != 32 && state_dim != 64 && state_dim != 96 && state_dim != 128) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
@@ -491,7 +741,7 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * state_dim;
     hipStream_t s = (hipStream_t)stream;
 #define SFB_CALL(BSV, DV)                                                                                        \
-    return launch_backward<BSV, DV>(s, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items, \
+    return launch_backward<BSV, DV>(s, dtype, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items, \
                                     n_col_heavy, n_col_parts, row_partials, col_partials)
     if (block_size == 64) {
         if (state_dim == 64) SFB_CALL(64, 64);

@@ -160,7 +160,7 @@ def test_argument_checks_of_the_newer_entry_points():
         return bwd(None, p, p, p, p, p, p, p, p, p, p, dtype, p, p, None, None, None, u32(0), u32(0), u32(0), None, u32(0),
                    u32(0), u32(0), None, C.c_size_t(0), u32(64), u32(6), u32(1), u32(4), u32(4), u32(d), u32(1), u32(10),
                    u32(1), C.c_float(-1.0))
-    assert backward(48) == 3 and backward(64, sfb.F32) == 5
+    assert backward(48) == 3 and backward(48, sfb.F32) == 3 and backward(64, 7) == 5
     assert backward(96) == 8 and backward(32) == 8 and backward(128) == 8   # size accepted; the scale is what is wrong
 
 

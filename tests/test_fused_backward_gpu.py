@@ -138,8 +138,8 @@ def test_fused_backward_per_head_tables_and_masks(bs):
     assert e.value.status == 4
 
 
-def test_fused_backward_rejects_fp32():
-    q = torch.zeros((1, 64, 1, 64), device="cuda")
+def test_fused_backward_rejects_other_dtypes():
+    q = torch.zeros((1, 64, 1, 64), device="cuda", dtype=torch.float16)
     lut = sfb.to_device(np.zeros((2, 2), np.uint32))
     with pytest.raises(sfb.SfbError) as e:
         sfb.fused_attention_backward(q, q, q, q, q, torch.zeros((1, 1, 64), device="cuda"), lut, lut, 64, 1, 0.125)

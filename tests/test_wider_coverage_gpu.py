@@ -188,6 +188,47 @@ def test_fused_backward_at_other_head_sizes(d, bs):
             assert (dq.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
 
 
+@pytest.mark.parametrize("d", [32, 64, 96, 128])
+@pytest.mark.parametrize("bs", [32, 64])
+def test_fused_backward_fp32_tensors(d, bs):
+    """fp32 Q, K, V and dO through the fused backward (true fp32 products): whole lines and lines cut into chunks,
+    with element mask and key padding, one table for all heads and one per head, to the fp32 tolerance."""
+    nb, B, H = 8, 2, 3
+    L = nb * bs
+    scale = float(1.0 / np.sqrt(d))
+    lay = PATTERNS["bigbird"](nb).copy()
+    lay[5] = 0
+    lay[:, 6] = 0
+    luts = sfb.build_luts(lay)
+    keep = (np.random.default_rng(3 * bs + d).random((luts["blocks"], bs, bs)) < 0.8).astype(np.uint8)
+    mask = sfb.pack_mask(keep)
+    valid = np.array([L, L - bs - 7], np.int32)
+    Q, K, V = qkv(B, L, H, d, seed=500 + bs + d)
+    dO = orc.fill_normal((B, L, H, d), 510)
+    q, k, v, do = (dev(x, False) for x in (Q, K, V, dO))
+    nn, tn = sfb.to_device(luts["nn_lut"]), sfb.to_device(luts["tn_lut"])
+    for masked in (False, True):
+        mk, vd = (mask, valid) if masked else (None, None)
+        m = None if mk is None else sfb.to_device(mk)
+        vl = None if vd is None else sfb.to_device(vd)
+        dQ, dK, dV, _ = orc.attention_backward(Q, K, V, dO, luts, bs, scale, mask=mk, valid_len=vd)
+        o, lse = forward(q, k, v, luts, bs, scale, mask=m, valid=vl)
+        for max_blocks in (None, 3):
+            rs = cs = None
+            if max_blocks:
+                rs, cs = sfb.build_schedule(luts["nn_lut"], nb, max_blocks), sfb.build_schedule(luts["tn_lut"], nb, max_blocks)
+                rs["items_dev"], cs["items_dev"] = sfb.to_device(rs["items"]), sfb.to_device(cs["items"])
+            dq, dk, dv = sfb.fused_attention_backward(q, k, v, o, do, lse, nn, tn, bs, luts["blocks"], scale, mask=m,
+                                                      valid_len=vl, row_sched=rs, col_sched=cs)
+            torch.cuda.synchronize()
+            for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+                got = got.cpu().numpy()
+                assert np.isfinite(got).all()
+                assert rel_err(got, want) <= TOL_F32, (name, masked, max_blocks)
+            assert (dq.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
+            assert (dk.cpu().numpy()[:, 6 * bs:7 * bs] == 0).all() and (dv.cpu().numpy()[:, 6 * bs:7 * bs] == 0).all()
+
+
 @pytest.mark.parametrize("d", [32, 96, 128])
 @pytest.mark.parametrize("bs", [32, 64])
 def test_unfused_bf16_tensors_at_other_head_sizes(d, bs):
