@@ -9,8 +9,22 @@ if ROOT not in sys.path:
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 
+def pytest_addoption(parser):
+    parser.addoption("--emulate", action="store_true",
+                     help="run the tests marked gpu without a GPU, on the host build of the kernel sources "
+                          "(tests/emu_lib.py); --emulate-order and --emulate-eager choose the lane order and when "
+                          "LDS-direct loads land")
+    parser.addoption("--emulate-order", type=int, default=0)
+    parser.addoption("--emulate-eager", action="store_true")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "needs_device: uses streams, graphs or timing that only a real device has")
+    if config.getoption("--emulate"):
+        import emu_lib
+        emu_lib.install()
+        emu_lib.configure(order=config.getoption("--emulate-order"), lazy_loads=not config.getoption("--emulate-eager"))
 
 
 def _gpu_available():
@@ -22,6 +36,12 @@ def _gpu_available():
 
 
 def pytest_collection_modifyitems(config, items):
+    if config.getoption("--emulate"):
+        skip = pytest.mark.skip(reason="needs a real device")
+        for item in items:
+            if "needs_device" in item.keywords:
+                item.add_marker(skip)
+        return
     if _gpu_available():
         return
     skip = pytest.mark.skip(reason="no GPU in this process")

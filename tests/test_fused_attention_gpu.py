@@ -301,6 +301,7 @@ def test_bf16_output_is_the_fp32_output_rounded_once(bs, max_blocks, bf16_in):
     assert rel_err(o16.float().cpu().numpy(), want) <= TOL_BF16
 
 
+@pytest.mark.needs_device
 def test_scheduled_launch_in_a_hip_graph():
     """The scheduled launch (split rows, counters reset by the kernel itself, no memset) captured into a graph:
     every replay, with eager launches and synchronisations in between, gives the eager result bit for bit."""

@@ -101,6 +101,7 @@ def test_model_forward_matches_oracle(bf16, pre_ln):
     assert model.forward(T(ids)) == {}
 
 
+@pytest.mark.needs_device
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_cpp_whole_model_host_program(dtype):
     """sf-bert_amd/host/transformer_inference: a C++ main in the shape of the reference's

@@ -244,6 +244,7 @@ def test_error_codes_instead_of_silent_no_op():
                                          u(1), u(64), u(1), u(2), u(1), C.c_float(0.125)) == 1
 
 
+@pytest.mark.needs_device
 def test_cpp_host_program_through_reference_named_launchers():
     """sf-bert_amd/host/attention_host_test: a C++ main in the shape of the reference's *_fusion_test.cu
     that calls bst_sgemm_nt / BlocksparseMaskedSoftmax / bst_sgemm_xn / fusion_attention2 / fusion_attention."""
