@@ -34,14 +34,17 @@ emu_switch:
 
 namespace emu {
 
-constexpr size_t kStackBytes = 512u << 10;   // the lowest page is inaccessible: an overflow faults
+constexpr size_t kStackBytes = 512u << 10;   // the lowest words hold a pattern that is checked when the lane ends
+constexpr uint64_t kCanary = 0x5afe57ac5afe57acull;
 constexpr size_t kLdsBytes = 160u << 10;
 
 struct Block {
     std::vector<Lane> lanes;
     dim3 idx;
     uint8_t* lds;
+    uint8_t* stacks;
     size_t lds_used;
+    uint32_t held, hold_left;
     std::map<const void*, void*> sites;
     uint32_t live;
 };
@@ -268,14 +271,34 @@ static void execute(int op, Lane* wave_lanes, const std::vector<int>& who, bool 
 
 // One pass over a work-group: runs every lane that can run, then executes what has gathered.  Returns whether
 // anything moved.
+static uint64_t g_rng;
+static uint32_t draw() {
+    g_rng = g_rng * 6364136223846793005ull + 1442695040888963407ull;
+    return (uint32_t)(g_rng >> 33);
+}
+
 static bool advance(Block& b, const std::vector<uint32_t>& order, bool force) {
     bool moved = false;
-    for (uint32_t t : order) {
-        Lane& l = b.lanes[t];
-        if (l.done || l.op != OP_NONE) continue;
-        run(l);
-        moved = true;
-        if (l.done) b.live--;
+    // shuffled orders also hold back waves at random, so that one wave can run several steps ahead of another
+    uint32_t held = 0;
+    if (g_config.order > 1 && !force) {
+        if (b.hold_left == 0) {
+            b.held = draw();   // half of the waves, on average, for one to four passes
+            b.hold_left = 1 + draw() % 4;
+        }
+        b.hold_left--;
+        held = b.held;
+    }
+    for (int pass = 0; pass < 2 && !moved; ++pass) {
+        for (uint32_t t : order) {
+            Lane& l = b.lanes[t];
+            if (l.done || l.op != OP_NONE) continue;
+            if (pass == 0 && ((held >> (l.wave & 31)) & 1)) continue;
+            run(l);
+            moved = true;
+            if (l.done) b.live--;
+        }
+        if (held == 0) break;
     }
     const uint32_t nt = (uint32_t)b.lanes.size();
     // work-group barriers: every live lane has arrived
@@ -334,15 +357,18 @@ static Block* make_block(uint32_t linear, uint32_t nt) {
     if (b->lds == (uint8_t*)MAP_FAILED) abort();
     memset(b->lds, 0xff, kLdsBytes);
     b->lds_used = 0;
+    b->held = b->hold_left = 0;
     b->live = nt;
     b->lanes.resize(nt);
+    // one mapping for all stacks of the work-group (the process may hold only so many mappings)
+    b->stacks = (uint8_t*)mmap(nullptr, nt * kStackBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
+    if (b->stacks == (uint8_t*)MAP_FAILED) abort();
     for (uint32_t t = 0; t < nt; ++t) {
         Lane& l = b->lanes[t];
         memset(&l, 0, offsetof(Lane, vm));
         l.vm_head = l.vm_count = 0;
-        l.stack = (uint8_t*)mmap(nullptr, kStackBytes, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
-        if (l.stack == (uint8_t*)MAP_FAILED) abort();
-        mprotect(l.stack, 4096, PROT_NONE);
+        l.stack = b->stacks + (size_t)t * kStackBytes;
+        for (int i = 0; i < 8; ++i) ((uint64_t*)l.stack)[i] = kCanary;
         l.block = b;
         l.tid = t;
         l.lane = t % 64;
@@ -353,7 +379,10 @@ static Block* make_block(uint32_t linear, uint32_t nt) {
 }
 
 static void free_block(Block* b) {
-    for (Lane& l : b->lanes) munmap(l.stack, kStackBytes);
+    for (Lane& l : b->lanes)
+        for (int i = 0; i < 8; ++i)
+            if (((uint64_t*)l.stack)[i] != kCanary) fail("a lane's stack overflowed (the model's, not the kernel's)");
+    munmap(b->stacks, b->lanes.size() * kStackBytes);
     munmap(b->lds, kLdsBytes);
     delete b;
 }
@@ -368,6 +397,7 @@ void launch(dim3 grid, dim3 block, size_t, hipStream_t, const std::function<void
     g_grid = grid;
     g_block_dim = block;
     g_body = &body;
+    g_rng = (uint64_t)g_config.order * 0x9E3779B97F4A7C15ull + 12345;
     std::vector<uint32_t> order(nt);
     for (uint32_t t = 0; t < nt; ++t) order[t] = g_config.order == 1 ? nt - 1 - t : t;
     if (g_config.order > 1) {

@@ -252,6 +252,7 @@ def _digest():
     h = hashlib.sha256()
     files = [os.path.join(CSRC, f) for f in KERNEL_SOURCES + HOST_SOURCES + HEADERS]
     files += [os.path.join(EMU, "hip", "hip_runtime.h"), os.path.join(EMU, "emu_runtime.cpp"), os.path.abspath(__file__),
+              os.path.join(EMU, "selftest_kernels.hip"),
               os.path.join(ROOT, "include", "sfbert_hip.h")]
     for f in files:
         h.update(open(f, "rb").read())
@@ -277,7 +278,10 @@ def build(verbose=False):
             f.write(text)
         if not name.endswith(".h"):
             units.append(target)
-    units += [os.path.join(CSRC, f) for f in HOST_SOURCES] + [os.path.join(EMU, "emu_runtime.cpp")]
+    selftest = os.path.join(gen, "selftest_kernels_emu.cpp")
+    with open(selftest, "w") as f:
+        f.write(rewrite(open(os.path.join(EMU, "selftest_kernels.hip")).read(), "selftest_kernels.hip"))
+    units += [selftest] + [os.path.join(CSRC, f) for f in HOST_SOURCES] + [os.path.join(EMU, "emu_runtime.cpp")]
     # entry points whose sources stay out (they need hipBLASLt): present, and refusing
     stubs = os.path.join(gen, "stubs_emu.cpp")
     with open(stubs, "w") as f:
@@ -381,7 +385,7 @@ def empty(shape, dtype, fill=None):
     import torch
     lib = load().lib
     n = int(np.prod(shape)) if len(shape) else 1
-    item = torch.empty((), dtype=dtype).element_size()
+    item = torch.finfo(dtype).bits // 8 if dtype.is_floating_point else torch.iinfo(dtype).bits // 8
     nbytes = max(n * item, 16)
     ptr = lib.emu_guarded_alloc(nbytes)
     assert ptr
@@ -393,14 +397,21 @@ def empty(shape, dtype, fill=None):
     return t
 
 
-def install():
+def install(monkeypatch=None):
     """Makes the tests marked gpu run on the host build: the package name resolves to the binding of the host build,
-    'device' tensors are host tensors in guarded memory, and the few torch.cuda calls the tests make are inert."""
+    'device' tensors are host tensors in guarded memory, and the few torch.cuda calls the tests make are inert.
+    With a pytest MonkeyPatch the changes to torch are undone with it (and the package name is left alone)."""
     import sys
     import torch
     mod = load()
     mod.capi = mod
-    sys.modules["sf-bert_amd"] = mod
+    if monkeypatch is None:
+        sys.modules["sf-bert_amd"] = mod
+
+        def put(owner, name, value):
+            setattr(owner, name, value)
+    else:
+        put = monkeypatch.setattr
 
     def to_guarded(t):
         if t.numel() * t.element_size() > (64 << 20):
@@ -409,13 +420,13 @@ def install():
         out.copy_(t)
         return out
 
-    torch.Tensor.cuda = lambda self, *a, **k: to_guarded(self)
-    torch.cuda.synchronize = lambda *a, **k: None
-    torch.cuda.memory_allocated = lambda *a, **k: 0
+    put(torch.Tensor, "cuda", lambda self, *a, **k: to_guarded(self))
+    put(torch.cuda, "synchronize", lambda *a, **k: None)
+    put(torch.cuda, "memory_allocated", lambda *a, **k: 0)
 
     class _Stream:
         cuda_stream = 0
-    torch.cuda.current_stream = lambda *a, **k: _Stream()
+    put(torch.cuda, "current_stream", lambda *a, **k: _Stream())
 
     def host(factory, guarded):
         def make(*args, **kwargs):
@@ -426,5 +437,5 @@ def install():
             return to_guarded(t) if (on_device and guarded) else t
         return make
     for name in ("zeros", "empty", "ones", "full", "randn", "rand", "randint", "tensor", "arange", "zeros_like", "empty_like"):
-        setattr(torch, name, host(getattr(torch, name), name != "tensor"))
+        put(torch, name, host(getattr(torch, name), name != "tensor"))
     return mod
