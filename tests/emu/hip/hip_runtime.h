@@ -40,7 +40,9 @@ struct dim3 {
 typedef void* hipStream_t;
 typedef int hipError_t;
 enum { hipSuccess = 0, hipErrorLaunchFailure = 719 };
-enum { hipMemcpyDeviceToHost = 2, hipMemcpyHostToDevice = 1 };
+enum { hipMemcpyDeviceToHost = 2, hipMemcpyHostToDevice = 1, hipMemcpyDeviceToDevice = 3 };
+typedef enum { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 } hipStreamCaptureStatus;
+typedef void* hipEvent_t;
 enum { hipDeviceAttributeMultiprocessorCount = 63 };
 
 namespace emu {
@@ -100,10 +102,22 @@ void s_waitcnt_vmcnt(int in_flight);
 inline hipError_t hipGetLastError() { return emu::last_error(); }
 inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
 inline hipError_t hipGetDeviceCount(int* n) { *n = 1; return hipSuccess; }
-inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 4; return hipSuccess; }   // 4 compute units
+inline hipError_t hipDeviceGetAttribute(int* v, int, int) { *v = 256; return hipSuccess; }   // compute units, as on the device
 template <typename F>
 inline hipError_t hipOccupancyMaxActiveBlocksPerMultiprocessor(int* n, F, int, size_t) { *n = 2; return hipSuccess; }
 inline hipError_t hipMemcpy(void* dst, const void* src, size_t n, int) { memcpy(dst, src, n); return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void* dst, const void* src, size_t n, int, hipStream_t) { memcpy(dst, src, n); return hipSuccess; }
+inline hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, int,
+                                   hipStream_t) {
+    for (size_t r = 0; r < height; ++r) memcpy((uint8_t*)dst + r * dpitch, (const uint8_t*)src + r * spitch, width);
+    return hipSuccess;
+}
+inline hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* s) { *s = hipStreamCaptureStatusNone; return hipSuccess; }
+inline hipError_t hipEventCreate(hipEvent_t* e) { *e = (void*)1; return hipSuccess; }
+inline hipError_t hipEventDestroy(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t, hipStream_t) { return hipSuccess; }
+inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+inline hipError_t hipEventElapsedTime(float* ms, hipEvent_t, hipEvent_t) { *ms = 1.0f; return hipSuccess; }
 template <typename T>
 inline hipError_t hipGetSymbolAddress(void** p, T* symbol) { *p = (void*)symbol; return hipSuccess; }
 
