@@ -109,6 +109,9 @@ def read_traffic(workload, dtype):
     return None
 
 
+RAMP_SECONDS, RAMP_BATCH = 0.3, 200   # untimed launches before the warm-up steps
+
+
 def _time(torch, fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -246,11 +249,13 @@ def time_fused_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, max_blocks
 
 
 GEMM_TUNING = 0   # what --gemm-tuning asked for (reported with the layer's numbers)
+# shape of the encoder-layer and whole-model legs (BERT-base at the length of workload c4)
+LAYER_SHAPE = {"B": 8, "L": 4096, "ffn": 3072, "vocab": 30522, "layers": 12}
 
 
 def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), steps=20):
     """One BERT-base encoder layer forward (hidden 768, FFN 3072, BigBird attention) at B8 L4096."""
-    B, L, ffn = 8, 4096, 3072
+    B, L, ffn, vocab = (LAYER_SHAPE[x] for x in ("B", "L", "ffn", "vocab"))
     n = H * d
     torch.manual_seed(1)
     w = {}
@@ -262,11 +267,12 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), s
         w[name] = torch.zeros(size, device="cuda")
     w["ln1_g"] = torch.ones(n, device="cuda")
     w["ln2_g"] = torch.ones(n, device="cuda")
-    ids = torch.randint(0, 30522, (B, L), device="cuda", dtype=torch.int32)
-    tok = torch.randn((30522, n), device="cuda") * 0.02
+    ids = torch.randint(0, vocab, (B, L), device="cuda", dtype=torch.int32)
+    tok = torch.randn((vocab, n), device="cuda") * 0.02
     pos = torch.randn((L, n), device="cuda") * 0.02
     x = sfb.embedding_lookup(tok, ids, pos).reshape(B * L, n)
-    out = {"shape": "B8 L4096 hidden 768 heads 12 ffn 3072, BigBird block 64", "gemm_flops": 2.0 * B * L * (4 * n * n + 2 * n * ffn)}
+    out = {"shape": "B%d L%d hidden %d heads %d ffn %d, BigBird block %d" % (B, L, n, H, ffn, bs),
+           "gemm_flops": 2.0 * B * L * (4 * n * n + 2 * n * ffn)}
     out["gemm_tuning"] = GEMM_TUNING
     y = torch.empty_like(x)
     attn_flops = luts["blocks"] * B * H * 4.0 * bs * bs * d
@@ -288,7 +294,7 @@ def time_layer(sfb, torch, luts, bs, H, d, max_blocks, dtypes=("bf16", "f32"), s
 def time_model(sfb, torch, luts, bs, H, d, max_blocks):
     """Forward pass of a whole BERT-base sized model (12 layers, hidden 768, FFN 3072, BigBird attention) with
     tied-embedding logits and cross-entropy loss over a 30522-token vocabulary at B8 L4096."""
-    B, L, ffn, vocab, n_layers = 8, 4096, 3072, 30522, 12
+    B, L, ffn, vocab, n_layers = (LAYER_SHAPE[x] for x in ("B", "L", "ffn", "vocab", "layers"))
     n = H * d
     torch.manual_seed(2)
     layers = []
@@ -307,7 +313,8 @@ def time_model(sfb, torch, luts, bs, H, d, max_blocks):
     pos = torch.randn((L, n), device="cuda") * 0.02
     ids = torch.randint(0, vocab, (B, L), device="cuda", dtype=torch.int32)
     labels = torch.randint(0, vocab, (B * L,), device="cuda", dtype=torch.int32)
-    out = {"shape": "B8 L4096, 12 layers hidden 768 heads 12 ffn 3072, BigBird block 64, vocab 30522, post-LN",
+    out = {"shape": "B%d L%d, %d layers hidden %d heads %d ffn %d, BigBird block %d, vocab %d, post-LN"
+                    % (B, L, n_layers, n, H, ffn, bs, vocab),
            "gemm_flops": 2.0 * B * L * (n_layers * (4 * n * n + 2 * n * ffn) + n * vocab)}
     for name, code in (("bf16", sfb.BF16), ("f32", sfb.F32)):
         model = sfb.Model(tok, pos, layers, luts, bs, H, d, ffn, dtype=code, max_blocks=max_blocks, pre_ln=False)
@@ -409,9 +416,9 @@ def main():
         torch.cuda.synchronize()
 
     # untimed: bring the clocks up before the warm-up steps (a handful of 50 us launches does not)
-    ramp_until = time.perf_counter() + 0.3
+    ramp_until = time.perf_counter() + RAMP_SECONDS
     while time.perf_counter() < ramp_until:
-        for _ in range(200):
+        for _ in range(RAMP_BATCH):
             step()
         torch.cuda.synchronize()
     for _ in range(args.warmup):
@@ -466,9 +473,7 @@ def main():
             extra("streamed", time_streamed, sfb, torch, luts, q, k, v, bs, blocks, scale, flops, peak)
         extra("unfused", time_unfused, sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
         extra("backward_unfused", time_backward, sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
-        if bf16:
-            extra("backward_fused", time_fused_backward, sfb, torch, luts, q, k, v, bs, blocks, scale, args.max_blocks,
-                  flops)
+        extra("backward_fused", time_fused_backward, sfb, torch, luts, q, k, v, bs, blocks, scale, args.max_blocks, flops)
         if args.workload == "c4":
             # the layer and the model run eight sequences: their own chunk length
             layer_blocks = sfb.suggest_max_blocks(luts["nn_lut"], nb, 8 * H) if auto_blocks else args.max_blocks

@@ -302,27 +302,53 @@ def build(verbose=False):
     # linked under another name and moved into place: a process that has the old library loaded keeps it
     subprocess.check_call([CLANG, "-shared", "-o", LIB + ".new"] + objects + ["-lm"])
     os.replace(LIB + ".new", LIB)
+    with open(os.path.join(BUILD, "objects"), "w") as f:
+        f.write("\n".join(objects))
     with open(stamp, "w") as f:
         f.write(digest)
     return LIB
 
 
+def build_variant(tag, defines, source="fused_attention.hip"):
+    """The host build with one kernel source compiled under other preprocessor definitions (the opt-in kernel
+    variants of sf-bert_amd/build.py): tests/_build/emu/libsfbert_emu_<tag>.so."""
+    build()
+    lib = os.path.join(BUILD, "libsfbert_emu_%s.so" % tag)
+    stamp = os.path.join(BUILD, "digest_" + tag)
+    digest = _digest() + " " + " ".join(defines)
+    if os.path.exists(lib) and os.path.exists(stamp) and open(stamp).read() == digest:
+        return lib
+    src = os.path.join(BUILD, "sf-bert_amd", "csrc", source.replace(".hip", "_emu.cpp"))
+    obj = os.path.join(BUILD, "%s_%s.o" % (os.path.basename(src), tag))
+    flags = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma",
+             "-mf16c"] + ["-D" + d for d in defines]
+    subprocess.check_call([CLANG, "-x", "c++"] + flags + ["-c", src, "-o", obj])
+    others = [o for o in open(os.path.join(BUILD, "objects")).read().split("\n")
+              if os.path.basename(o) != os.path.basename(src) + ".o"]
+    subprocess.check_call([CLANG, "-shared", "-o", lib + ".new", obj] + others + ["-lm"])
+    os.replace(lib + ".new", lib)
+    with open(stamp, "w") as f:
+        f.write(digest)
+    return lib
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # use
 # ---------------------------------------------------------------------------------------------------------------
-_module = None
+_modules = {}
 
 
-def load():
-    """The package's ctypes binding (capi.py), bound to the host build instead of libsfbert_hip.so."""
-    global _module
-    if _module is not None:
-        return _module
-    lib_path = build()
+def load(tag="", defines=()):
+    """The package's ctypes binding (capi.py), bound to the host build instead of libsfbert_hip.so (tag, defines: to
+    a variant of it, see build_variant)."""
+    if tag in _modules:
+        return _modules[tag]
+    lib_path = build_variant(tag, defines) if tag else build()
     saved = os.environ.get("SFBERT_HIP_LIB")
     os.environ["SFBERT_HIP_LIB"] = lib_path
     try:
-        spec = importlib.util.spec_from_file_location("sfb_emulated", os.path.join(ROOT, "sf-bert_amd", "capi.py"))
+        spec = importlib.util.spec_from_file_location("sfb_emulated" + ("_" + tag if tag else ""),
+                                                      os.path.join(ROOT, "sf-bert_amd", "capi.py"))
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
     finally:
@@ -331,7 +357,6 @@ def load():
         else:
             os.environ["SFBERT_HIP_LIB"] = saved
     mod._stream = lambda: None
-    import torch
     mod.to_device = lambda a: tensor(np.ascontiguousarray(a).view(np.uint8).reshape(-1))
     lib = mod.lib
     lib.emu_guarded_alloc.restype = C.c_void_p
@@ -339,12 +364,16 @@ def load():
     lib.emu_message.restype = C.c_char_p
     lib.emu_count.restype = C.c_uint64
     lib.emu_partial_count.restype = C.c_uint64
-    _module = mod
+    _modules[tag] = mod
     return mod
 
 
 def configure(order=0, lazy_loads=True, resident=64):
-    load().lib.emu_configure(int(order), int(bool(lazy_loads)), int(resident))
+    """Lane order (0 ascending, 1 descending, n > 1 shuffled with seed n and waves held back at random), whether
+    LDS-direct loads land only at the wait that asks for them, and the work-groups in flight; for every build loaded."""
+    load()
+    for mod in _modules.values():
+        mod.lib.emu_configure(int(order), int(bool(lazy_loads)), int(resident))
 
 
 def counts():

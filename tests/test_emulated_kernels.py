@@ -225,3 +225,33 @@ def test_scheduled_launch_with_one_table_per_head(E):
     got = E.fused_attention_scheduled_heads(q, k, v, E.to_device(nn), E.to_device(sched["items"]), sched, ws, bs, blocks,
                                             0.125, mask=E.to_device(mask), mask_heads=H).numpy()
     assert rel_err(got, want) <= TOL[True], emu_lib.message()
+
+
+@pytest.mark.parametrize("tag,define", [("once", "SFB_TILE_LOAD_ONCE=1"), ("staged", "SFB_TILE_LOAD_STAGED=1")])
+def test_tile_load_variants_of_the_bf16_loop(E, tag, define):
+    """The two opt-in forms of the bf16 tile loads (one group of loads per tile with the steps in the instruction
+    offsets; tiles staged through registers) give the same results as the default form, bit for bit, and agree with
+    the oracle: plain and scheduled launches, lean and general loop."""
+    variant = emu_lib.load(tag, (define,))
+    bs, nb, B, H, d = 64, 5, 1, 2, 64
+    luts = E.build_luts(layout(E, nb))
+    mask, valid = masks(E, luts, bs, nb * bs, B, 5)
+    Q, K, V = inputs(B, nb * bs, H, d, 140, True)
+    q, k, v = (dev(x, True) for x in (Q, K, V))
+    nn = E.to_device(luts["nn_lut"])
+    sched = E.build_schedule(luts["nn_lut"], nb, 2)
+    items = E.to_device(sched["items"])
+    for order, lazy in (MODES[0], MODES[3]):
+        emu_lib.configure(order=order, lazy_loads=lazy)
+        for m, vl in ((None, None), (mask, valid)):
+            md, vd = (None if m is None else E.to_device(m)), (None if vl is None else E.to_device(vl))
+            want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, mask=m, valid_len=vl)
+            outs = []
+            for mod in (E, variant):
+                plain = mod.fused_attention(q, k, v, nn, bs, luts["blocks"], 0.125, mask=md, valid_len=vd).numpy()
+                ws = zeros(E.schedule_workspace_bytes(sched, B, H, bs, d))
+                cut = mod.fused_attention_scheduled(q, k, v, nn, items, sched, ws, bs, luts["blocks"], 0.125, mask=md,
+                                                    valid_len=vd).numpy()
+                outs.append((plain, cut))
+            assert rel_err(outs[1][0], want) <= TOL[True] and rel_err(outs[1][1], want) <= TOL[True]
+            assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
