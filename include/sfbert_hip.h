@@ -245,15 +245,14 @@ uint32_t sfb_resident_work_groups(void);
  * Device entry points
  * ============================================================================================== */
 
-/* state_dim (the head size d).  The fused forward entry points (sfb_fused_attention*, and the encoder layer
- * through them) take 32, 64, 96 and 128 with fp32 and with bf16 tensors, on every launch form; plain and scheduled
- * launches also take every other multiple of 4 (fp32) or 8 (bf16: rows are whole 16-byte vectors) up to 128 -- the
- * reference's `d % 4 == 0` -- through the kernel of the next multiple of 32 with zero-padded queries (streamed
- * launches return SFB_ERR_HEAD_STATE for those); the products of the unfused path
- * (sfb_sdd_nt, sfb_dsd_xn and the kernels made of them) take 32, 64, 96 and 128 with either type -- the
- * reference's K64 = false paths,
- * openai_blocksparse.h:221-222; the fused backward takes 32, 64, 96 and 128 (bf16).  Anything else returns
- * SFB_ERR_HEAD_STATE. */
+/* state_dim (the head size d).  Every attention entry point takes every multiple of 4 (fp32 tensors) or 8 (bf16
+ * tensors: rows are whole 16-byte vectors) up to 128 -- the reference's `d % 4 == 0` of its K64 = false paths,
+ * openai_blocksparse.h:221-222: the fused forward (plain and scheduled launches), the products of the unfused path
+ * (sfb_sdd_nt, sfb_dsd_xn, sfb_fused_sdd_softmax, sfb_sdd_softmax_grad, sfb_row_dot) and the fused backward.  32, 64,
+ * 96 and 128 are what the kernels' tiles divide; a size between them runs the kernel of the next multiple of 32 with
+ * the missing features read as zeros and only d output columns stored.  Streamed launches
+ * (sfb_fused_attention_streamed, sfb_encoder_layer_forward_streamed) and sfb_fused_sdd_softmax_split take the
+ * multiples of 32 / 64 only.  Anything else returns SFB_ERR_HEAD_STATE. */
 
 /* Fully fused attention: O = softmax_rows(scale * Q K^T restricted to layout & mask & key<valid_len) V,
  * one work-group per (batch, head, block-row), no S/P in memory.  Replaces the sequence
@@ -368,7 +367,7 @@ int sfb_stream_status(const sfb_stream_plan* plan, uint32_t state_dim, const voi
  * 924-965; ewops.h:101-124; matmul.h:81-99): P = exp2(S scale log2e - lse), dV = P^T dO, dS = P (dO V^T - delta)
  * scale, dK = dS^T Q, dQ = dS K, where delta = rowsum(dO * O) (computed here into the caller's buffer) stands for
  * the gradient's sum over the sparse row.  q, k, v, d_out [dev] bf16 or fp32 (dtype; fp32 tensors get true fp32
- * products) [batch, ctx, heads, state_dim], state_dim 32, 64, 96 or 128; o [dev] fp32, the
+ * products) [batch, ctx, heads, state_dim], state_dim a multiple of 8 (bf16) or 4 (fp32) up to 128; o [dev] fp32, the
  * forward output; lse [dev] from sfb_fused_attention_scheduled_lse; delta [dev] fp32 [batch][heads][ctx]
  * (scratch, overwritten); dq, dk, dv [dev] fp32; nn_lut, tn_lut [dev]: one layout for all heads (lut_heads 1), or
  * one table per head, lut_dim = ctx_blks + blocks entries apart, every head with the same number of blocks

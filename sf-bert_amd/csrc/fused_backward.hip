@@ -38,6 +38,7 @@ struct BackwardParams {
     float* partials;            // partial results of split rows / columns, or nullptr
     uint32_t ranks, heavy, n_parts;
     uint32_t batch, heads, nb, blocks, mask_stride;
+    uint32_t state;             // head size of the tensors (the kernels' D is the next multiple of 32)
     uint32_t lut_stride;        // entries between the tables of consecutive heads, 0: one table for all
     float scale, scale_log2e;
 };
@@ -91,6 +92,18 @@ __device__ __forceinline__ void store_rows_f32(float* row, const f32x16 (&acc)[N
         }
 }
 
+// rows of hd < NO * 32 floats (hd a multiple of 4): the columns beyond hd are dropped
+template <int NO>
+__device__ __forceinline__ void store_rows_f32_ragged(float* row, const f32x16 (&acc)[NO], uint32_t half, uint32_t hd) {
+#pragma unroll
+    for (int mt = 0; mt < NO; ++mt)
+#pragma unroll
+        for (int ig = 0; ig < 4; ++ig) {
+            const f32x4 out = {acc[mt][ig * 4 + 0], acc[mt][ig * 4 + 1], acc[mt][ig * 4 + 2], acc[mt][ig * 4 + 3]};
+            if (mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(row + mt * 32 + ig * 8 + half * 4) = out;
+        }
+}
+
 // The same rows to an output tensor through a wave-private LDS slab (32 rows of D floats + 16 bytes each), so that
 // memory sees whole 256-byte rows as streaming stores instead of 32-byte pieces of 32 rows per instruction: the
 // gradients are written once and read by nobody in this launch.  my_row: this lane's row; row_floats: distance
@@ -120,7 +133,10 @@ __device__ __forceinline__ void store_rows_slab(float* my_row, uint32_t row_floa
 // dQ: row owner
 // ------------------------------------------------------------------------------------------------
 // wg: index of the work-group among those of this part of the launch; smem: 4 tiles (K0 K1 V0 V1)
-template <int BS, int D, bool MASKED>
+// RAGGED: tensors with rows of hd = p.state < D elements.  The query-side operands are loaded with zeros in place of
+// the missing features, so whatever the tiles hold there (other features of the same rows) drops out of the
+// score-like products; in the transposed products it only reaches output columns that are not stored.
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t wg, uint8_t* smem) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
@@ -133,9 +149,10 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_bytes = p.heads * D * 2;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_bytes = p.heads * hd * 2;
     const uint32_t off = __builtin_amdgcn_readfirstlane(work.first), count = __builtin_amdgcn_readfirstlane(work.count);
-    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, hd);
 
     f32x16 dq_acc[NO];
 #pragma unroll
@@ -144,10 +161,10 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
         for (int i = 0; i < 16; ++i) dq_acc[n][i] = 0.f;
 
     if (count > 0) {
-        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
+        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, hd) * 2;
         const uint8_t* const k_base = (const uint8_t*)p.k + bh_bytes;
         const uint8_t* const v_base = (const uint8_t*)p.v + bh_bytes;
-        const typename T::Sources src = T::sources(lane, row_bytes);
+        const typename T::Sources src = RAGGED ? T::sources_ragged(lane, row_bytes, hd) : T::sources(lane, row_bytes);
         const uint32_t lds0 = T::lds_address(smem);
         const uint32_t k_lane = T::k_lane_base(qn, half), v_lane = T::v_lane_base(lane);
         const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
@@ -155,8 +172,13 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
         const float c = p.scale_log2e;
 
         bf16x8 qf[KS], dof[KS];
-        T::load_q(qf, (const __bf16*)p.q + my_row, half);
-        T::load_q(dof, (const __bf16*)p.d_out + my_row, half);
+        if constexpr (RAGGED) {
+            T::load_q_ragged(qf, (const __bf16*)p.q + my_row, half, hd);
+            T::load_q_ragged(dof, (const __bf16*)p.d_out + my_row, half, hd);
+        } else {
+            T::load_q(qf, (const __bf16*)p.q + my_row, half);
+            T::load_q(dof, (const __bf16*)p.d_out + my_row, half);
+        }
         const size_t stat = ((size_t)work.bh * p.nb + r) * BS + q_in_block;
         const float lse = p.lse[stat], delta = p.delta[stat];
 
@@ -165,8 +187,8 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
             return u;
         };
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
-            T::load_tile_all(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
-            T::load_tile_all(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::template load_tile_all<RAGGED>(lds0 + buf * TILE, k_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::template load_tile_all<RAGGED>(lds0 + (2 + buf) * TILE, v_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
         };
         const sfb_uint2* const nn_lut = p.nn_lut + (size_t)h * p.lut_stride;
         sfb_uint2 e = uniform(nn_lut[off]);
@@ -221,7 +243,8 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
         // memory carries the output slabs now
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        store_rows_slab<NO>(p.dq + my_row, p.heads * D, dq_acc, lane, smem + wave * (32 * (D * 4 + 16)));
+        if constexpr (RAGGED) store_rows_f32_ragged<NO>(p.dq + my_row, dq_acc, half, hd);
+        else store_rows_slab<NO>(p.dq + my_row, p.heads * D, dq_acc, lane, smem + wave * (32 * (D * 4 + 16)));
     } else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
 }
 
@@ -229,7 +252,7 @@ __device__ __forceinline__ void attention_dq(const BackwardParams& p, uint32_t w
 // dK, dV: column owner
 // ------------------------------------------------------------------------------------------------
 // wg: index of the work-group among those of this part of the launch; smem: 4 tiles (Q0 Q1 dO0 dO1)
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t wg, uint8_t* smem) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, KS = D / 16, PU = BS / 16, TILE = T::TILE_BYTES;
@@ -242,9 +265,10 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t kn = lane & 31, half = lane >> 5;
     const uint32_t key_in_block = wave * 32 + kn;
-    const uint32_t row_bytes = p.heads * D * 2;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_bytes = p.heads * hd * 2;
     const uint32_t off = __builtin_amdgcn_readfirstlane(work.first), count = __builtin_amdgcn_readfirstlane(work.count);
-    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, D);
+    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, hd);
 
     f32x16 dk_acc[NO], dv_acc[NO];
 #pragma unroll
@@ -253,10 +277,10 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
         for (int i = 0; i < 16; ++i) { dk_acc[n][i] = 0.f; dv_acc[n][i] = 0.f; }
 
     if (count > 0) {
-        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, D) * 2;
+        const size_t bh_bytes = token_offset(b, 0, h, L, p.heads, hd) * 2;
         const uint8_t* const q_base = (const uint8_t*)p.q + bh_bytes;
         const uint8_t* const do_base = (const uint8_t*)p.d_out + bh_bytes;
-        const typename T::Sources src = T::sources(lane, row_bytes);
+        const typename T::Sources src = RAGGED ? T::sources_ragged(lane, row_bytes, hd) : T::sources(lane, row_bytes);
         const uint32_t lds0 = T::lds_address(smem);
         const uint32_t k_lane = T::k_lane_base(kn, half), v_lane = T::v_lane_base(lane);
         const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
@@ -267,16 +291,21 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
         const float* delta_bh = p.delta + (size_t)work.bh * L;
 
         bf16x8 kf[KS], vf[KS];   // this lane's key as the B operand of both score-like products
-        T::load_q(kf, (const __bf16*)p.k + my_row, half);
-        T::load_q(vf, (const __bf16*)p.v + my_row, half);
+        if constexpr (RAGGED) {
+            T::load_q_ragged(kf, (const __bf16*)p.k + my_row, half, hd);
+            T::load_q_ragged(vf, (const __bf16*)p.v + my_row, half, hd);
+        } else {
+            T::load_q(kf, (const __bf16*)p.k + my_row, half);
+            T::load_q(vf, (const __bf16*)p.v + my_row, half);
+        }
 
         auto uniform = [](const sfb_uint2 e) -> sfb_uint2 {
             const sfb_uint2 u = {(uint32_t)__builtin_amdgcn_readfirstlane(e.x), (uint32_t)__builtin_amdgcn_readfirstlane(e.y)};
             return u;
         };
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {   // e = {block id, row block}
-            T::load_tile_all(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
-            T::load_tile_all(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::template load_tile_all<RAGGED>(lds0 + buf * TILE, q_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
+            T::template load_tile_all<RAGGED>(lds0 + (2 + buf) * TILE, do_base + (size_t)e.y * BS * row_bytes, wave, src, row_bytes);
         };
         const sfb_uint2* const tn_lut = p.tn_lut + (size_t)h * p.lut_stride;
         sfb_uint2 e = uniform(tn_lut[off]);
@@ -349,8 +378,13 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         uint8_t* const slab = smem + wave * (32 * (D * 4 + 16));
-        store_rows_slab<NO>(p.dk + my_row, p.heads * D, dk_acc, lane, slab);
-        store_rows_slab<NO>(p.dv + my_row, p.heads * D, dv_acc, lane, slab);
+        if constexpr (RAGGED) {
+            store_rows_f32_ragged<NO>(p.dk + my_row, dk_acc, half, hd);
+            store_rows_f32_ragged<NO>(p.dv + my_row, dv_acc, half, hd);
+        } else {
+            store_rows_slab<NO>(p.dk + my_row, p.heads * D, dk_acc, lane, slab);
+            store_rows_slab<NO>(p.dv + my_row, p.heads * D, dv_acc, lane, slab);
+        }
     } else {   // partial record of a split column: dK rows, then dV rows
         float* part = p.partials + (((size_t)work.bh * p.n_parts + work.slot) * 2 * BS + key_in_block) * D;
         store_rows_f32<NO>(part, dk_acc, half);
@@ -365,12 +399,12 @@ __device__ __forceinline__ void attention_dkdv(const BackwardParams& p, uint32_t
 // items, so they go first), the others own query rows (dQ).  As two launches, the second waits until the last
 // work-group of the first is done; as one, its work-groups fill the slots as the first's drain.  col_wgs is a
 // multiple of 8, so both halves see the same work-group -> XCD assignment as a launch of their own.
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void attention_backward_kernel(BackwardParams cols, BackwardParams rows,
                                                                        uint32_t col_wgs) {
     __shared__ __attribute__((aligned(1024))) uint8_t smem[4 * Bf16DirectTiles<BS, D>::TILE_BYTES];
-    if (blockIdx.x < col_wgs) attention_dkdv<BS, D, MASKED>(cols, blockIdx.x, smem);
-    else attention_dq<BS, D, MASKED>(rows, blockIdx.x - col_wgs, smem);
+    if (blockIdx.x < col_wgs) attention_dkdv<BS, D, MASKED, RAGGED>(cols, blockIdx.x, smem);
+    else attention_dq<BS, D, MASKED, RAGGED>(rows, blockIdx.x - col_wgs, smem);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -386,7 +420,7 @@ __device__ __forceinline__ float tile_column_elem(const float* lds, int kt, int 
     return lds[row * F32Tiles<BS, D>::K_STRIDE + mt * 32 + qn];
 }
 
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32_t wg, float* k_lds, float* v_lds) {
     using T = F32Tiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, QG = D / 8;
@@ -399,9 +433,14 @@ __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_stride = p.heads * hd;
     const uint32_t off = work.first, count = work.count;
-    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+    const size_t my_row = token_offset(b, r * BS + q_in_block, h, L, p.heads, hd);
+    auto fetch = [&](typename T::Regs& regs, const float* X, size_t base) {   // missing features of short rows: zeros
+        if constexpr (RAGGED) T::fetch_ragged(regs, X, base, row_stride, t, hd);
+        else T::fetch(regs, X, base, row_stride, t);
+    };
 
     f32x16 dq_acc[NO];
 #pragma unroll
@@ -417,8 +456,13 @@ __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32
         const float c = p.scale_log2e;
 
         f32x4 qf[QG], dof[QG];
-        T::load_q(qf, (const float*)p.q + my_row, half);
-        T::load_q(dof, (const float*)p.d_out + my_row, half);
+        if constexpr (RAGGED) {
+            T::load_q_ragged(qf, (const float*)p.q + my_row, half, hd);
+            T::load_q_ragged(dof, (const float*)p.d_out + my_row, half, hd);
+        } else {
+            T::load_q(qf, (const float*)p.q + my_row, half);
+            T::load_q(dof, (const float*)p.d_out + my_row, half);
+        }
         const size_t stat = ((size_t)work.bh * p.nb + r) * BS + q_in_block;
         const float lse = p.lse[stat], delta = p.delta[stat];
 
@@ -426,9 +470,9 @@ __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32
         typename T::Regs gk, gv;
         sfb_uint2 entry = nn_lut[off];
         {
-            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
-            T::fetch(gk, K, base, row_stride, t);
-            T::fetch(gv, V, base, row_stride, t);
+            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, hd);
+            fetch(gk, K, base);
+            fetch(gv, V, base);
         }
         for (uint32_t j = 0; j < count; ++j) {
             const sfb_uint2 e = entry;
@@ -437,9 +481,9 @@ __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32
             __syncthreads();
             if (j + 1 < count) {
                 entry = nn_lut[off + j + 1];
-                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
-                T::fetch(gk, K, base, row_stride, t);
-                T::fetch(gv, V, base, row_stride, t);
+                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, hd);
+                fetch(gk, K, base);
+                fetch(gv, V, base);
             }
             f32x16 s[KT], dp[KT];
 #pragma unroll
@@ -481,11 +525,13 @@ __device__ __forceinline__ void attention_dq_f32(const BackwardParams& p, uint32
             __syncthreads();   // every wave is done with the tiles before the next block is staged
         }
     }
-    if (work.slot < 0) store_rows_f32<NO>(p.dq + my_row, dq_acc, half);
-    else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
+    if (work.slot < 0) {
+        if constexpr (RAGGED) store_rows_f32_ragged<NO>(p.dq + my_row, dq_acc, half, hd);
+        else store_rows_f32<NO>(p.dq + my_row, dq_acc, half);
+    } else store_rows_f32<NO>(p.partials + (((size_t)work.bh * p.n_parts + work.slot) * BS + q_in_block) * D, dq_acc, half);
 }
 
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint32_t wg, float* q_lds, float* do_lds) {
     using T = F32Tiles<BS, D>;
     constexpr int KT = BS / 32, NO = D / 32, QG = D / 8;
@@ -498,9 +544,14 @@ __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const uint32_t kn = lane & 31, half = lane >> 5;
     const uint32_t key_in_block = wave * 32 + kn;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_stride = p.heads * hd;
     const uint32_t off = work.first, count = work.count;
-    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, D);
+    const size_t my_row = token_offset(b, col * BS + key_in_block, h, L, p.heads, hd);
+    auto fetch = [&](typename T::Regs& regs, const float* X, size_t base) {
+        if constexpr (RAGGED) T::fetch_ragged(regs, X, base, row_stride, t, hd);
+        else T::fetch(regs, X, base, row_stride, t);
+    };
 
     f32x16 dk_acc[NO], dv_acc[NO];
 #pragma unroll
@@ -519,16 +570,21 @@ __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint
         const float* delta_bh = p.delta + (size_t)work.bh * L;
 
         f32x4 kf[QG], vf[QG];   // this lane's key as the B operand of both score-like products
-        T::load_q(kf, (const float*)p.k + my_row, half);
-        T::load_q(vf, (const float*)p.v + my_row, half);
+        if constexpr (RAGGED) {
+            T::load_q_ragged(kf, (const float*)p.k + my_row, half, hd);
+            T::load_q_ragged(vf, (const float*)p.v + my_row, half, hd);
+        } else {
+            T::load_q(kf, (const float*)p.k + my_row, half);
+            T::load_q(vf, (const float*)p.v + my_row, half);
+        }
 
         const sfb_uint2* const tn_lut = p.tn_lut + (size_t)h * p.lut_stride;
         typename T::Regs gq, gd;
         sfb_uint2 entry = tn_lut[off];   // {block id, row block}
         {
-            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
-            T::fetch(gq, Q, base, row_stride, t);
-            T::fetch(gd, DO, base, row_stride, t);
+            const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, hd);
+            fetch(gq, Q, base);
+            fetch(gd, DO, base);
         }
         for (uint32_t j = 0; j < count; ++j) {
             const sfb_uint2 e = entry;
@@ -537,9 +593,9 @@ __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint
             __syncthreads();
             if (j + 1 < count) {
                 entry = tn_lut[off + j + 1];
-                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, D);
-                T::fetch(gq, Q, base, row_stride, t);
-                T::fetch(gd, DO, base, row_stride, t);
+                const size_t base = token_offset(b, entry.y * BS, h, L, p.heads, hd);
+                fetch(gq, Q, base);
+                fetch(gd, DO, base);
             }
             // S[query][key], dP[query][key]: element i of tile kt is query kt*32 + (i/4)*8 + half*4 + i%4, key = lane's
             f32x16 s[KT], dp[KT];
@@ -598,8 +654,13 @@ __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint
         }
     }
     if (work.slot < 0) {
-        store_rows_f32<NO>(p.dk + my_row, dk_acc, half);
-        store_rows_f32<NO>(p.dv + my_row, dv_acc, half);
+        if constexpr (RAGGED) {
+            store_rows_f32_ragged<NO>(p.dk + my_row, dk_acc, half, hd);
+            store_rows_f32_ragged<NO>(p.dv + my_row, dv_acc, half, hd);
+        } else {
+            store_rows_f32<NO>(p.dk + my_row, dk_acc, half);
+            store_rows_f32<NO>(p.dv + my_row, dv_acc, half);
+        }
     } else {   // partial record of a split column: dK rows, then dV rows
         float* part = p.partials + (((size_t)work.bh * p.n_parts + work.slot) * 2 * BS + key_in_block) * D;
         store_rows_f32<NO>(part, dk_acc, half);
@@ -607,21 +668,21 @@ __device__ __forceinline__ void attention_dkdv_f32(const BackwardParams& p, uint
     }
 }
 
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, 1) void attention_backward_f32_kernel(BackwardParams cols, BackwardParams rows,
                                                                            uint32_t col_wgs) {
     using T = F32Tiles<BS, D>;
     __shared__ __attribute__((aligned(16))) float a_lds[T::K_FLOATS];
     __shared__ __attribute__((aligned(16))) float b_lds[T::K_FLOATS];
-    if (blockIdx.x < col_wgs) attention_dkdv_f32<BS, D, MASKED>(cols, blockIdx.x, a_lds, b_lds);
-    else attention_dq_f32<BS, D, MASKED>(rows, blockIdx.x - col_wgs, a_lds, b_lds);
+    if (blockIdx.x < col_wgs) attention_dkdv_f32<BS, D, MASKED, RAGGED>(cols, blockIdx.x, a_lds, b_lds);
+    else attention_dq_f32<BS, D, MASKED, RAGGED>(rows, blockIdx.x - col_wgs, a_lds, b_lds);
 }
 
 // Sum of the partial records of one split line, in chunk order (so the result does not depend on which chunk
 // finished when), written to the line's rows of the output tensors.
 template <int BS, int D, int TENSORS>
 __device__ __forceinline__ void reduce_line(float* out0, float* out1, const float* partials, const sfb_work_item& it,
-                                            uint32_t n_parts, uint32_t bh, uint32_t heads, uint32_t ctx) {
+                                            uint32_t n_parts, uint32_t bh, uint32_t heads, uint32_t ctx, uint32_t hd) {
     const uint32_t b = bh / heads, h = bh % heads;
     constexpr int VECS = BS * D / 4;
     for (int tensor = 0; tensor < TENSORS; ++tensor) {
@@ -631,7 +692,7 @@ __device__ __forceinline__ void reduce_line(float* out0, float* out1, const floa
             f32x4 sum = {0.f, 0.f, 0.f, 0.f};
             for (uint32_t ch = 0; ch < it.nchunks; ++ch)
                 sum += *(const f32x4*)(partials + ((((size_t)bh * n_parts + it.part + ch) * TENSORS + tensor) * BS + row) * D + c4 * 4);
-            *(f32x4*)(out + token_offset(b, it.row * BS + row, h, ctx, heads, D) + c4 * 4) = sum;
+            if (c4 * 4 < hd) *(f32x4*)(out + token_offset(b, it.row * BS + row, h, ctx, heads, hd) + c4 * 4) = sum;
         }
     }
 }
@@ -643,12 +704,12 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(float* dk, float* 
                                                               const float* row_partials, const sfb_work_item* col_items,
                                                               const sfb_work_item* row_items, uint32_t n_col_items,
                                                               uint32_t n_col_parts, uint32_t n_row_parts, uint32_t heads,
-                                                              uint32_t ctx) {
+                                                              uint32_t ctx, uint32_t hd) {
     const bool column = blockIdx.x < n_col_items;
     const sfb_work_item it = column ? col_items[blockIdx.x] : row_items[blockIdx.x - n_col_items];
     if (it.nchunks <= 1 || it.chunk != 0) return;
-    if (column) reduce_line<BS, D, 2>(dk, dv, col_partials, it, n_col_parts, blockIdx.y, heads, ctx);
-    else reduce_line<BS, D, 1>(dq, nullptr, row_partials, it, n_row_parts, blockIdx.y, heads, ctx);
+    if (column) reduce_line<BS, D, 2>(dk, dv, col_partials, it, n_col_parts, blockIdx.y, heads, ctx, hd);
+    else reduce_line<BS, D, 1>(dq, nullptr, row_partials, it, n_row_parts, blockIdx.y, heads, ctx, hd);
 }
 
 template <int BS, int D>
@@ -666,7 +727,10 @@ static int launch_backward(hipStream_t stream, int dtype, const BackwardParams& 
     clear_stale_error();
     const uint32_t col_wgs = groups * 8u * cols.ranks, row_wgs = groups * 8u * rows.ranks;
     const dim3 grid(col_wgs + row_wgs), block(BS * 2);
-    if (dtype == SFB_F32) {
+    if (p.state != (uint32_t)D) {   // head sizes between the multiples of 32: the masked form serves both
+        if (dtype == SFB_F32) attention_backward_f32_kernel<BS, D, true, true><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+        else attention_backward_kernel<BS, D, true, true><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
+    } else if (dtype == SFB_F32) {
         if (masked) attention_backward_f32_kernel<BS, D, true><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
         else attention_backward_f32_kernel<BS, D, false><<<grid, block, 0, stream>>>(cols, rows, col_wgs);
     } else if (masked) {
@@ -679,7 +743,7 @@ static int launch_backward(hipStream_t stream, int dtype, const BackwardParams& 
     if (reduce_cols + reduce_rows)
         reduce_partials_kernel<BS, D><<<dim3(reduce_cols + reduce_rows, p.batch * p.heads), dim3(256), 0, stream>>>(
             p.dk, p.dv, p.dq, col_partials, row_partials, col_items, row_items, reduce_cols, n_col_parts, n_row_parts,
-            p.heads, p.nb * BS);
+            p.heads, p.nb * BS, p.state);
     return launch_status();
 }
 
@@ -687,7 +751,7 @@ static int launch_backward(hipStream_t stream, int dtype, const BackwardParams& 
 
 extern "C" size_t sfb_backward_workspace_bytes(uint32_t n_row_parts, uint32_t n_col_parts, uint32_t batch_dim,
                                                uint32_t head_dim, uint32_t block_size, uint32_t state_dim) {
-    const size_t record = (size_t)block_size * state_dim * sizeof(float);
+    const size_t record = (size_t)block_size * ((state_dim + 31u) / 32u * 32u) * sizeof(float);   // rows of the kernels' D floats
     return (size_t)batch_dim * head_dim * ((size_t)n_row_parts + 2 * (size_t)n_col_parts) * record;
 }
 
@@ -708,7 +772,9 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
         return SFB_ERR_NULL_POINTER;
     if (dtype != SFB_BF16 && dtype != SFB_F32) return SFB_ERR_DTYPE;
     if (block_size != 32 && block_size != 64) return SFB_ERR_BLOCK_SIZE;
-    if (state_dim != 32 && state_dim != 64 && state_dim != 96 && state_dim != 128) return SFB_ERR_HEAD_STATE;
+    // every multiple of the 16-byte vector up to 128 (32, 64, 96, 128: what the tiles divide; the others run the kernel
+    // of the next multiple of 32 with its short-row loads and stores)
+    if (state_dim == 0 || state_dim > 128 || state_dim % (dtype == SFB_BF16 ? 8u : 4u) != 0) return SFB_ERR_HEAD_STATE;
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (!batch_dim || !ctx_blks || !head_dim || !mask_heads || !lut_heads) return SFB_ERR_SHAPE;
     if (mask_heads > 1 && mask_heads != head_dim) return SFB_ERR_SHAPE;
@@ -733,25 +799,26 @@ extern "C" int sfb_fused_attention_backward(sfb_stream_t stream, const void* q, 
     BackwardParams p = {};
     p.q = q; p.k = k; p.v = v; p.d_out = d_out; p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
     p.nn_lut = nn_lut; p.tn_lut = tn_lut; p.mask = mask; p.valid_len = valid_len;
-    p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks;
+    p.batch = batch_dim; p.heads = head_dim; p.nb = ctx_blks; p.blocks = blocks; p.state = state_dim;
     p.mask_stride = mask_heads > 1 ? blocks * block_size : 0;
     p.lut_stride = lut_heads > 1 ? lut_dim : 0;
     p.scale = scale; p.scale_log2e = scale * kLog2e;
     float* row_partials = (float*)workspace;
-    float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * state_dim;
+    const uint32_t padded = (state_dim + 31u) / 32u * 32u;
+    float* col_partials = row_partials + (size_t)batch_dim * head_dim * n_row_parts * block_size * padded;
     hipStream_t s = (hipStream_t)stream;
 #define SFB_CALL(BSV, DV)                                                                                        \
     return launch_backward<BSV, DV>(s, dtype, p, row_items, n_row_items, n_row_heavy, n_row_parts, col_items, n_col_items, \
                                     n_col_heavy, n_col_parts, row_partials, col_partials)
     if (block_size == 64) {
-        if (state_dim == 64) SFB_CALL(64, 64);
-        if (state_dim == 32) SFB_CALL(64, 32);
-        if (state_dim == 96) SFB_CALL(64, 96);
+        if (padded == 64) SFB_CALL(64, 64);
+        if (padded == 32) SFB_CALL(64, 32);
+        if (padded == 96) SFB_CALL(64, 96);
         SFB_CALL(64, 128);
     }
-    if (state_dim == 64) SFB_CALL(32, 64);
-    if (state_dim == 32) SFB_CALL(32, 32);
-    if (state_dim == 96) SFB_CALL(32, 96);
+    if (padded == 64) SFB_CALL(32, 64);
+    if (padded == 32) SFB_CALL(32, 32);
+    if (padded == 96) SFB_CALL(32, 96);
     SFB_CALL(32, 128);
 #undef SFB_CALL
 }

@@ -46,9 +46,21 @@ template <> struct Elem<__bf16> {
 
 // Transposed score tile of one wave (32 queries x BS keys), operands read straight from memory.
 // Accumulator element i of key tile kt is key kt*32 + (i/4)*8 + half*4 + i%4 of query qn.
-template <int BS, int D, typename TIn>
+// RAGGED: rows of hd < D elements (hd a multiple of the 16-byte vector); the missing features count as zeros on
+// both sides and nothing beyond a row is read.
+template <bool RAGGED, typename Vec, typename T>
+__device__ __forceinline__ Vec operand_vector(const T* row, uint32_t first, uint32_t hd) {
+    if constexpr (RAGGED) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        return first < hd ? *(const Vec*)(row + first) : __builtin_bit_cast(Vec, zero);
+    } else {
+        return *(const Vec*)(row + first);
+    }
+}
+
+template <int BS, int D, typename TIn, bool RAGGED = false>
 __device__ __forceinline__ void score_tile_direct(f32x16 (&s)[BS / 32], const TIn* q_row, const TIn* k_blk,
-                                                  uint32_t row_stride, uint32_t qn, uint32_t half) {
+                                                  uint32_t row_stride, uint32_t qn, uint32_t half, uint32_t hd = D) {
     constexpr int KT = BS / 32;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -57,20 +69,20 @@ __device__ __forceinline__ void score_tile_direct(f32x16 (&s)[BS / 32], const TI
     if constexpr (sizeof(TIn) == 2) {
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks) {
-            const bf16x8 b = *(const bf16x8*)(q_row + (2 * ks + half) * 8);
+            const bf16x8 b = operand_vector<RAGGED, bf16x8>(q_row, (2 * ks + half) * 8, hd);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
-                const bf16x8 a = *(const bf16x8*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + (2 * ks + half) * 8);
+                const bf16x8 a = operand_vector<RAGGED, bf16x8>(k_blk + (size_t)(kt * 32 + qn) * row_stride, (2 * ks + half) * 8, hd);
                 s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, s[kt], 0, 0, 0);
             }
         }
     } else {
 #pragma unroll
         for (int g = 0; g < D / 8; ++g) {
-            const f32x4 b = *(const f32x4*)(q_row + 8 * g + 4 * half);
+            const f32x4 b = operand_vector<RAGGED, f32x4>(q_row, 8 * g + 4 * half, hd);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
-                const f32x4 a = *(const f32x4*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + 8 * g + 4 * half);
+                const f32x4 a = operand_vector<RAGGED, f32x4>(k_blk + (size_t)(kt * 32 + qn) * row_stride, 8 * g + 4 * half, hd);
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     s[kt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], s[kt], 0, 0, 0);
@@ -86,13 +98,14 @@ struct KTile {
     static constexpr int KT = BS / 32, STEPS = sizeof(TIn) == 2 ? D / 16 : D / 8;
     typedef typename std::conditional<sizeof(TIn) == 2, bf16x8, f32x4>::type Vec;
     Vec v[KT][STEPS];
-    __device__ __forceinline__ void load(const TIn* k_blk, uint32_t row_stride, uint32_t qn, uint32_t half) {
+    template <bool RAGGED = false>
+    __device__ __forceinline__ void load(const TIn* k_blk, uint32_t row_stride, uint32_t qn, uint32_t half, uint32_t hd = D) {
         constexpr int W = sizeof(TIn) == 2 ? 8 : 4;   // elements per vector
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int st = 0; st < STEPS; ++st)
-                v[kt][st] = *(const Vec*)(k_blk + (size_t)(kt * 32 + qn) * row_stride + (2 * st + half) * W);
+                v[kt][st] = operand_vector<RAGGED, Vec>(k_blk + (size_t)(kt * 32 + qn) * row_stride, (2 * st + half) * W, hd);
     }
 };
 template <int D, typename TIn>
@@ -100,10 +113,11 @@ struct QRow {
     static constexpr int STEPS = sizeof(TIn) == 2 ? D / 16 : D / 8;
     typedef typename std::conditional<sizeof(TIn) == 2, bf16x8, f32x4>::type Vec;
     Vec v[STEPS];
-    __device__ __forceinline__ void load(const TIn* q_row, uint32_t half) {
+    template <bool RAGGED = false>
+    __device__ __forceinline__ void load(const TIn* q_row, uint32_t half, uint32_t hd = D) {
         constexpr int W = sizeof(TIn) == 2 ? 8 : 4;
 #pragma unroll
-        for (int st = 0; st < STEPS; ++st) v[st] = *(const Vec*)(q_row + (2 * st + half) * W);
+        for (int st = 0; st < STEPS; ++st) v[st] = operand_vector<RAGGED, Vec>(q_row, (2 * st + half) * W, hd);
     }
 };
 template <int BS, int D, typename TIn>
@@ -192,6 +206,7 @@ struct SddParams {
     const void* b;
     void* c;
     uint32_t blocks, heads, ctx_a, ctx_b, lut_stride, batch, by_xcd;
+    uint32_t state;   // head size of the tensors (the kernels' D is the next multiple of 32)
 };
 
 // Blocks per work-group: a launch of one work-group per block is bound by the rate at which work-groups start,
@@ -199,22 +214,25 @@ struct SddParams {
 // current block's product and write-out.
 constexpr uint32_t kSddGroup = 2;
 
-template <int BS, int D, typename TIn, typename TOut>
+template <int BS, int D, typename TIn, typename TOut, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2) void sdd_nt_kernel(SddParams p) {
     const uint32_t b = blockIdx.y, h = blockIdx.z;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
     const uint32_t blk0 = blockIdx.x * kSddGroup;
     const uint32_t n = p.blocks - blk0 < kSddGroup ? p.blocks - blk0 : kSddGroup;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride + blk0;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_stride = p.heads * hd;
     __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TOut>::BYTES];
     TOut* out = (TOut*)p.c + ((((size_t)b * p.heads + h) * p.blocks + blk0) * BS + wave * 32) * BS;
     KTile<BS, D, TIn> k_tile[2];
     QRow<D, TIn> q_row[2];
     auto fetch = [&](uint32_t g, int buf) {
         const sfb_uint2 e = lut[g];
-        q_row[buf].load((const TIn*)p.a + token_offset(b, e.x * BS + wave * 32 + qn, h, p.ctx_a, p.heads, D), half);
-        k_tile[buf].load((const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, D), row_stride, qn, half);
+        q_row[buf].template load<RAGGED>((const TIn*)p.a + token_offset(b, e.x * BS + wave * 32 + qn, h, p.ctx_a, p.heads, hd),
+                                         half, hd);
+        k_tile[buf].template load<RAGGED>((const TIn*)p.b + token_offset(b, e.y * BS, h, p.ctx_b, p.heads, hd), row_stride, qn,
+                                          half, hd);
     };
     fetch(0, 0);
 #pragma unroll
@@ -328,18 +346,20 @@ struct SddGradParams {
     void* ds;                // dS sparse
     uint32_t blocks, heads, ctx, lut_stride;
     float scale;
+    uint32_t state;          // head size of the tensors
 };
 
-template <int BS, int D, typename TIn, typename TS>
+template <int BS, int D, typename TIn, typename TS, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2) void sdd_softmax_grad_kernel(SddGradParams p) {
     const uint32_t blk = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
     const sfb_uint2 e = p.lut[(size_t)h * p.lut_stride + blk];
     const uint32_t q = e.x * BS + wave * 32 + qn;
-    const TIn* do_row = (const TIn*)p.d_out + token_offset(b, q, h, p.ctx, p.heads, D);
-    const TIn* v_blk = (const TIn*)p.v + token_offset(b, e.y * BS, h, p.ctx, p.heads, D);
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const TIn* do_row = (const TIn*)p.d_out + token_offset(b, q, h, p.ctx, p.heads, hd);
+    const TIn* v_blk = (const TIn*)p.v + token_offset(b, e.y * BS, h, p.ctx, p.heads, hd);
     f32x16 s[BS / 32];
-    score_tile_direct<BS, D, TIn>(s, do_row, v_blk, p.heads * D, qn, half);   // dP^T: this lane's query, 16 keys per tile
+    score_tile_direct<BS, D, TIn, RAGGED>(s, do_row, v_blk, p.heads * hd, qn, half, hd);   // dP^T: this lane's query, 16 keys per tile
     const float delta = p.delta[((size_t)b * p.heads + h) * p.ctx + q];
     __shared__ __attribute__((aligned(16))) uint8_t slabs[BS / 32][RowSlab<BS, TS>::BYTES];
     const size_t rows = ((((size_t)b * p.heads + h) * p.blocks + blk) * BS + wave * 32) * BS;   // the wave's 32 rows
@@ -1128,6 +1148,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(sizeof(T) =
     }
 }
 
+// the same for rows of any length (head sizes that are not multiples of 32): lane `part` takes elements part, part + 16, ..
+template <typename TIn>
+__global__ __launch_bounds__(256) void row_dot_any_kernel(float* delta, const TIn* d_out, const float* o, uint32_t batch,
+                                                          uint32_t ctx, uint32_t heads, uint32_t hd) {
+    const uint64_t row = ((uint64_t)blockIdx.x * 256 + threadIdx.x) / 16;
+    const uint32_t part = threadIdx.x & 15;
+    const bool live = row < (uint64_t)batch * ctx * heads;   // whole groups of 16 lanes: the shuffles below stay among live lanes
+    float sum = 0.f;
+    if (live)
+        for (uint32_t i = part; i < hd; i += 16) sum += Elem<TIn>::load(d_out + row * hd + i) * o[row * hd + i];
+#pragma unroll
+    for (int d = 8; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
+    if (live && part == 0) {
+        const uint32_t hh = (uint32_t)(row % heads);
+        const uint64_t tok = row / heads;
+        const uint32_t bb = (uint32_t)(tok / ctx), qq = (uint32_t)(tok % ctx);
+        delta[((size_t)bb * heads + hh) * ctx + qq] = sum;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // dsd, transposed sparse operand (TN): C[col block] = sum over the column's blocks of A_blk^T . B_rowblk
 // (matmul.h:81-99; dV = P^T dO and dK = dS^T Q of the backward pass).  One work-group per (batch, head,
@@ -1142,9 +1182,10 @@ struct DsdParams {
     const void* b;          // dense operand: V, or dO / Q
     float* c;               // dense result
     uint32_t blocks, batch, heads, nb_b, nb_c, lut_stride, groups;
+    uint32_t state;         // head size of the dense tensors (the kernels' D is the next multiple of 32)
 };
 
-template <int BS, int D, typename TA, typename TB>
+template <int BS, int D, typename TA, typename TB, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && sizeof(TB) == 2) ? 1 : 2) void dsd_tn_kernel(DsdParams p) {
     constexpr int NO = D / 32;
     constexpr bool kFast = sizeof(TA) == 2 && sizeof(TB) == 2 && BS == 64;
@@ -1163,10 +1204,11 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t kn = lane & 31, half = lane >> 5;
     const uint32_t key_in_block = wave * 32 + kn;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_stride = p.heads * hd;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
     const uint32_t off = __builtin_amdgcn_readfirstlane(lut[col].x), count = __builtin_amdgcn_readfirstlane(lut[col].y);
-    float* c_row = p.c + token_offset(b, col * BS + key_in_block, h, p.nb_c * BS, p.heads, D);
+    float* c_row = p.c + token_offset(b, col * BS + key_in_block, h, p.nb_c * BS, p.heads, hd);
     const TA* A = (const TA*)p.a + (size_t)work.bh * p.blocks * BS * BS;
     const TB* X = (const TB*)p.b;
 
@@ -1179,13 +1221,15 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
     if constexpr (kFast) {
         // tiles 0, 1: X row blocks [q][D]; tiles 2, 3: sparse blocks [q][key]; LDS-direct loads, double-buffered
         const uint32_t row_bytes = row_stride * 2;
-        const typename TD::Sources x_src = TD::sources(lane, row_bytes);
+        // (a short last slice holds other features of its rows in place of the missing ones: they only reach output
+        // columns that are not stored)
+        const typename TD::Sources x_src = RAGGED ? TD::sources_ragged(lane, row_bytes, hd) : TD::sources(lane, row_bytes);
         const uint32_t a_even = TD::lane_source(lane, 0, BS * 2), a_odd = TD::lane_source(lane, 1, BS * 2);
         const uint32_t lds0 = TD::lds_address(smem);
         const uint32_t x_lane = TD::v_lane_base(lane);
-        const uint8_t* const x_base = (const uint8_t*)X + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
+        const uint8_t* const x_base = (const uint8_t*)X + token_offset(b, 0, h, p.nb_b * BS, p.heads, hd) * 2;
         auto fetch = [&](const sfb_uint2 e, uint32_t buf) {
-            TD::load_tile_all(lds0 + buf * TILE, x_base + (size_t)e.y * BS * row_bytes, wave, x_src, row_bytes);
+            TD::template load_tile_all<RAGGED>(lds0 + buf * TILE, x_base + (size_t)e.y * BS * row_bytes, wave, x_src, row_bytes);
             TD::load_tile(lds0 + (2 + buf) * TILE, (const uint8_t*)A + (size_t)e.x * BS * BS * 2, wave, a_even, a_odd,
                           BS * 2);
         };
@@ -1220,12 +1264,13 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
         float a_cur[BS / 2], a_next[BS / 2];
         auto fetch_block = [&](uint32_t j, float (&adst)[BS / 2]) {
             const sfb_uint2 e = lut[off + j];
-            const TB* x_blk = X + token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D);
+            const TB* x_blk = X + token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, hd);
             const TA* a_blk = A + (size_t)e.x * BS * BS;
 #pragma unroll
             for (int i = 0; i < XV; ++i) {
                 const uint32_t cid = i * BS * 2 + t, row = cid / (D / 4), cc = cid % (D / 4);
-                xr[i] = Elem<TB>::load4(x_blk + (size_t)row * row_stride + cc * 4);
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                xr[i] = (!RAGGED || cc * 4 < hd) ? Elem<TB>::load4(x_blk + (size_t)row * row_stride + cc * 4) : zero;
             }
 #pragma unroll
             for (int s2 = 0; s2 < BS / 2; ++s2) adst[s2] = Elem<TA>::load(a_blk + (size_t)(2 * s2 + half) * BS + key_in_block);
@@ -1258,20 +1303,20 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
 #pragma unroll
         for (int ig = 0; ig < 4; ++ig) {
             const f32x4 out = {acc[mt][ig * 4 + 0], acc[mt][ig * 4 + 1], acc[mt][ig * 4 + 2], acc[mt][ig * 4 + 3]};
-            *(f32x4*)(c_row + mt * 32 + ig * 8 + half * 4) = out;
+            if (!RAGGED || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(c_row + mt * 32 + ig * 8 + half * 4) = out;
         }
 }
 
 // ---------------------------------------------------------------------------------------------
 // dsd: one work-group per (batch, head, block-row), V staged through LDS, P read in operand layout
 // ---------------------------------------------------------------------------------------------
-template <int BS, int D, typename TP, typename TV>
+template <int BS, int D, typename TP, typename TV, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int KT = BS / 32, NO = D / 32;
     constexpr bool kBf16 = sizeof(TV) == 2;
     using TD = Bf16DirectTiles<BS, D>;
     using TF = F32Tiles<BS, D>;
-    constexpr bool kRing = kBf16 && sizeof(TP) == 2 && BS == 64 && D == 64;   // the streaming form below
+    constexpr bool kRing = kBf16 && sizeof(TP) == 2 && BS == 64 && D == 64 && !RAGGED;   // the streaming form below
     constexpr int LDS_BYTES = kBf16 ? (kRing ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
@@ -1285,10 +1330,11 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
-    const uint32_t row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t row_stride = p.heads * hd;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
     const uint32_t off = __builtin_amdgcn_readfirstlane(lut[r].x), count = __builtin_amdgcn_readfirstlane(lut[r].y);
-    float* o_row = p.c + token_offset(b, r * BS + q_in_block, h, p.nb_c * BS, p.heads, D);
+    float* o_row = p.c + token_offset(b, r * BS + q_in_block, h, p.nb_c * BS, p.heads, hd);
     const TP* P = (const TP*)p.a + (size_t)work.bh * p.blocks * BS * BS;
     const TV* V = (const TV*)p.b;
 
@@ -1397,9 +1443,9 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         // multiplied.  One barrier per key block.
         constexpr int PU = BS / 16;
         const uint32_t row_bytes = row_stride * 2;
-        const typename TD::Sources src = TD::sources(lane, row_bytes);
+        const typename TD::Sources src = RAGGED ? TD::sources_ragged(lane, row_bytes, hd) : TD::sources(lane, row_bytes);
         const uint32_t lds0 = TD::lds_address(smem), v_lane = TD::v_lane_base(lane);
-        const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, D) * 2;
+        const uint8_t* const v_base = (const uint8_t*)V + token_offset(b, 0, h, p.nb_b * BS, p.heads, hd) * 2;
         // slots j of product step u: keys 16u + 8(j/4) + 4*half + j%4
         f32x4 pc[2 * PU], pn[2 * PU];
         auto fetch_p = [&](f32x4 (&dst)[2 * PU], uint32_t blk) {
@@ -1411,7 +1457,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
             }
         };
         auto fetch_v = [&](uint32_t col, uint32_t buf) {
-            TD::load_tile_all(lds0 + buf * TD::TILE_BYTES, v_base + (size_t)col * BS * row_bytes, wave, src, row_bytes);
+            TD::template load_tile_all<RAGGED>(lds0 + buf * TD::TILE_BYTES, v_base + (size_t)col * BS * row_bytes, wave, src,
+                                               row_bytes);
         };
         if (count > 0) {
             const sfb_uint2 e0 = lut[off];
@@ -1447,7 +1494,8 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         f32x4 pc[KT][4], pn[KT][4];
         auto fetch_block = [&](uint32_t j, f32x4 (&pdst)[KT][4]) {
             const sfb_uint2 e = lut[off + j];
-            TF::fetch(gv, (const float*)V, token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D), row_stride, t);
+            if constexpr (RAGGED) TF::fetch_ragged(gv, (const float*)V, token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, hd), row_stride, t, hd);
+            else TF::fetch(gv, (const float*)V, token_offset(b, e.y * BS, h, p.nb_b * BS, p.heads, D), row_stride, t);
             const TP* p_row = P + ((size_t)e.x * BS + q_in_block) * BS;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
@@ -1483,7 +1531,7 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         for (int ig = 0; ig < 4; ++ig) {
             const f32x4 out = {o_acc[mt][ig * 4 + 0], o_acc[mt][ig * 4 + 1], o_acc[mt][ig * 4 + 2],
                                o_acc[mt][ig * 4 + 3]};
-            *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
+            if (!RAGGED || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
         }
 }
 
@@ -1503,6 +1551,7 @@ struct SddSoftmaxParams {
     const uint32_t* row_order;   // rank -> block-row, or nullptr
     uint32_t blocks, batch, heads, nb, lut_stride, mask_stride, groups;
     float scale_log2e;
+    uint32_t state;              // head size of the tensors
 };
 
 // bf16 operands, 64 x 64 blocks, 64 features: the work-group of a block-row (two waves, 32 queries each, the
@@ -1619,7 +1668,7 @@ __global__ __launch_bounds__(128) void sdd_softmax_stream_kernel(SddSoftmaxParam
 // rows of 64 blocks and slower on rows of 11, where the larger work-group leaves fewer of them per CU).
 constexpr int kSddSoftmaxKeyGroups = 2;
 
-template <int BS, int D, typename TIn, typename TOut>
+template <int BS, int D, typename TIn, typename TOut, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_kernel(SddSoftmaxParams p) {
     constexpr int KT = BS / 32, QW = BS / 32, KG = kSddSoftmaxKeyGroups;
     __shared__ float stats[KG][BS][2];
@@ -1631,10 +1680,11 @@ __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_ker
     const uint32_t t = threadIdx.x, lane = t & 63, wave = t >> 6, qn = lane & 31, half = lane >> 5;
     const uint32_t group = wave / QW;
     const uint32_t q_in_block = (wave % QW) * 32 + qn;
-    const uint32_t L = p.nb * BS, row_stride = p.heads * D;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t L = p.nb * BS, row_stride = p.heads * hd;
     const sfb_uint2* lut = p.nn_lut + (size_t)h * p.lut_stride;
     const uint32_t off = lut[r].x, count = lut[r].y;
-    const TIn* q_row = (const TIn*)p.a + token_offset(b, r * BS + q_in_block, h, L, p.heads, D);
+    const TIn* q_row = (const TIn*)p.a + token_offset(b, r * BS + q_in_block, h, L, p.heads, hd);
     const TIn* K = (const TIn*)p.b;
     const uint8_t* mask = p.mask ? (const uint8_t*)p.mask + (size_t)h * p.mask_stride * (BS / 8) : nullptr;
     const int valid = p.valid_len ? p.valid_len[b] : (int)L;
@@ -1642,7 +1692,7 @@ __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_ker
     TOut* Y = (TOut*)p.y + (size_t)work.bh * p.blocks * BS * BS;
 
     QRow<D, TIn> q_ops;
-    q_ops.load(q_row, half);
+    q_ops.template load<RAGGED>(q_row, half, hd);
     float m = kMaxSeed, l = 0.f;   // exact running maximum and the sum relative to it (this lane's keys)
     for (int pass = 0; pass < 2; ++pass) {
         float inv = 0.f;
@@ -1668,10 +1718,10 @@ __global__ __launch_bounds__(BS * 2 * kSddSoftmaxKeyGroups) void sdd_softmax_ker
         // the K tile of this group's next block is fetched while the current one is multiplied
         KTile<BS, D, TIn> k_cur, k_next;
         sfb_uint2 e = group < count ? lut[off + group] : sfb_uint2{0u, 0u};
-        if (group < count) k_cur.load(K + token_offset(b, e.y * BS, h, L, p.heads, D), row_stride, qn, half);
+        if (group < count) k_cur.template load<RAGGED>(K + token_offset(b, e.y * BS, h, L, p.heads, hd), row_stride, qn, half, hd);
         for (uint32_t j = group; j < count; j += KG) {
             const sfb_uint2 e_next = lut[off + (j + KG < count ? j + KG : j)];
-            k_next.load(K + token_offset(b, e_next.y * BS, h, L, p.heads, D), row_stride, qn, half);
+            k_next.template load<RAGGED>(K + token_offset(b, e_next.y * BS, h, L, p.heads, hd), row_stride, qn, half, hd);
             f32x16 s[KT];
             score_tile<BS, D, TIn>(s, k_cur, q_ops);
             const int limit = valid - (int)(e.y * BS);
@@ -1826,12 +1876,15 @@ static int check_dtype(int d) { return (d == SFB_F32 || d == SFB_BF16) ? SFB_OK 
 
 using namespace sfb;
 
-// Head sizes: 32, 64, 96 and 128 with every type combination (the reference's K64 = false paths,
-// openai_blocksparse.h:221-222, for the sizes the MFMA tiles divide).
+// Head sizes: every multiple of the 16-byte vector (4 floats, 8 bf16) up to 128, with every type combination (the
+// reference's K64 = false paths take d % 4 == 0, openai_blocksparse.h:221-222).  32, 64, 96 and 128 are what the
+// MFMA tiles divide; the sizes between run the kernel of the next multiple of 32 with its RAGGED form of loads and
+// stores.
 static int check_head_state(uint32_t state_dim, int dense_dtype) {
-    (void)dense_dtype;
-    return state_dim == 32 || state_dim == 64 || state_dim == 96 || state_dim == 128 ? SFB_OK : SFB_ERR_HEAD_STATE;
+    const uint32_t vec = dense_dtype == SFB_BF16 ? 8u : 4u;
+    return state_dim >= vec && state_dim <= 128 && state_dim % vec == 0 ? SFB_OK : SFB_ERR_HEAD_STATE;
 }
+static uint32_t padded_head_state(uint32_t state_dim) { return (state_dim + 31u) / 32u * 32u; }
 // CALL(D, TD, TS) for a head size other than 64: TD = the dense tensors' type, TS = the sparse tensor's
 #define SFB_DISPATCH_D(DV, TDN, TS, CALL)                                            \
     do {                                                                             \
@@ -1846,6 +1899,12 @@ static int check_head_state(uint32_t state_dim, int dense_dtype) {
         if ((STATE) == 32) SFB_DISPATCH_D(32, TDN, TS, CALL);              \
         else if ((STATE) == 96) SFB_DISPATCH_D(96, TDN, TS, CALL);         \
         else SFB_DISPATCH_D(128, TDN, TS, CALL);                           \
+    } while (0)
+
+#define SFB_DISPATCH_PADDED_D(PAD, TDN, TS, CALL)                          \
+    do {                                                                  \
+        if ((PAD) == 64) SFB_DISPATCH_D(64, TDN, TS, CALL);                \
+        else SFB_DISPATCH_OTHER_D(PAD, TDN, TS, CALL);                     \
     } while (0)
 
 #define SFB_DISPATCH_2(BSV, T0, T1, CALL)                                                  \
@@ -1869,10 +1928,19 @@ extern "C" int sfb_sdd_nt(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (batch_dim > 65535 || head_dim > 65535) return SFB_ERR_SHAPE;
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
     SddParams p = {lut, a, b, c, blocks, head_dim, ctx_blks_a * block_size, ctx_blks_b * block_size,
-                   lut_heads > 1 ? lut_dim : 0, batch_dim, 0};
+                   lut_heads > 1 ? lut_dim : 0, batch_dim, 0, state_dim};
     const dim3 grid((blocks + kSddGroup - 1) / kSddGroup, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim % 32 != 0) {
+#define SFB_CALL64(DV, TI, TO) sdd_nt_kernel<64, DV, TI, TO, true><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_CALL32(DV, TI, TO) sdd_nt_kernel<32, DV, TI, TO, true><<<grid, dim3(64), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, out_dtype, SFB_CALL64);
+        else SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, out_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
     if (state_dim != 64) {
 #define SFB_CALL64(DV, TI, TO) sdd_nt_kernel<64, DV, TI, TO><<<grid, dim3(128), 0, s>>>(p)
 #define SFB_CALL32(DV, TI, TO) sdd_nt_kernel<32, DV, TI, TO><<<grid, dim3(64), 0, s>>>(p)
@@ -1952,10 +2020,29 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (lut_heads > 1 && (lut_heads != head_dim || lut_dim != ctx_blks_c + blocks)) return SFB_ERR_SHAPE;
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
     DsdParams p = {lut, a, b, c, blocks, batch_dim, head_dim, ctx_blks_b, ctx_blks_c,
-                   lut_heads > 1 ? lut_dim : 0, bh_groups(batch_dim * head_dim)};
+                   lut_heads > 1 ? lut_dim : 0, bh_groups(batch_dim * head_dim), state_dim};
     const dim3 grid(p.groups * 8u * ctx_blks_c);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim % 32 != 0) {
+        const uint32_t pad = padded_head_state(state_dim);
+#define SFB_TN64(DV, TB, TA) dsd_tn_kernel<64, DV, TA, TB, true><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_TN32(DV, TB, TA) dsd_tn_kernel<32, DV, TA, TB, true><<<grid, dim3(64), 0, s>>>(p)
+#define SFB_NN64(DV, TB, TA) dsd_nn_kernel<64, DV, TA, TB, true><<<grid, dim3(128), 0, s>>>(p)
+#define SFB_NN32(DV, TB, TA) dsd_nn_kernel<32, DV, TA, TB, true><<<grid, dim3(64), 0, s>>>(p)
+        if (op == SFB_TN_OP) {
+            if (block_size == 64) SFB_DISPATCH_PADDED_D(pad, b_dtype, a_dtype, SFB_TN64);
+            else SFB_DISPATCH_PADDED_D(pad, b_dtype, a_dtype, SFB_TN32);
+        } else {
+            if (block_size == 64) SFB_DISPATCH_PADDED_D(pad, b_dtype, a_dtype, SFB_NN64);
+            else SFB_DISPATCH_PADDED_D(pad, b_dtype, a_dtype, SFB_NN32);
+        }
+#undef SFB_TN64
+#undef SFB_TN32
+#undef SFB_NN64
+#undef SFB_NN32
+        return launch_status();
+    }
     if (state_dim != 64) {
 #define SFB_TN64(DV, TB, TA) dsd_tn_kernel<64, DV, TA, TB><<<grid, dim3(128), 0, s>>>(p)
 #define SFB_TN32(DV, TB, TA) dsd_tn_kernel<32, DV, TA, TB><<<grid, dim3(64), 0, s>>>(p)
@@ -2036,10 +2123,19 @@ extern "C" int sfb_fused_sdd_softmax(sfb_stream_t stream, const sfb_uint2* nn_lu
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)y) & 15u) return SFB_ERR_ALIGNMENT;
     SddSoftmaxParams p = {nn_lut, a, b, y, mask, valid_len, row_order, blocks, batch_dim, head_dim, ctx_blks,
                           lut_heads > 1 ? lut_dim : 0, mask_heads > 1 ? blocks * block_size : 0,
-                          bh_groups(batch_dim * head_dim), scale * kLog2e};
+                          bh_groups(batch_dim * head_dim), scale * kLog2e, state_dim};
     const dim3 grid(p.groups * 8u * ctx_blks);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim % 32 != 0) {
+#define SFB_CALL64(DV, TI, TO) sdd_softmax_kernel<64, DV, TI, TO, true><<<grid, dim3(128 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+#define SFB_CALL32(DV, TI, TO) sdd_softmax_kernel<32, DV, TI, TO, true><<<grid, dim3(64 * kSddSoftmaxKeyGroups), 0, s>>>(p)
+        if (block_size == 64) SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, y_dtype, SFB_CALL64);
+        else SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, y_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
     if (state_dim != 64) {
 #define SFB_CALL64(DV, TI, TO) sdd_softmax_kernel<64, DV, TI, TO><<<grid, dim3(128 * kSddSoftmaxKeyGroups), 0, s>>>(p)
 #define SFB_CALL32(DV, TI, TO) sdd_softmax_kernel<32, DV, TI, TO><<<grid, dim3(64 * kSddSoftmaxKeyGroups), 0, s>>>(p)
@@ -2128,7 +2224,9 @@ extern "C" int sfb_row_dot(sfb_stream_t stream, float* delta, const void* d_out,
     if (state_dim == 64) SFB_CALL(64);
     else if (state_dim == 32) SFB_CALL(32);
     else if (state_dim == 96) SFB_CALL(96);
-    else SFB_CALL(128);
+    else if (state_dim == 128) SFB_CALL(128);
+    else if (dtype == SFB_F32) row_dot_any_kernel<float><<<grid, dim3(256), 0, s>>>(delta, (const float*)d_out, o, batch_dim, ctx, head_dim, state_dim);
+    else row_dot_any_kernel<__bf16><<<grid, dim3(256), 0, s>>>(delta, (const __bf16*)d_out, o, batch_dim, ctx, head_dim, state_dim);
 #undef SFB_CALL
     return launch_status();
 }
@@ -2147,10 +2245,19 @@ extern "C" int sfb_sdd_softmax_grad(sfb_stream_t stream, const sfb_uint2* nt_lut
     if (!(scale > 0.f) || !(scale < 3.0e38f)) return SFB_ERR_ARGUMENT;
     if (((uintptr_t)d_out | (uintptr_t)v | (uintptr_t)p | (uintptr_t)ds) & 15u) return SFB_ERR_ALIGNMENT;
     SddGradParams g = {nt_lut, d_out, v, p, delta, ds, blocks, head_dim, ctx_blks * block_size,
-                       lut_heads > 1 ? blocks : 0, scale};
+                       lut_heads > 1 ? blocks : 0, scale, state_dim};
     const dim3 grid(blocks, batch_dim, head_dim);
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    if (state_dim % 32 != 0) {
+#define SFB_CALL64(DV, TI, TS) sdd_softmax_grad_kernel<64, DV, TI, TS, true><<<grid, dim3(128), 0, s>>>(g)
+#define SFB_CALL32(DV, TI, TS) sdd_softmax_grad_kernel<32, DV, TI, TS, true><<<grid, dim3(64), 0, s>>>(g)
+        if (block_size == 64) SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, sparse_dtype, SFB_CALL64);
+        else SFB_DISPATCH_PADDED_D(padded_head_state(state_dim), in_dtype, sparse_dtype, SFB_CALL32);
+#undef SFB_CALL64
+#undef SFB_CALL32
+        return launch_status();
+    }
     if (state_dim != 64) {
 #define SFB_CALL64(DV, TI, TS) sdd_softmax_grad_kernel<64, DV, TI, TS><<<grid, dim3(128), 0, s>>>(g)
 #define SFB_CALL32(DV, TI, TS) sdd_softmax_grad_kernel<32, DV, TI, TS><<<grid, dim3(64), 0, s>>>(g)

@@ -165,7 +165,7 @@ def test_sdd_softmax_stream_step_issues_what_its_waits_count(kernels, elem, elem
 
 def test_dsd_stream_steps_issue_what_their_wait_counts(kernels):
     L = lib()
-    body = find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bE")
+    body = find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bLb0EE")
     assert scratch_bytes(body) == 0
     ev = events(loop_lines(body))
     spans = between_counted_waits(ev, L.ti_dsd_wait_count())
@@ -220,7 +220,7 @@ def test_registers_of_loads_in_flight_are_left_alone(kernels):
     """dsd (bf16): the P blocks are loaded into registers from inline assembly several blocks ahead and made valid by a
     counted wait, so the compiler believes them defined from the moment of issue: it must not read, copy or spill
     them before the wait that retires their loads.  Checked on the compiled loop (one straight-line block)."""
-    body = loop_lines(find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bE"))
+    body = loop_lines(find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bLb0EE"))
     code = [line.strip() for line in body if re.match(r"^\s+[a-z]", line)]
     assert not any(re.match(r"s_c?branch", c.split()[0]) for c in code[:-1]), "one straight-line block"
     loads_seen, touched = in_flight_violations(code)

@@ -153,14 +153,15 @@ def test_argument_checks_of_the_newer_entry_points():
                                             u32(4)) == 4    # a table shorter than its header
     assert sfb.lib.sfb_build_schedule_heads(None, C.byref(n), C.byref(n), C.byref(n), C.byref(n), p, 4, u32(1), u32(8),
                                             u32(0)) == 8    # max_blocks
-    # the fused backward takes head sizes 32, 64, 96, 128
+    # the fused backward takes every multiple of 8 (bf16) / 4 (fp32) up to 128
     bwd = sfb.lib.sfb_fused_attention_backward
 
     def backward(d, dtype=sfb.BF16):
         return bwd(None, p, p, p, p, p, p, p, p, p, p, dtype, p, p, None, None, None, u32(0), u32(0), u32(0), None, u32(0),
                    u32(0), u32(0), None, C.c_size_t(0), u32(64), u32(6), u32(1), u32(4), u32(4), u32(d), u32(1), u32(10),
                    u32(1), C.c_float(-1.0))
-    assert backward(48) == 3 and backward(48, sfb.F32) == 3 and backward(64, 7) == 5
+    assert backward(44) == 3 and backward(42, sfb.F32) == 3 and backward(136) == 3 and backward(64, 7) == 5
+    assert backward(48) == 8 and backward(44, sfb.F32) == 8   # head sizes taken: the call gets as far as the scale check
     assert backward(96) == 8 and backward(32) == 8 and backward(128) == 8   # size accepted; the scale is what is wrong
 
 

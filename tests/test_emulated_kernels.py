@@ -123,10 +123,11 @@ def test_peaked_rows_take_the_general_loop(E):
     assert rel_err(got.numpy(), want) <= TOL[True]
 
 
-@pytest.mark.parametrize("bs,d,bf16,order,lazy", cases([(64, 64), (32, 32), (32, 96), (64, 128)]))
+@pytest.mark.parametrize("bs,d,bf16,order,lazy", cases([(64, 64), (32, 32), (32, 96), (64, 128), (64, 40), (32, 72)]))
 def test_fused_backward(E, bs, d, bf16, order, lazy):
     """dQ, dK, dV of the fused backward (whole lines, and lines cut into chunks with partial records) against the
-    oracle's backward chain, without and with element mask and key padding."""
+    oracle's backward chain, without and with element mask and key padding.  d = 40 and 72: head sizes between the
+    multiples of 32."""
     emu_lib.configure(order=order, lazy_loads=lazy)
     nb, B, H = 4, 2, 2
     L = nb * bs
@@ -159,7 +160,7 @@ def test_fused_backward(E, bs, d, bf16, order, lazy):
 
 
 @pytest.mark.parametrize("order,lazy", [MODES[0], MODES[2], MODES[3]])
-@pytest.mark.parametrize("bs,d", [(64, 64), (32, 64), (64, 96)])
+@pytest.mark.parametrize("bs,d", [(64, 64), (32, 64), (64, 96), (64, 40), (32, 120)])
 def test_unfused_sequence_bf16(E, bs, d, order, lazy):
     """sdd -> softmax -> dsd with bf16 tensors and bf16 S / P (at block 64, head 64: the streaming kernels with their
     counted waits and the ring-buffered dsd), the two-stage fusion, and the backward sequence."""
@@ -186,10 +187,10 @@ def test_unfused_sequence_bf16(E, bs, d, order, lazy):
         assert rel_err(got.numpy(), want) <= 2e-2, (name, emu_lib.message())   # P, dP, dS each rounded to bf16 on the way
 
 
-@pytest.mark.parametrize("bs", [32, 64])
-def test_unfused_sequence_fp32(E, bs):
+@pytest.mark.parametrize("bs,d", [(32, 64), (64, 64), (64, 36), (32, 100)])
+def test_unfused_sequence_fp32(E, bs, d):
     emu_lib.configure()
-    nb, B, H, d = 4, 1, 2, 64
+    nb, B, H = 4, 1, 2
     luts = E.build_luts(layout(E, nb))
     blocks = luts["blocks"]
     Q, K, V, dO = inputs(B, nb * bs, H, d, 70, False, n=4)

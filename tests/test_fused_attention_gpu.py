@@ -271,8 +271,9 @@ def test_token_stride_of_a_merged_projection(bf16, d):
 
 def test_head_size_errors():
     luts = sfb.build_luts(PATTERNS["full"](1))
-    for dtype in (torch.bfloat16, torch.float32):   # head sizes are 32, 64, 96 and 128
-        q = torch.zeros((1, 64, 1, 80), device="cuda", dtype=dtype)
+    # head sizes: multiples of the 16-byte vector (8 bf16, 4 floats) up to 128
+    for dtype, d in ((torch.bfloat16, 132), (torch.float32, 132), (torch.bfloat16, 84), (torch.float32, 42)):
+        q = torch.zeros((1, 64, 1, d), device="cuda", dtype=dtype)
         with pytest.raises(sfb.SfbError) as e:
             sfb.fused_attention(q, q, q, sfb.to_device(luts["nn_lut"]), 64, 1, 0.125)
         assert e.value.status == 3

@@ -1,6 +1,7 @@
 """GPU parity tests of the wider coverage: peaked bf16 rows and the error budget of the two bf16 loops, scheduled
-launches with one table per head, head sizes that are not multiples of 32, the fused backward and the unfused path
-with bf16 tensors at head sizes 32 / 96 / 128.  Everything through the C ABI against the CPU oracle."""
+launches with one table per head, head sizes that are not multiples of 32 (fused forward, unfused sequence, both
+backward paths), the fused backward with fp32 tensors and the unfused path with bf16 tensors at head sizes
+32 / 96 / 128.  Everything through the C ABI against the CPU oracle."""
 import numpy as np
 import pytest
 import torch
@@ -254,3 +255,60 @@ def test_unfused_bf16_tensors_at_other_head_sizes(d, bs):
         for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
             # P, dP and dS each pass through memory as bf16: three roundings more than the fused backward carries
             assert rel_err(got.cpu().numpy(), want) <= 2 * TOL_BF16, (name, o is not None)
+
+
+@pytest.mark.parametrize("d,bf16", [(48, True), (80, True), (8, True), (120, True), (48, False), (80, False), (4, False),
+                                    (100, False)])
+@pytest.mark.parametrize("bs", [32, 64])
+def test_unfused_sequence_and_backward_paths_at_head_sizes_between_the_multiples_of_32(d, bs, bf16):
+    """The reference's K64 = false product kernels take any head size that is a multiple of 4
+    (openai_blocksparse.h:221-222).  Here: the three products, the two-stage fusion, the backward sequence and the
+    fused backward with rows of d elements (multiples of 8 for bf16, of 4 for fp32), run by the kernels of the next
+    multiple of 32 with short-row loads and stores; with element mask and key padding in the fused backward."""
+    nb, B, H = 8, 2, 3
+    L = nb * bs
+    tol = TOL_BF16 if bf16 else TOL_F32
+    scale = float(1.0 / np.sqrt(d))
+    lay = PATTERNS["bigbird"](nb).copy()
+    lay[5] = 0
+    luts = sfb.build_luts(lay)
+    blocks = luts["blocks"]
+    Q, K, V = qkv(B, L, H, d, seed=600 + bs + d, bf16=bf16)
+    dO = orc.fill_normal((B, L, H, d), 610 + d)
+    dO = orc.round_bf16(dO) if bf16 else dO
+    dQ, dK, dV, P = orc.attention_backward(Q, K, V, dO, luts, bs, scale)
+    q, k, v, do = (dev(x, bf16) for x in (Q, K, V, dO))
+    ld = {name: sfb.to_device(luts[name]) for name in ("nt_lut", "nn_lut", "tn_lut")}
+    code = sfb.BF16 if bf16 else sfb.F32
+    S = sfb.bst_sgemm_nt(ld["nt_lut"], q, k, bs, blocks, out_dtype=code)
+    assert rel_err(S.float().cpu().numpy(), orc.sdd_nt(Q, K, luts["nt_lut"], bs)) <= tol
+    p = sfb.fusion_attention2(ld["nn_lut"], q, k, bs, blocks, scale, out_dtype=code)
+    assert rel_err(p.float().cpu().numpy(), P) <= tol
+    O = sfb.bst_sgemm_xn(ld["nn_lut"], p, v, nb)
+    assert rel_err(O.cpu().numpy(), orc.attention(Q, K, V, luts["nn_lut"], bs, scale)) <= tol
+    assert (O.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
+    for o in (None, O):
+        dq, dk, dv = sfb.attention_backward(q, k, v, do, p, ld, bs, blocks, scale, o=o)
+        for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+            # with bf16 storage P, dP and dS each pass through memory as bf16
+            assert rel_err(got.cpu().numpy(), want) <= (2 * tol if bf16 else tol), (name, o is None)
+    keep = (np.random.default_rng(bs + d).random((blocks, bs, bs)) < 0.8).astype(np.uint8)
+    mask, valid = sfb.pack_mask(keep), np.array([L, L - bs - 7], np.int32)
+    for mk, vd in ((None, None), (mask, valid)):
+        m = None if mk is None else sfb.to_device(mk)
+        vl = None if vd is None else sfb.to_device(vd)
+        dQ, dK, dV, _ = orc.attention_backward(Q, K, V, dO, luts, bs, scale, mask=mk, valid_len=vd)
+        o, lse = forward(q, k, v, luts, bs, scale, mask=m, valid=vl)
+        for max_blocks in (None, 3):
+            rs = cs = None
+            if max_blocks:
+                rs, cs = sfb.build_schedule(luts["nn_lut"], nb, max_blocks), sfb.build_schedule(luts["tn_lut"], nb, max_blocks)
+                rs["items_dev"], cs["items_dev"] = sfb.to_device(rs["items"]), sfb.to_device(cs["items"])
+            dq, dk, dv = sfb.fused_attention_backward(q, k, v, o, do, lse, ld["nn_lut"], ld["tn_lut"], bs, blocks, scale,
+                                                      mask=m, valid_len=vl, row_sched=rs, col_sched=cs)
+            torch.cuda.synchronize()
+            for name, got, want in (("dq", dq, dQ), ("dk", dk, dK), ("dv", dv, dV)):
+                got = got.cpu().numpy()
+                assert np.isfinite(got).all()
+                assert rel_err(got, want) <= tol, (name, mk is not None, max_blocks)
+            assert (dq.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
