@@ -256,3 +256,47 @@ def test_the_model_of_a_step_is_not_vacuous(kernels):
     assert between_counted_waits(ev, L.ti_sdd_wait_count(2)) == []
     spans = between_counted_waits(ev, L.ti_sdd_wait_count(4))
     assert kinds(spans[0]) != {"lds": L.ti_sdd_wait_loads(2), "store": L.ti_slab_passes(2)}
+
+
+def innermost_loops(body):
+    """[label, backward branch] spans that contain no other such span."""
+    labels = {m.group(1): i for i, line in enumerate(body) if (m := re.match(r"^(\.LBB\w+):", line))}
+    spans = []
+    for i, line in enumerate(body):
+        m = re.match(r"^\s+s_c?branch\w*\s+(\.LBB\w+)", line)
+        if m and labels.get(m.group(1), len(body)) < i:
+            spans.append((labels[m.group(1)], i))
+    return [body[a:b + 1] for a, b in spans if not any((c, d) != (a, b) and a <= c and d <= b for c, d in spans)]
+
+
+def instruction_mix(lines):
+    mix = {}
+    for line in lines:
+        m = re.match(r"^\s+([a-z][a-z0-9_]+)", line)
+        if not m:
+            continue
+        op = m.group(1)
+        kind = ("mfma" if op.startswith("v_mfma") else "exp" if op.startswith("v_exp") else
+                "lds_direct" if op.startswith("global_load_lds") else "vmem" if op.startswith(("global_", "buffer_", "scratch_")) else
+                "tr_read" if op.startswith("ds_read_b64_tr") else "ds_read" if op.startswith("ds_read") else
+                "ds_write" if op.startswith("ds_write") else "barrier" if op == "s_barrier" else
+                "valu" if op.startswith("v_") else "salu" if op.startswith("s_") else "other")
+        mix[kind] = mix.get(kind, 0) + 1
+    return mix
+
+
+def test_instruction_mix_of_the_benchmarked_loop(kernels):
+    """The loop that the benchmarked launch runs (bf16, block 64, head 64, no mask: scale and offset folded into the
+    score product) handles two key blocks per trip (one per tile-buffer parity).  Per trip and wave: the 2 x 16 matrix
+    instructions of the two products, one v_exp per probability and nothing more transcendental, 16 LDS-direct loads
+    (a K and a V tile per block, four loads each), fragments read from LDS only as 128-bit and transposing reads, no
+    LDS writes, no other memory traffic than the two look-up entries, two barriers; and a bounded count of ordinary
+    vector instructions beside them (the softmax's share of the issue slots: about 5.5 per probability pair)."""
+    body = find(kernels, "fused_attention_bf16_kernelILi64ELi64ELb0ELb0E")
+    assert scratch_bytes(body) == 0
+    lean = [loop for loop in innermost_loops(body) if instruction_mix(loop).get("mfma", 0) == 32]
+    assert lean, "no loop with the matrix instructions of two key blocks"
+    mix = instruction_mix(lean[0])
+    assert mix["exp"] == 64 and mix["lds_direct"] == 16 and mix["ds_read"] == 16 and mix["tr_read"] == 32
+    assert mix.get("ds_write", 0) == 0 and mix["barrier"] == 2 and mix.get("vmem", 0) <= 2
+    assert mix["valu"] <= 190, mix
