@@ -247,12 +247,11 @@ uint32_t sfb_resident_work_groups(void);
 
 /* state_dim (the head size d).  Every attention entry point takes every multiple of 4 (fp32 tensors) or 8 (bf16
  * tensors: rows are whole 16-byte vectors) up to 128 -- the reference's `d % 4 == 0` of its K64 = false paths,
- * openai_blocksparse.h:221-222: the fused forward (plain and scheduled launches), the products of the unfused path
+ * openai_blocksparse.h:221-222: the fused forward (plain, scheduled and streamed launches), the products of the unfused path
  * (sfb_sdd_nt, sfb_dsd_xn, sfb_fused_sdd_softmax, sfb_sdd_softmax_grad, sfb_row_dot) and the fused backward.  32, 64,
  * 96 and 128 are what the kernels' tiles divide; a size between them runs the kernel of the next multiple of 32 with
- * the missing features read as zeros and only d output columns stored.  Streamed launches
- * (sfb_fused_attention_streamed, sfb_encoder_layer_forward_streamed) and sfb_fused_sdd_softmax_split take the
- * multiples of 32 / 64 only.  Anything else returns SFB_ERR_HEAD_STATE. */
+ * the missing features read as zeros and only d output columns stored.  sfb_fused_sdd_softmax_split (the per-block
+ * comparison kernel) takes 64 only.  Anything else returns SFB_ERR_HEAD_STATE. */
 
 /* Fully fused attention: O = softmax_rows(scale * Q K^T restricted to layout & mask & key<valid_len) V,
  * one work-group per (batch, head, block-row), no S/P in memory.  Replaces the sequence

@@ -965,14 +965,15 @@ __device__ __forceinline__ RowWork stream_row_work(const FusedParams& p, const_w
 // End of a streamed item.  A whole row is normalised and stored straight from the accumulators; a chunk of a cut
 // row leaves its partial record and returns the record's index + 1: its flag is to be set once these stores have
 // completed (the caller does that after its next wait for memory).  Returns 0 otherwise.
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __device__ __forceinline__ uint32_t stream_end_item(const FusedParams& p, const StreamItem& it, f32x16 (&o)[D / 32],
                                                     float m_used, float m_true, float l, float c, uint32_t t) {
     constexpr int NO = D / 32, PART = BS * D + 4 * BS;
     const uint32_t lane = t & 63, qn = lane & 31, half = lane >> 5, q_in_block = (t >> 6) * 32 + qn;
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
     const float total = l + __shfl_xor(l, 32);
     if (it.tag == 0) {
-        float* o_row = output_row(p, ((size_t)it.q_off + (size_t)q_in_block * p.heads) * D);
+        float* o_row = output_row(p, ((size_t)it.q_off + (size_t)q_in_block * p.heads) * hd);
         const float f = exp2_fast((m_true - m_used) * c);
         const float inv = 1.0f / (total + 1e-6f * f);
         if (p.lse != nullptr && half == 0)
@@ -981,6 +982,7 @@ __device__ __forceinline__ uint32_t stream_end_item(const FusedParams& p, const 
             const f32x4 out = {o[mt][ig * 4 + 0] * inv, o[mt][ig * 4 + 1] * inv, o[mt][ig * 4 + 2] * inv,
                                o[mt][ig * 4 + 3] * inv};
             const uint32_t col = mt * 32 + ig * 8 + half * 4;
+            if (RAGGED && col >= hd) return;
             if (p.o_bf16) {
                 const u32x2 packed = {pack_bf16(out.x, out.y), pack_bf16(out.z, out.w)};
                 *(u32x2*)((uint8_t*)o_row + col * 2) = packed;
@@ -1009,20 +1011,22 @@ __device__ __forceinline__ void stream_set_flag(const FusedParams& p, uint32_t p
 // Merge tasks of a work-group, done after its stream: wait (bounded) for the flags of the row's partial records, add
 // the records, write the row, clear the flags for the next launch.  lds: at least BS * (D * 4 + 16) bytes that nobody
 // uses any more.
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __device__ __forceinline__ void stream_merges(const FusedParams& p, const_words merges, uint32_t n_merges, uint8_t* lds) {
     constexpr int PART = BS * D + 4 * BS;
     constexpr uint32_t kMaxPolls = 1u << 20;   // of about a microsecond each
     const uint32_t t = threadIdx.x, lane = t & 63, q_in_block = (t >> 6) * 32 + (lane & 31);
-    const uint32_t o_row_bytes = p.heads * D * (p.o_bf16 ? 2u : 4u);
+    const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
+    const uint32_t o_row_bytes = p.heads * hd * (p.o_bf16 ? 2u : 4u);
     uint8_t* const slab = lds + (t >> 6) * (32u * (D * 4 + 16));
     for (uint32_t i = 0; i < n_merges; ++i) {
         const const_words w = merges + (size_t)i * (sizeof(sfb_stream_merge) / 4);
         const uint32_t q_off = w[0], batch = w[1], head = w[2], row = w[3], part = w[4], nparts = w[5];
-        float* o_row = output_row(p, ((size_t)q_off + (size_t)q_in_block * p.heads) * D);
+        float* o_row = output_row(p, ((size_t)q_off + (size_t)q_in_block * p.heads) * hd);
         float* lse_row = p.lse ? p.lse + ((size_t)(batch * p.heads + head) * p.nb + row) * BS + q_in_block : nullptr;
         if (nparts == 0) {
-            store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
+            if constexpr (RAGGED) store_zero_row_ragged(o_row, p.o_bf16, lane >> 5, hd);
+            else store_zero_row<D>(o_row, p.o_bf16, lane >> 5);
             if (lse_row && (lane >> 5) == 0) *lse_row = 0.f;
             continue;
         }
@@ -1039,8 +1043,8 @@ __device__ __forceinline__ void stream_merges(const FusedParams& p, const_words 
             if (t == 0) __hip_atomic_store(p.st_status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             continue;
         }
-        merge_partials<BS, D>(p.partials + (size_t)part * PART, nparts, o_row, o_row_bytes, p.o_bf16, lse_row,
-                              p.scale_log2e, q_in_block, lane, slab);
+        merge_partials<BS, D, RAGGED>(p.partials + (size_t)part * PART, nparts, o_row, o_row_bytes, p.o_bf16, lse_row,
+                                      p.scale_log2e, q_in_block, lane, slab, hd);
         for (uint32_t f = t; f < nparts; f += BS * 2)
             __hip_atomic_store(p.st_flags + part + f, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();   // the slabs are used again by the next merge
@@ -1332,7 +1336,7 @@ __global__ __launch_bounds__(BS * 2, 2) void fused_attention_stream_bf16_kernel(
 // Other element types and head sizes: the work-group does the items of its stream one after the other.
 // bf16 tensors with a head size other than 64: the stream's items one after the other (the chained form above is
 // built around one score product step per chunk, which is what 64 features give).
-template <int BS, int D, bool MASKED>
+template <int BS, int D, bool MASKED, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream_items_bf16_kernel(FusedParams p) {
     using T = Bf16DirectTiles<BS, D>;
     constexpr int TILE = T::TILE_BYTES;
@@ -1349,21 +1353,21 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream
         const sfb_uint2 window = lut_window(p, w, 0, lane);
         uint32_t made = 0;
         auto finish = [&](f32x16 (&o)[D / 32], const RowState& rs) {
-            made = stream_end_item<BS, D>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
+            made = stream_end_item<BS, D, RAGGED>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
         };
         bool done = false;
-        if constexpr (!MASKED) done = attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window, finish);
-        if (!done) attend_item_bf16<BS, D, MASKED, false>(p, w, smem, &retry_flag, window, finish);
+        if constexpr (!MASKED && !RAGGED) done = attend_item_bf16<BS, D, false, true>(p, w, smem, &retry_flag, window, finish);
+        if (!done) attend_item_bf16<BS, D, MASKED, false, RAGGED>(p, w, smem, &retry_flag, window, finish);
         if (made != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();   // the record is complete, and the tiles' memory is free for the next item
         if (made != 0 && t == 0) stream_set_flag(p, made);
     }
     if (n_merges != 0)
-        stream_merges<BS, D>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4), n_merges,
-                             smem);
+        stream_merges<BS, D, RAGGED>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4),
+                                     n_merges, smem);
 }
 
-template <int BS, int D>
+template <int BS, int D, bool RAGGED = false>
 __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream_f32_kernel(FusedParams p) {
     using T = F32Tiles<BS, D>;
     __shared__ __attribute__((aligned(16))) float k_lds[T::K_FLOATS];
@@ -1376,16 +1380,16 @@ __global__ __launch_bounds__(BS * 2, D > 64 ? 1 : 2) void fused_attention_stream
     for (uint32_t i = 0; i < n_items; ++i) {
         const StreamItem it = stream_item(items, i, n_items);
         uint32_t made = 0;
-        attend_item_f32<BS, D>(p, stream_row_work(p, items, i), k_lds, v_lds, [&](f32x16 (&o)[D / 32], const RowState& rs) {
-            made = stream_end_item<BS, D>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
+        attend_item_f32<BS, D, RAGGED>(p, stream_row_work(p, items, i), k_lds, v_lds, [&](f32x16 (&o)[D / 32], const RowState& rs) {
+            made = stream_end_item<BS, D, RAGGED>(p, it, o, rs.m_used, rs.m_true, rs.l, p.scale_log2e, t);
         });
         if (made != 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (made != 0 && t == 0) stream_set_flag(p, made);
     }
     if (n_merges != 0)
-        stream_merges<BS, D>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4), n_merges,
-                             (uint8_t*)k_lds);
+        stream_merges<BS, D, RAGGED>(p, (const_words)(uintptr_t)p.st_merges + (size_t)merge_begin * (sizeof(sfb_stream_merge) / 4),
+                                     n_merges, (uint8_t*)k_lds);
 }
 
 // Fill kernel (a captured graph must not hold a memset node): words[0 .. n) = 0.
@@ -1432,9 +1436,12 @@ static int launch_fused(hipStream_t stream, FusedParams& p, int in_dtype, uint32
 // Work-groups per compute unit the device keeps resident of the kernel a streamed launch of this kind runs (the
 // same choice as launch_fused makes); 0 if the runtime cannot say.
 template <int BS, int D>
-static int stream_kernel_occupancy(int in_dtype, bool masked) {
+static int stream_kernel_occupancy(int in_dtype, bool masked, bool ragged = false) {
     const void* kernel;
-    if (in_dtype == SFB_BF16) {
+    if (ragged) {
+        kernel = in_dtype == SFB_BF16 ? (const void*)fused_attention_stream_items_bf16_kernel<BS, D, true, true>
+                                      : (const void*)fused_attention_stream_f32_kernel<BS, D, true>;
+    } else if (in_dtype == SFB_BF16) {
         if constexpr (D == 64) {
             kernel = masked ? (const void*)fused_attention_stream_bf16_kernel<BS, D, true>
                             : (const void*)fused_attention_stream_bf16_kernel<BS, D, false>;
@@ -1459,18 +1466,29 @@ static int stream_kernel_occupancy_any(int in_dtype, bool masked, uint32_t state
         case 32: return stream_kernel_occupancy<BS, 32>(in_dtype, masked);
         case 96: return stream_kernel_occupancy<BS, 96>(in_dtype, masked);
         case 128: return stream_kernel_occupancy<BS, 128>(in_dtype, masked);
+        default: break;
+    }
+    switch ((state_dim + 31) / 32) {   // head sizes between: the kernel of the next multiple of 32
+        case 1: return stream_kernel_occupancy<BS, 32>(in_dtype, true, true);
+        case 2: return stream_kernel_occupancy<BS, 64>(in_dtype, true, true);
+        case 3: return stream_kernel_occupancy<BS, 96>(in_dtype, true, true);
+        case 4: return stream_kernel_occupancy<BS, 128>(in_dtype, true, true);
         default: return 0;
     }
 }
 
 // Head sizes that are not a multiple of 32 (the reference's kernels take any multiple of 4,
 // openai_blocksparse.h:221-222): the kernel of the next multiple of 32 with zero-padded queries, the general loop
-// only.  Plain and scheduled launches; streamed ones do not take them.
+// only.  Streamed launches walk their items one after the other (the masked form serves both kinds of launch).
 template <int BS, int D>
 static int launch_fused_ragged(hipStream_t stream, FusedParams& p, int in_dtype, uint32_t ranks) {
-    if (p.st_slots != nullptr) return SFB_ERR_HEAD_STATE;
     p.ranks = ranks;
     clear_stale_error();
+    if (p.st_slots != nullptr) {   // ranks = resident work-groups
+        if (in_dtype == SFB_BF16) fused_attention_stream_items_bf16_kernel<BS, D, true, true><<<dim3(ranks), dim3(BS * 2), 0, stream>>>(p);
+        else fused_attention_stream_f32_kernel<BS, D, true><<<dim3(ranks), dim3(BS * 2), 0, stream>>>(p);
+        return launch_status();
+    }
     const dim3 g(p.groups * 8u * ranks), b(BS * 2);
     if (in_dtype == SFB_BF16) fused_attention_bf16_kernel<BS, D, true, true><<<g, b, 0, stream>>>(p);
     else fused_attention_f32_kernel<BS, D, true><<<g, b, 0, stream>>>(p);
@@ -1703,7 +1721,8 @@ extern "C" int sfb_fused_attention_scheduled_heads(sfb_stream_t stream, const vo
 extern "C" size_t sfb_stream_workspace_bytes(const sfb_stream_plan* plan, uint32_t state_dim) {
     if (!plan) return 0;
     const size_t flags = ((size_t)plan->n_parts * sizeof(uint32_t) + 255) / 256 * 256;
-    const size_t part = ((size_t)plan->block_size * state_dim + 4 * (size_t)plan->block_size) * sizeof(float);
+    const size_t padded = (state_dim + 31u) / 32u * 32u;   // records hold rows of the kernels' D floats
+    const size_t part = ((size_t)plan->block_size * padded + 4 * (size_t)plan->block_size) * sizeof(float);
     return flags + (size_t)plan->n_parts * part + 256;   // the last 256 bytes hold the status word (at their end)
 }
 
@@ -1719,7 +1738,7 @@ extern "C" uint32_t sfb_resident_work_groups_for(int in_dtype, uint32_t block_si
     const int per_cu = block_size == 64 ? stream_kernel_occupancy_any<64>(in_dtype, masked != 0, state_dim)
                                         : stream_kernel_occupancy_any<32>(in_dtype, masked != 0, state_dim);
     // (a runtime that cannot answer: what the kernels' registers and LDS allow by design)
-    return (uint32_t)(per_cu > 0 ? per_cu : (state_dim > 64 ? 2 : 4)) * (uint32_t)cus;
+    return (uint32_t)(per_cu > 0 ? per_cu : (state_dim > 64 || state_dim % 32 != 0 ? 2 : 4)) * (uint32_t)cus;
 }
 
 // bf16 tensors, blocks of 64, head size 64, no mask: the benched case

@@ -111,8 +111,8 @@ def test_scheduled_launch_with_per_head_tables(bf16, bs):
 def test_head_sizes_that_are_not_multiples_of_32(d, bs, bf16):
     """The reference's K64 = false kernels take any head size that is a multiple of 4 (openai_blocksparse.h:221-222).
     Here: multiples of 4 (fp32) or 8 (bf16 -- rows of whole 16-byte vectors) up to 128, through the kernel of the
-    next multiple of 32 with zero-padded queries; plain and scheduled launches, with and without mask and padding,
-    a row without blocks, split rows merged from partial records, bf16 output, log-sum-exp output."""
+    next multiple of 32 with zero-padded queries; plain, scheduled and streamed launches, with and without mask and
+    padding, a row without blocks, split rows merged from partial records, bf16 output, log-sum-exp output."""
     nb, B, H = 8, 2, 3
     L = nb * bs
     tol = TOL_BF16 if bf16 else TOL_F32
@@ -142,12 +142,17 @@ def test_head_sizes_that_are_not_multiples_of_32(d, bs, bf16):
     torch.cuda.synchronize()
     check(o32.cpu().numpy(), plain, tol)
     assert torch.isfinite(lse).all() and float(lse[:, :, 5 * bs:6 * bs].abs().max()) == 0.0
-    # streamed launches do not take these sizes: a checked error, not a wrong result
-    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=16)
+    # streamed launches: rows cut into chunks, merged from partial records
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=64)
+    assert stream["plan"].n_parts > 0
     sws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
-    with pytest.raises(sfb.SfbError) as info:
-        sfb.fused_attention_streamed(q, k, v, nn, sfb.to_device(stream["blob"]), stream, sws, bs, luts["blocks"], scale)
-    assert info.value.status == 3
+    blob = sfb.to_device(stream["blob"])
+    for m, vl, ref in ((None, None, plain), (sfb.to_device(mask), sfb.to_device(valid), want)):
+        for _ in range(2):   # the second launch finds the flags as the first one left them
+            out = sfb.fused_attention_streamed(q, k, v, nn, blob, stream, sws, bs, luts["blocks"], scale, mask=m, valid_len=vl)
+            torch.cuda.synchronize()
+            assert sfb.stream_status(stream, d, sws) == 0
+            check(out.cpu().numpy(), ref, tol)
 
 
 @pytest.mark.parametrize("d", [32, 96, 128])
