@@ -14,6 +14,9 @@ def pytest_addoption(parser):
                      help="run the tests marked gpu without a GPU, on the host build of the kernel sources "
                           "(tests/emu_lib.py); --emulate-order and --emulate-eager choose the lane order and when "
                           "LDS-direct loads land")
+    parser.addoption("--ubsan", action="store_true",
+                     help="also run test_emulated_kernels.py's sanitizer pass (builds the host model with the undefined-"
+                          "behaviour sanitizer: minutes)")
     parser.addoption("--emulate-order", type=int, default=0)
     parser.addoption("--emulate-eager", action="store_true")
 
@@ -48,3 +51,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """Host-model runs leave what the model executed (per kind of wave-wide operation: all, and those that ran with
+    part of their wave because the wave had diverged) beside the build, one file per process."""
+    if not session.config.getoption("--emulate"):
+        return
+    import json
+    import emu_lib
+    path = os.path.join(emu_lib.BUILD, "counts_%d.json" % os.getpid())
+    with open(path, "w") as f:
+        json.dump(emu_lib.counts(), f)

@@ -309,6 +309,38 @@ def build(verbose=False):
     return LIB
 
 
+def build_sanitized(verbose=False):
+    """Every unit of the host build compiled with the undefined-behaviour sanitizer (misaligned vector accesses,
+    out-of-range shifts and indices of fixed arrays, signed overflow): tests/_build/emu/libsfbert_emu_ubsan.so.
+    Findings are printed to stderr and counted by the runtime's own handler; see test_emulated_kernels.py."""
+    build()
+    lib = os.path.join(BUILD, "libsfbert_emu_ubsan.so")
+    stamp = os.path.join(BUILD, "digest_ubsan")
+    digest = _digest()
+    if os.path.exists(lib) and os.path.exists(stamp) and open(stamp).read() == digest:
+        return lib
+    gen = os.path.join(BUILD, "sf-bert_amd", "csrc")
+    units = [os.path.join(gen, name.replace(".hip", "_emu.cpp")) for name in KERNEL_SOURCES]
+    units += [os.path.join(gen, "selftest_kernels_emu.cpp")] + [os.path.join(CSRC, f) for f in HOST_SOURCES]
+    units += [os.path.join(EMU, "emu_runtime.cpp")]
+    flags = ["-O1", "-g1", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma", "-mf16c",
+             "-fsanitize=undefined", "-fno-sanitize=vptr,function", "-fno-sanitize-recover=undefined",
+             "-fsanitize-trap=undefined"]
+
+    def compile_unit(src):
+        obj = os.path.join(BUILD, os.path.basename(src) + ".ubsan.o")
+        subprocess.check_call([CLANG, "-x", "c++"] + flags + ["-c", src, "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=6) as pool:
+        objects = list(pool.map(compile_unit, units))
+    subprocess.check_call([CLANG, "-shared", "-o", lib + ".new"] + objects + ["-lm"])
+    os.replace(lib + ".new", lib)
+    with open(stamp, "w") as f:
+        f.write(digest)
+    return lib
+
+
 def build_variant(tag, defines, source="fused_attention.hip"):
     """The host build with one kernel source compiled under other preprocessor definitions (the opt-in kernel
     variants of sf-bert_amd/build.py): tests/_build/emu/libsfbert_emu_<tag>.so."""
@@ -343,7 +375,7 @@ def load(tag="", defines=()):
     a variant of it, see build_variant)."""
     if tag in _modules:
         return _modules[tag]
-    lib_path = build_variant(tag, defines) if tag else build()
+    lib_path = build_sanitized() if tag == "ubsan" else build_variant(tag, defines) if tag else build()
     saved = os.environ.get("SFBERT_HIP_LIB")
     os.environ["SFBERT_HIP_LIB"] = lib_path
     try:

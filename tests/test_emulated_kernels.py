@@ -256,3 +256,20 @@ def test_tile_load_variants_of_the_bf16_loop(E, tag, define):
                 outs.append((plain, cut))
             assert rel_err(outs[1][0], want) <= TOL[True] and rel_err(outs[1][1], want) <= TOL[True]
             assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
+def test_kernels_under_the_undefined_behaviour_sanitizer(E, request):
+    """The host build compiled with -fsanitize=undefined in trapping mode (misaligned vector accesses, indices past
+    fixed arrays, out-of-range shifts, signed overflow): one pass over the attention entry points.  A finding ends
+    the process with an illegal-instruction trap, which is the failure.  Takes minutes to build: only with --ubsan."""
+    if not request.config.getoption("--ubsan"):
+        pytest.skip("needs --ubsan (a build of several minutes)")
+    S = emu_lib.load("ubsan")
+    for case in cases([(64, 64), (32, 96), (64, 40)]):
+        if case[3] == 0:
+            test_fused_forward_plain_scheduled_streamed(S, *case)
+            test_fused_backward(S, *case)
+    for bs, d in ((64, 64), (32, 120)):
+        test_unfused_sequence_bf16(S, bs, d, 0, True)
+    test_unfused_sequence_fp32(S, 64, 36)
+    test_scheduled_launch_with_one_table_per_head(S)
