@@ -341,6 +341,19 @@ def build_sanitized(verbose=False):
     return lib
 
 
+def build_host_program(name):
+    """A C++ host program of sf-bert_amd/host/ (they drive the library through the reference-named launchers) built
+    against the stand-in runtime and the host build: tests/_build/emu/<name>."""
+    lib = build()
+    src = os.path.join(ROOT, "sf-bert_amd", "host", name + ".cpp")
+    exe = os.path.join(BUILD, name)
+    if os.path.exists(exe) and os.path.getmtime(exe) > max(os.path.getmtime(src), os.path.getmtime(lib)):
+        return exe
+    subprocess.check_call([CLANG, "-O1", "-std=c++17", "-w", "-I" + EMU, "-o", exe, "-x", "c++", src, "-x", "none", lib,
+                           "-Wl,-rpath," + BUILD, "-lm"])
+    return exe
+
+
 def build_variant(tag, defines, source="fused_attention.hip"):
     """The host build with one kernel source compiled under other preprocessor definitions (the opt-in kernel
     variants of sf-bert_amd/build.py): tests/_build/emu/libsfbert_emu_<tag>.so."""

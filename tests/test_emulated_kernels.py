@@ -273,3 +273,17 @@ def test_kernels_under_the_undefined_behaviour_sanitizer(E, request):
         test_unfused_sequence_bf16(S, bs, d, 0, True)
     test_unfused_sequence_fp32(S, 64, 36)
     test_scheduled_launch_with_one_table_per_head(S)
+
+
+@pytest.mark.parametrize("name,args", [("attention_host_test", []),
+                                       ("transformer_inference", ["2", "2", "256", "2", "64", "bf16"]),
+                                       ("transformer_inference", ["1", "1", "256", "2", "64", "f32"])])
+def test_cpp_host_programs_on_the_host_build(name, args):
+    """The C++ mains of sf-bert_amd/host/ -- one in the shape of the reference's *_fusion_test.cu that goes through the
+    reference-named launchers (bst_sgemm_nt, BlocksparseMaskedSoftmax, bst_sgemm_xn, fusion_attention2,
+    fusion_attention) of the replacement headers, one in the shape of transformer_inference_part.cpp on
+    sfb_model_forward -- compiled against the stand-in runtime and linked with the host build of the kernels."""
+    import subprocess
+    exe = emu_lib.build_host_program(name)
+    out = subprocess.run([exe] + args, capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0 and "PASSED" in out.stdout, (out.stdout[-600:], out.stderr[-600:])
