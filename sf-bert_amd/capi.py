@@ -417,7 +417,7 @@ def fused_attention_forward_lse(q, k, v, nn_lut, items, sched, workspace, block_
 def fused_attention_backward(q, k, v, o, d_out, lse, nn_lut, tn_lut, block_size, blocks, scale, mask=None,
                              valid_len=None, mask_heads=1, row_sched=None, col_sched=None, workspace=None,
                              lut_heads=1):
-    """(dq, dk, dv) fp32 from bf16 q, k, v, d_out, the forward output o and lse, in two kernels
+    """(dq, dk, dv) fp32 from bf16 or fp32 q, k, v, d_out (head sizes: multiples of 8 / 4 up to 128), the forward output o and lse, in two kernels
     (sfb_fused_attention_backward); nothing sparse goes through memory.  row_sched / col_sched: build_schedule()
     over the NN / TN look-up table with its "items" already on the device under "items_dev" (None: one
     work-group per block-row / block-column).  lut_heads = H: nn_lut / tn_lut hold one table per head (then without

@@ -317,3 +317,23 @@ def test_unfused_sequence_and_backward_paths_at_head_sizes_between_the_multiples
                 assert np.isfinite(got).all()
                 assert rel_err(got, want) <= tol, (name, mk is not None, max_blocks)
             assert (dq.cpu().numpy()[:, 5 * bs:6 * bs] == 0).all()
+
+
+@pytest.mark.parametrize("bf16,d,heads,streamed,pre_ln", [(True, 40, 4, False, False), (False, 36, 4, False, True),
+                                                          (True, 72, 2, True, False), (False, 20, 4, True, False)])
+def test_encoder_layer_at_head_sizes_between_the_multiples_of_32(bf16, d, heads, streamed, pre_ln):
+    """One encoder layer (both wirings, attention as a scheduled and as a streamed launch) with such head sizes."""
+    from test_layer_gpu import T, layer_weights
+    B, L, ffn, bs = 2, 512, 256, 64
+    n, nb = heads * d, L // bs
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    w = layer_weights(n, ffn, 100)
+    x = orc.fill_normal((B * L, n), 300)
+    oracle = orc.encoder_layer_pre_ln if pre_ln else orc.encoder_layer
+    want = oracle(x, w, luts["nn_lut"], B, L, heads, d, ffn, bs, luts["blocks"], operands_bf16=bf16, nthreads=THREADS)
+    layer = sfb.EncoderLayer({k: T(v) for k, v in w.items()}, luts, bs, heads, d, ffn,
+                             dtype=sfb.BF16 if bf16 else sfb.F32, max_blocks=2, pre_ln=pre_ln, streamed=streamed)
+    for _ in range(2):
+        got = layer.forward(T(x), B, L).cpu().numpy()
+        torch.cuda.synchronize()
+        assert rel_err(got, want) <= (TOL_BF16 if bf16 else TOL_F32)
