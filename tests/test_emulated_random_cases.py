@@ -93,7 +93,7 @@ def test_one_table_and_mask_per_head(E, seed):
     rng = np.random.default_rng(seed)
     bs, bf16 = int(rng.choice([32, 64])), bool(rng.integers(2))
     d = int(rng.choice([32, 64, 96, 128] + ([40, 72] if bf16 else [36, 100])))
-    nb, B, H = int(rng.integers(2, 17)), int(rng.integers(1, 3)), int(rng.integers(2, 4))
+    nb, B, H = int(rng.integers(2, 11)), int(rng.integers(1, 3)), int(rng.integers(2, 4))
     base = (rng.random((nb, nb)) < rng.choice([0.1, 0.3, 0.6])).astype(np.uint32)
     if base.sum() == 0:
         base[0, 0] = 1
