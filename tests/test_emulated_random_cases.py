@@ -154,3 +154,41 @@ def test_one_table_and_mask_per_head(E, seed):
     p2 = E.fusion_attention2(nnd, q, k, bs, blocks, scale, mask=md, valid_len=vd, out_dtype=code, lut_heads=H, mask_heads=mask_heads)
     check("two-stage fusion", p2.float().numpy(), P_want, tol, case)
     check("dsd", E.bst_sgemm_xn(nnd, p2, v, nb, lut_heads=H).numpy(), want, 2 * tol if bf16 else tol, case)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_encoder_layer(E, seed):
+    """One encoder layer with random widths (hidden = heads x head size, FFN width down to 4), wiring (post- / pre-LN),
+    attention launch (scheduled with a random chunk length, streamed), Q/K/V as one product or three, over a random
+    layout that may leave block-rows empty."""
+    rng = np.random.default_rng(seed)
+    bf16, bs = bool(rng.integers(2)), int(rng.choice([32, 64]))
+    d = int(rng.choice([32, 64, 96] + ([40, 8] if bf16 else [36, 20])))
+    H, B, nb = int(rng.integers(1, 5)), int(rng.integers(1, 3)), int(rng.integers(1, 6))
+    ffn = int(rng.choice([4, 64, 100, 256, 516]))
+    L, n = nb * bs, H * d
+    lay = (rng.random((nb, nb)) < rng.choice([0.3, 0.7, 1.0])).astype(np.uint32)
+    if lay.sum() == 0:
+        lay[0, 0] = 1
+    luts = E.build_luts(lay)
+    pre_ln, streamed, merge = bool(rng.integers(2)), bool(rng.integers(2)), bool(rng.integers(2))
+    max_blocks = int(rng.choice([0, 1, 3, 16]))
+    emu_lib.configure(order=int(rng.choice([0, 1, int(rng.integers(2, 60))])), lazy_loads=bool(rng.integers(2)))
+    case = dict(seed=seed, bf16=bf16, bs=bs, d=d, H=H, B=B, nb=nb, ffn=ffn, pre_ln=pre_ln, streamed=streamed, merge=merge,
+                max_blocks=max_blocks)
+    shapes = [("wq", (n, n)), ("wk", (n, n)), ("wv", (n, n)), ("wo", (n, n)), ("w1", (n, ffn)), ("w2", (ffn, n)),
+              ("bq", (n,)), ("bk", (n,)), ("bv", (n,)), ("bo", (n,)), ("b1", (ffn,)), ("b2", (n,)),
+              ("ln1_g", (n,)), ("ln1_b", (n,)), ("ln2_g", (n,)), ("ln2_b", (n,))]
+    w = {name: orc.fill_normal(shape, 100 + 20 * seed + i, 0.1 if name[0] == "b" else 0.02) for i, (name, shape) in enumerate(shapes)}
+    w["ln1_g"], w["ln2_g"] = w["ln1_g"] + 1, w["ln2_g"] + 1
+    x = orc.fill_normal((B * L, n), 300 + seed)
+    oracle = orc.encoder_layer_pre_ln if pre_ln else orc.encoder_layer
+    want = oracle(x, w, luts["nn_lut"], B, L, H, d, ffn, bs, luts["blocks"], operands_bf16=bf16, nthreads=4)
+    kw = dict(dtype=E.BF16 if bf16 else E.F32, pre_ln=pre_ln, max_blocks=max_blocks)
+    if streamed:
+        kw["streamed"] = True
+    else:
+        kw["merge_qkv"] = merge
+    layer = E.EncoderLayer({name: dev(a) for name, a in w.items()}, luts, bs, H, d, ffn, **kw)
+    for _ in range(2):
+        check("encoder layer", layer.forward(dev(x), B, L).numpy(), want, 1e-2 if bf16 else 1e-4, case)
