@@ -17,6 +17,8 @@ def pytest_addoption(parser):
     parser.addoption("--ubsan", action="store_true",
                      help="also run test_emulated_kernels.py's sanitizer pass (builds the host model with the undefined-"
                           "behaviour sanitizer: minutes)")
+    parser.addoption("--mutants", action="store_true",
+                     help="run test_host_model_mutants.py (a build of the host model per seeded mistake: minutes)")
     parser.addoption("--emulate-order", type=int, default=0)
     parser.addoption("--emulate-eager", action="store_true")
 

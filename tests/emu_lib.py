@@ -354,6 +354,59 @@ def build_host_program(name):
     return exe
 
 
+def build_mutant(tag, source, old, new, count=1):
+    """The host build with one deliberate mistake: the text `old` of the rewritten kernel source (or of a rewritten
+    header, when `source` is one) replaced by `new`.  tests/_build/emu/mutants/<tag>/libsfbert_emu.so.  For the check
+    that the tests on the host model notice mistakes in the real kernels (test_host_model_mutants.py)."""
+    build()
+    gen = os.path.join(BUILD, "sf-bert_amd", "csrc")
+    out = os.path.join(BUILD, "mutants", tag)
+    mgen = os.path.join(out, "sf-bert_amd", "csrc")
+    os.makedirs(mgen, exist_ok=True)
+    os.makedirs(os.path.join(out, "include"), exist_ok=True)
+    with open(os.path.join(out, "include", "sfbert_hip.h"), "w") as f:
+        f.write(open(os.path.join(ROOT, "include", "sfbert_hip.h")).read())
+    lib = os.path.join(out, "libsfbert_emu.so")
+    stamp = os.path.join(out, "digest")
+    digest = _digest() + repr((source, old, new))
+    if os.path.exists(lib) and os.path.exists(stamp) and open(stamp).read() == digest:
+        return lib
+    changed = source if source.endswith(".h") else source.replace(".hip", "_emu.cpp")
+    for name in HEADERS:   # every header beside the units that include it
+        text = open(os.path.join(gen, name)).read()
+        if name == changed:
+            assert text.count(old) == count, (tag, text.count(old))
+            text = text.replace(old, new)
+        with open(os.path.join(mgen, name), "w") as f:
+            f.write(text)
+    flags = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma", "-mf16c"]
+    objects = open(os.path.join(BUILD, "objects")).read().split("\n")
+    # a header is included by the three attention sources; a source stands for itself
+    units = (["fused_attention_emu.cpp", "fused_backward_emu.cpp", "unfused_attention_emu.cpp"] if source.endswith(".h")
+             else [changed])
+
+    def compile_unit(unit):
+        text = open(os.path.join(gen, unit)).read()
+        if unit == changed:
+            assert text.count(old) == count, (tag, text.count(old))
+            text = text.replace(old, new)
+        src = os.path.join(mgen, unit)
+        with open(src, "w") as f:
+            f.write(text)
+        obj = os.path.join(out, unit + ".o")
+        subprocess.check_call([CLANG, "-x", "c++"] + flags + ["-c", src, "-o", obj])
+        return unit, obj
+
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        rebuilt = dict(pool.map(compile_unit, units))
+    linked = [rebuilt.get(os.path.basename(o)[:-2], o) for o in objects]
+    subprocess.check_call([CLANG, "-shared", "-o", lib + ".new"] + linked + ["-lm"])
+    os.replace(lib + ".new", lib)
+    with open(stamp, "w") as f:
+        f.write(digest)
+    return lib
+
+
 def build_variant(tag, defines, source="fused_attention.hip"):
     """The host build with one kernel source compiled under other preprocessor definitions (the opt-in kernel
     variants of sf-bert_amd/build.py): tests/_build/emu/libsfbert_emu_<tag>.so."""
@@ -388,7 +441,10 @@ def load(tag="", defines=()):
     a variant of it, see build_variant)."""
     if tag in _modules:
         return _modules[tag]
-    lib_path = build_sanitized() if tag == "ubsan" else build_variant(tag, defines) if tag else build()
+    if isinstance(defines, dict):   # a mutant: dict(source=, old=, new=[, count=])
+        lib_path = build_mutant(tag, **defines)
+    else:
+        lib_path = build_sanitized() if tag == "ubsan" else build_variant(tag, defines) if tag else build()
     saved = os.environ.get("SFBERT_HIP_LIB")
     os.environ["SFBERT_HIP_LIB"] = lib_path
     try:
