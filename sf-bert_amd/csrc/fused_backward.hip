@@ -14,7 +14,8 @@
 //   * dkdv kernel, one work-group per (batch, head, key-block column), a lane owns one key: per query block
 //         S = Q K^T, dP = dO V^T (row-wise reads of the Q and dO tiles; lse and delta per accumulator element),
 //         dV^T += dO^T P, dK^T += Q^T dS (transposed reads of the dO and Q tiles).
-// bf16 or fp32 tensors (the latter with true fp32 products, further down), head sizes 32 / 64 / 96 / 128, block
+// bf16 or fp32 tensors (the latter with true fp32 products, further down), head sizes 32 / 64 / 96 / 128 and, through
+// the RAGGED forms of the same kernels, every multiple of 8 (bf16) or 4 (fp32) between them, block
 // size 32 or 64; fp32 accumulation and fp32 gradients.
 #include "tiles.hip.h"
 
