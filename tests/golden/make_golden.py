@@ -31,6 +31,16 @@ def main():
     np.savez_compressed(os.path.join(HERE, "attention_backward_dense_causal.npz"), dO=dO, dQ=dQ, dK=dK, dV=dV,
                         shape=np.array([B, L, H, d]), bs=bs, seed=seed, scale=scale)
 
+    # a second shape: blocks of 64, head size 64 (the benchmarked tile shape)
+    B, H, L, d, bs, seed = 1, 1, 192, 64, 64, 2025
+    scale = np.float32(1.0 / np.sqrt(d))
+    Q, K, V, _, _ = causal_case(B, H, L, d, bs, seed)
+    O, _, _ = ref_dense_causal(Q, K, V, float(scale))
+    dO = orc.fill_normal((B, L, H, d), seed + 4)
+    dQ, dK, dV, _ = ref_dense_causal_backward(Q, K, V, dO, float(scale))
+    np.savez_compressed(os.path.join(HERE, "attention_dense_causal_block64.npz"), Q=Q, K=K, V=V, O=O, dO=dO, dQ=dQ, dK=dK,
+                        dV=dV, shape=np.array([B, L, H, d]), bs=bs, seed=seed, scale=scale)
+
     rows, state = 6, 48
     x = orc.fill_normal((rows, state), 77) * 3 + 0.5
     g = orc.fill_normal((state,), 78)

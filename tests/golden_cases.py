@@ -22,8 +22,11 @@ def causal_descriptors(S, L, bs):
     return luts, S.pack_mask(S.element_mask(luts["nt_lut"], bs, S.MASK_CAUSAL_DIAG))
 
 
-def attention_forward(S, dev, zeros):
-    z = np.load(os.path.join(GOLDEN, "attention_dense_causal.npz"))
+FORWARD_FIXTURES = ["attention_dense_causal.npz", "attention_dense_causal_block64.npz"]
+
+
+def attention_forward(S, dev, zeros, fixture=FORWARD_FIXTURES[0]):
+    z = np.load(os.path.join(GOLDEN, fixture))
     B, L, H, d = (int(x) for x in z["shape"])
     bs, scale = int(z["bs"]), float(z["scale"])
     luts, mask = causal_descriptors(S, L, bs)
@@ -48,9 +51,9 @@ def attention_forward(S, dev, zeros):
     assert rel_err(S.bst_sgemm_xn(nn, p2, v, nb).cpu().numpy(), want) <= TOL
 
 
-def attention_backward(S, dev, zeros):
-    z = np.load(os.path.join(GOLDEN, "attention_dense_causal.npz"))
-    g = np.load(os.path.join(GOLDEN, "attention_backward_dense_causal.npz"))
+def attention_backward(S, dev, zeros, fixture=FORWARD_FIXTURES[0]):
+    z = np.load(os.path.join(GOLDEN, fixture))
+    g = z if "dQ" in z.files else np.load(os.path.join(GOLDEN, "attention_backward_dense_causal.npz"))
     B, L, H, d = (int(x) for x in z["shape"])
     bs, scale = int(z["bs"]), float(z["scale"])
     luts, mask = causal_descriptors(S, L, bs)

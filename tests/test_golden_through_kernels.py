@@ -22,13 +22,15 @@ def host_backend(E):
 
 
 @pytest.mark.gpu
-def test_attention_forward_against_the_reference_outputs_on_the_device():
-    golden_cases.attention_forward(*device_backend())
+@pytest.mark.parametrize("fixture", golden_cases.FORWARD_FIXTURES)
+def test_attention_forward_against_the_reference_outputs_on_the_device(fixture):
+    golden_cases.attention_forward(*device_backend(), fixture=fixture)
 
 
 @pytest.mark.gpu
-def test_attention_backward_against_the_reference_outputs_on_the_device():
-    golden_cases.attention_backward(*device_backend())
+@pytest.mark.parametrize("fixture", golden_cases.FORWARD_FIXTURES)
+def test_attention_backward_against_the_reference_outputs_on_the_device(fixture):
+    golden_cases.attention_backward(*device_backend(), fixture=fixture)
 
 
 @pytest.mark.gpu
@@ -38,12 +40,14 @@ def test_layer_ops_and_loss_against_the_reference_outputs_on_the_device():
     golden_cases.cross_entropy(S, dev)
 
 
-def test_attention_forward_against_the_reference_outputs_on_the_host_model(E):
-    golden_cases.attention_forward(*host_backend(E))
+@pytest.mark.parametrize("fixture", golden_cases.FORWARD_FIXTURES)
+def test_attention_forward_against_the_reference_outputs_on_the_host_model(E, fixture):
+    golden_cases.attention_forward(*host_backend(E), fixture=fixture)
 
 
-def test_attention_backward_against_the_reference_outputs_on_the_host_model(E):
-    golden_cases.attention_backward(*host_backend(E))
+@pytest.mark.parametrize("fixture", golden_cases.FORWARD_FIXTURES)
+def test_attention_backward_against_the_reference_outputs_on_the_host_model(E, fixture):
+    golden_cases.attention_backward(*host_backend(E), fixture=fixture)
 
 
 def test_layer_ops_and_loss_against_the_reference_outputs_on_the_host_model(E):

@@ -62,8 +62,9 @@ def test_attention_bit_exact_vs_reference_dense_causal(bs, L, d):
     assert np.array_equal(O3, want)
 
 
-def test_attention_matches_golden_fixture():
-    fx = np.load(os.path.join(GOLDEN, "attention_dense_causal.npz"))
+@pytest.mark.parametrize("fixture", ["attention_dense_causal.npz", "attention_dense_causal_block64.npz"])
+def test_attention_matches_golden_fixture(fixture):
+    fx = np.load(os.path.join(GOLDEN, fixture))
     B, L, H, d = (int(v) for v in fx["shape"])
     bs = int(fx["bs"])
     Q, K, V, luts, words = causal_case(B, H, L, d, bs, seed=int(fx["seed"]))

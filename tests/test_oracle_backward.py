@@ -49,8 +49,9 @@ def test_backward_bit_exact_vs_reference_dense_causal(bs, L, d):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-def test_backward_matches_golden_fixture():
-    fx = np.load(os.path.join(GOLDEN, "attention_backward_dense_causal.npz"))
+@pytest.mark.parametrize("fixture", ["attention_backward_dense_causal.npz", "attention_dense_causal_block64.npz"])
+def test_backward_matches_golden_fixture(fixture):
+    fx = np.load(os.path.join(GOLDEN, fixture))
     B, L, H, d = (int(v) for v in fx["shape"])
     bs = int(fx["bs"])
     Q, K, V, luts, words = causal_case(B, H, L, d, bs, seed=int(fx["seed"]))
