@@ -53,6 +53,8 @@ struct Config {
     int order = 0;        // 0 ascending, 1 descending, n > 1: shuffled with seed n
     int lazy_loads = 1;   // LDS-direct loads land at the wait (1) or when issued (0)
     int resident = 64;    // work-groups in flight at a time
+    bool fixed = false;   // no further work-group is started for lanes that poll (a launch with more work-groups
+                          // than the device keeps resident: what its bounded waits are for)
 };
 
 static Config g_config;
@@ -412,7 +414,7 @@ void launch(dim3 grid, dim3 block, size_t, hipStream_t, const std::function<void
     size_t room = (size_t)g_config.resident;
     while (true) {
         // a launch that polls for other work-groups' results is one whose work-groups are all resident on the device
-        if (g_polling && room < 2048) room += 16;
+        if (g_polling && room < 2048 && !g_config.fixed) room += 16;
         g_polling = false;
         while (active.size() < room && next < total) active.push_back(make_block((uint32_t)next++, nt));
         if (active.empty()) break;
@@ -448,7 +450,8 @@ extern "C" {
 void emu_configure(int order, int lazy_loads, int resident) {
     emu::g_config.order = order;
     emu::g_config.lazy_loads = lazy_loads;
-    emu::g_config.resident = resident > 0 ? resident : 1;
+    emu::g_config.fixed = resident < 0;   // a negative count: exactly that many, whatever the lanes do
+    emu::g_config.resident = resident > 0 ? resident : resident < 0 ? -resident : 1;
 }
 void emu_reset_counts() {
     memset(emu::g_counts, 0, sizeof emu::g_counts);

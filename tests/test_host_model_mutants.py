@@ -5,6 +5,7 @@ one tile short -- and expects the corresponding test of test_emulated_kernels.py
 lane orders / load timings it uses (and the unmodified build to pass, which the CPU suite checks anyway).
 A build per mistake: minutes.  Run with `pytest tests/test_host_model_mutants.py --mutants`."""
 import pytest
+import torch
 
 import emu_lib
 import test_emulated_kernels as T
@@ -58,3 +59,45 @@ def test_a_seeded_mistake_is_noticed(E, name, request):
             noticed.append((order, lazy, str(failure)[:80]))
     print(name, "noticed under", [(o, l) for o, l, _ in noticed])
     assert noticed, "the mistake went unnoticed under every order and timing"
+
+
+def test_a_merge_that_runs_out_of_its_wait_is_reported_and_the_workspace_recovers(E, request):
+    """A merge that waits for a partial record nobody writes (the plan's copy on the device is altered: the merge of the
+    last records expects one record more than exist, whose flag -- in the padding of the flag area -- is never set), in
+    a build with a short bound on the wait (64 polls instead of 2^20): the merge gives up, the launch reports status
+    1, nothing hangs and every other row is right; the binding then clears the workspace (sfb_stream_reset), and the
+    next launch, with the plan as built, is right and reports 0."""
+    if not request.config.getoption("--mutants"):
+        pytest.skip("needs --mutants (a build of the host model)")
+    import numpy as np
+    import oracle_lib as orc
+    short = emu_lib.load("mutant_short_merge_wait", dict(
+        source="fused_attention.hip", old="constexpr uint32_t kMaxPolls = 1u << 20;", new="constexpr uint32_t kMaxPolls = 1u << 6;"))
+    emu_lib.configure()
+    bs, nb, B, H, d = 64, 5, 2, 2, 64
+    luts = short.build_luts(T.layout(short, nb))   # two long rows per head: they are what the plan cuts
+    Q, K, V = T.inputs(B, nb * bs, H, d, 77, True)
+    q, k, v = (T.dev(x, True) for x in (Q, K, V))
+    nn = short.to_device(luts["nn_lut"])
+    stream = short.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=24, d=d, bf16=True, masked=False)
+    n_parts = stream["plan"].n_parts
+    assert n_parts > 0 and (4 * n_parts) % 256 != 0, "the flag area has padding after the last flag"
+    ws = T.zeros(short.stream_workspace_bytes(stream, d))
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125)
+    good = stream["blob"].copy()
+    merges = stream["merges"]
+    last = int(np.argmax(merges["part"] + merges["nparts"]))
+    assert merges["part"][last] + merges["nparts"][last] == n_parts
+    merges["nparts"][last] += 1            # (a view of stream["blob"])
+    starved = (int(merges["batch"][last]), int(merges["head"][last]), int(merges["row"][last]))
+    out = short.fused_attention_streamed(q, k, v, nn, short.to_device(stream["blob"]), stream, ws, bs, luts["blocks"], 0.125,
+                                         out=emu_lib.empty((B, nb * bs, H, d), torch.float32, fill=7.0)).numpy()
+    assert short.stream_status(stream, d, ws) == 1          # (and the binding has reset the workspace)
+    b, h, r = starved
+    assert (out[b, r * bs:(r + 1) * bs, h] == 7.0).all(), "the starved row is left alone"
+    out[b, r * bs:(r + 1) * bs, h] = want[b, r * bs:(r + 1) * bs, h]
+    assert T.rel_err(out, want) <= T.TOL[True]
+    for _ in range(2):
+        got = short.fused_attention_streamed(q, k, v, nn, short.to_device(good), stream, ws, bs, luts["blocks"], 0.125)
+        assert short.stream_status(stream, d, ws) == 0
+        assert T.rel_err(got.numpy(), want) <= T.TOL[True]

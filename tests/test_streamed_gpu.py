@@ -147,3 +147,40 @@ def test_streamed_overflowing_scores_take_the_general_loop():
     from gpu_common import run_fused
     assert rel_err(run_fused(Q, K, V, luts, bs, 0.125, bf16=True), want) <= TOL_BF16
     assert rel_err(run_fused(Q, K, V, luts, bs, 0.125, bf16=True, max_blocks=3), want) <= TOL_BF16
+
+
+@pytest.mark.needs_device
+def test_a_merge_whose_record_never_arrives_gives_up_and_the_workspace_recovers():
+    """Failure handling, forced from the host: in the plan's copy on the device the merge of the last records expects
+    one record more than exist (its flag, in the padding of the flag area, is never set).  The merge's wait is
+    bounded (about a second), so the launch ends normally with status 1 and every other row right; the binding then
+    clears the workspace (sfb_stream_reset) and the next launch, with the plan as built, is right and reports 0."""
+    bs, nb, B, H, d = 64, 16, 2, 3, 64
+    luts = sfb.build_luts(PATTERNS["bigbird"](nb))
+    Q, K, V = qkv(B, nb * bs, H, d, seed=515, bf16=True)
+    q, k, v = (dev(x, True) for x in (Q, K, V))
+    nn = sfb.to_device(luts["nn_lut"])
+    stream = sfb.build_stream(luts["nn_lut"], nb, B, H, bs, wg_slots=61)
+    n_parts = stream["plan"].n_parts
+    assert n_parts > 0 and (4 * n_parts) % 256 != 0, "the flag area has padding after the last flag"
+    ws = torch.zeros(sfb.stream_workspace_bytes(stream, d), dtype=torch.uint8, device="cuda")
+    want = orc.attention(Q, K, V, luts["nn_lut"], bs, 0.125, nthreads=THREADS)
+    good = stream["blob"].copy()
+    merges = stream["merges"]   # a view of stream["blob"]
+    last = int(np.argmax(merges["part"] + merges["nparts"]))
+    assert merges["part"][last] + merges["nparts"][last] == n_parts
+    merges["nparts"][last] += 1
+    b, h, r = int(merges["batch"][last]), int(merges["head"][last]), int(merges["row"][last])
+    out = torch.full((B, nb * bs, H, d), 7.0, device="cuda")
+    sfb.fused_attention_streamed(q, k, v, nn, sfb.to_device(stream["blob"]), stream, ws, bs, luts["blocks"], 0.125, out=out)
+    torch.cuda.synchronize()
+    assert sfb.stream_status(stream, d, ws) == 1
+    got = out.cpu().numpy()
+    assert (got[b, r * bs:(r + 1) * bs, h] == 7.0).all()
+    got[b, r * bs:(r + 1) * bs, h] = want[b, r * bs:(r + 1) * bs, h]
+    assert rel_err(got, want) <= TOL_BF16
+    for _ in range(2):
+        out = sfb.fused_attention_streamed(q, k, v, nn, sfb.to_device(good), stream, ws, bs, luts["blocks"], 0.125)
+        torch.cuda.synchronize()
+        assert sfb.stream_status(stream, d, ws) == 0
+        assert rel_err(out.cpu().numpy(), want) <= TOL_BF16
