@@ -40,6 +40,10 @@ KERNEL_SOURCES = ["fused_attention.hip", "fused_backward.hip", "unfused_attentio
 HOST_SOURCES = ["descriptors.cpp"]
 HEADERS = ["common.hip.h", "tiles.hip.h", "tile_index.h"]
 
+# plain x86-64 (no instruction-set extensions: the build runs wherever the tests do); products and sums are not
+# contracted, so that host arithmetic rounds where the kernels' source says it does
+HOST_FLAGS = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off"]
+
 OPS = ["none", "block_barrier", "block_and", "wave_barrier", "mfma_bf16", "mfma_f32", "readfirstlane", "readlane",
        "ballot", "shfl_xor", "ds_read_tr16", "dpp", "yield"]
 
@@ -286,8 +290,7 @@ def build(verbose=False):
     with open(selftest, "w") as f:
         f.write(rewrite(open(os.path.join(EMU, "selftest_kernels.hip")).read(), "selftest_kernels.hip"))
     units += [selftest] + [os.path.join(CSRC, f) for f in HOST_SOURCES] + [os.path.join(EMU, "emu_runtime.cpp")]
-    flags = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off",
-             "-mavx2", "-mfma", "-mf16c"]
+    flags = HOST_FLAGS
 
     def compile_unit(src):
         obj = os.path.join(BUILD, os.path.basename(src) + ".o")
@@ -323,7 +326,7 @@ def build_sanitized(verbose=False):
     units = [os.path.join(gen, name.replace(".hip", "_emu.cpp")) for name in KERNEL_SOURCES]
     units += [os.path.join(gen, "selftest_kernels_emu.cpp")] + [os.path.join(CSRC, f) for f in HOST_SOURCES]
     units += [os.path.join(EMU, "emu_runtime.cpp")]
-    flags = ["-O1", "-g1", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma", "-mf16c",
+    flags = [f if f != "-g0" else "-g1" for f in HOST_FLAGS] + [
              "-fsanitize=undefined", "-fno-sanitize=vptr,function", "-fno-sanitize-recover=undefined",
              "-fsanitize-trap=undefined"]
 
@@ -379,7 +382,7 @@ def build_mutant(tag, source, old, new, count=1):
             text = text.replace(old, new)
         with open(os.path.join(mgen, name), "w") as f:
             f.write(text)
-    flags = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma", "-mf16c"]
+    flags = HOST_FLAGS
     objects = open(os.path.join(BUILD, "objects")).read().split("\n")
     # a header is included by the three attention sources; a source stands for itself
     units = (["fused_attention_emu.cpp", "fused_backward_emu.cpp", "unfused_attention_emu.cpp"] if source.endswith(".h")
@@ -418,8 +421,7 @@ def build_variant(tag, defines, source="fused_attention.hip"):
         return lib
     src = os.path.join(BUILD, "sf-bert_amd", "csrc", source.replace(".hip", "_emu.cpp"))
     obj = os.path.join(BUILD, "%s_%s.o" % (os.path.basename(src), tag))
-    flags = ["-O1", "-g0", "-std=c++17", "-fPIC", "-I" + EMU, "-Wno-everything", "-ffp-contract=off", "-mavx2", "-mfma",
-             "-mf16c"] + ["-D" + d for d in defines]
+    flags = HOST_FLAGS + ["-D" + d for d in defines]
     subprocess.check_call([CLANG, "-x", "c++"] + flags + ["-c", src, "-o", obj])
     others = [o for o in open(os.path.join(BUILD, "objects")).read().split("\n")
               if os.path.basename(o) != os.path.basename(src) + ".o"]
