@@ -181,10 +181,12 @@ static void execute(int op, Lane* wave_lanes, const std::vector<int>& who, bool 
         break;
     case OP_MFMA_BF16:
     case OP_MFMA_F32: {
+        // D[m][n] = C[m][n] + sum_k A[m][k] B[k][n] in fp32, inactive lanes' operands read as zeros
         const int K = op == OP_MFMA_BF16 ? 16 : 2, per_lane = K / 2;
-        static float A[32][16], B[16][32];
+        static float A[32][16], B[16][32], D[32][32];
         memset(A, 0, sizeof A);
         memset(B, 0, sizeof B);
+        memset(D, 0, sizeof D);
         for (int i : who) {
             const Lane& l = wave_lanes[i];
             const int r = l.lane % 32, h = l.lane / 32;
@@ -193,15 +195,15 @@ static void execute(int op, Lane* wave_lanes, const std::vector<int>& who, bool 
                 B[per_lane * h + e][r] = op == OP_MFMA_BF16 ? bf16_value(l.b16[e]) : l.b32;
             }
         }
+        for (int m = 0; m < 32; ++m)
+            for (int k = 0; k < K; ++k) {
+                const float a = A[m][k];
+                for (int n = 0; n < 32; ++n) D[m][n] += a * B[k][n];
+            }
         for (int i : who) {
             Lane& l = wave_lanes[i];
             const int n = l.lane % 32, h = l.lane / 32;
-            for (int e = 0; e < 16; ++e) {
-                const int m = 8 * (e / 4) + 4 * h + e % 4;
-                double sum = 0.0;
-                for (int k = 0; k < K; ++k) sum += (double)A[m][k] * (double)B[k][n];
-                l.acc[e] = (float)((double)l.acc[e] + sum);
-            }
+            for (int e = 0; e < 16; ++e) l.acc[e] += D[8 * (e / 4) + 4 * h + e % 4][n];
         }
         break;
     }
