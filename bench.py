@@ -196,6 +196,29 @@ def time_unfused(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, fused_ms):
     return dict(ms_per_call=ms, fused_speedup=ms / fused_ms, sp_storage="bf16" if bf16 else "f32", **parts)
 
 
+def time_dsd_scheduled(sfb, torch, luts, q, v, bs, blocks, bf16, max_blocks=16):
+    """The two dsd products (P V over block-rows, P^T dO over block-columns) launched over work items of at most
+    max_blocks blocks against the launch by lines, each with its HBM rate on the algorithmic bytes."""
+    B, L, H, d = q.shape
+    nb = L // bs
+    store = torch.bfloat16 if bf16 else torch.float32
+    P = torch.randn((B, H, blocks, bs, bs), device="cuda").to(store)
+    c = torch.empty((B, L, H, d), device="cuda", dtype=torch.float32)
+    moved = P.numel() * P.element_size() + v.numel() * v.element_size() + c.numel() * 4
+    out = {"max_blocks": max_blocks}
+    for name, key, op in (("nn", "nn_lut", sfb.NN_OP), ("tn", "tn_lut", sfb.TN_OP)):
+        lut = sfb.to_device(luts[key])
+        sched = sfb.build_schedule(luts[key], nb, max_blocks)
+        items = sfb.to_device(sched["items"])
+        ws = torch.empty(max(sfb.dsd_workspace_bytes(sched, B, H, bs, d), 256), dtype=torch.uint8, device="cuda")
+        by_items = _time(torch, lambda: sfb.bst_sgemm_xn_scheduled(lut, P, v, nb, items, sched, ws, op=op, c=c), 200, 20)
+        by_lines = _time(torch, lambda: sfb.bst_sgemm_xn(lut, P, v, nb, op=op, c=c), 200, 20)
+        out.update({name + "_items": sched["n_items"], name + "_cut_lines_parts": sched["n_parts"],
+                    name + "_ms": by_items, name + "_hbm_GBs": moved / by_items / 1e6,
+                    name + "_by_lines_ms": by_lines, name + "_by_lines_hbm_GBs": moved / by_lines / 1e6})
+    return out
+
+
 def time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16):
     """Backward of the unfused path from the stored P (dV, dP, dS, dK, dQ), each stage and the whole chain, with
     the HBM rate of the two memory-bound stage types on their algorithmic bytes."""
@@ -472,6 +495,7 @@ def main():
         if bf16 or d == 64:
             extra("streamed", time_streamed, sfb, torch, luts, q, k, v, bs, blocks, scale, flops, peak)
         extra("unfused", time_unfused, sfb, torch, luts, q, k, v, bs, blocks, scale, bf16, kernel_ms)
+        extra("dsd_scheduled", time_dsd_scheduled, sfb, torch, luts, q, v, bs, blocks, bf16)
         extra("backward_unfused", time_backward, sfb, torch, luts, q, k, v, bs, blocks, scale, bf16)
         extra("backward_fused", time_fused_backward, sfb, torch, luts, q, k, v, bs, blocks, scale, args.max_blocks, flops)
         if args.workload == "c4":

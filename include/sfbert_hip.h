@@ -448,6 +448,23 @@ int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const v
                uint32_t lut_heads, uint32_t lut_dim, uint32_t op, uint32_t magic, uint32_t shift,
                uint32_t max_lut);
 
+/* MI355X addition (no reference counterpart): sfb_dsd_xn launched over work items instead of lines, so that no
+ * work-group walks a long block-row (NN) or block-column (TN) alone -- BigBird's global rows and columns have 64 blocks
+ * at L = 4096 against 8 elsewhere, and the work-group that owns one is the tail of the plain launch.  items [dev]:
+ * sfb_build_schedule() over the same look-up table (the NN LUT for SFB_NN_OP, the TN LUT for SFB_TN_OP), or
+ * [lut_heads][n_items] from sfb_build_schedule_heads() with one table per head; n_items, n_heavy, n_parts as returned
+ * there.  The chunks of a cut line leave their sums in workspace ([dev], 256-byte aligned,
+ * sfb_dsd_workspace_bytes() bytes, no initial contents needed; may be NULL when n_parts is 0) and a second small
+ * kernel adds them in chunk order, so results do not depend on timing.  Both operands must have one type
+ * (SFB_ERR_DTYPE otherwise); head sizes as for sfb_dsd_xn. */
+size_t sfb_dsd_workspace_bytes(uint32_t n_parts, uint32_t batch_dim, uint32_t head_dim, uint32_t block_size,
+                               uint32_t state_dim);
+int sfb_dsd_xn_scheduled(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
+                         int a_dtype, int b_dtype, const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy,
+                         uint32_t n_parts, void* workspace, size_t workspace_bytes, uint32_t block_size,
+                         uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks_b, uint32_t ctx_blks_c,
+                         uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads, uint32_t lut_dim, uint32_t op);
+
 /* fusion_attention1 / fusion_attention2 (fusion_blocksparse.h:400-455, 1212-1268): sdd + masked
  * softmax in one kernel, y = P in the sparse layout (fp32 or bf16).  One work-group owns a whole
  * block-row, so the reference's rblk_flag / rblk_flag1 / Max / Sum scratch and its spin-waits are not

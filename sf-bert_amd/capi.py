@@ -52,6 +52,7 @@ lib.sfb_suggest_max_blocks.restype = C.c_uint32
 lib.sfb_model_workspace_bytes.restype = C.c_size_t
 lib.sfb_split_softmax_scratch_bytes.restype = C.c_size_t
 lib.sfb_backward_workspace_bytes.restype = C.c_size_t
+lib.sfb_dsd_workspace_bytes.restype = C.c_size_t
 lib.sfb_resident_work_groups.restype = C.c_uint32
 lib.sfb_resident_work_groups_for.restype = C.c_uint32
 lib.sfb_stream_workspace_bytes.restype = C.c_size_t
@@ -73,7 +74,8 @@ EXPORTED = [
     "sfb_fused_attention", "sfb_fused_attention_scheduled", "sfb_fused_attention_scheduled_to",
     "sfb_fused_attention_scheduled_strided", "sfb_fused_attention_scheduled_heads",
     "sfb_fused_attention_scheduled_lse", "sfb_fused_attention_backward", "sfb_backward_workspace_bytes",
-    "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_fused_sdd_softmax",
+    "sfb_sdd_nt", "sfb_masked_softmax", "sfb_masked_softmax_grad", "sfb_dsd_xn", "sfb_dsd_xn_scheduled",
+    "sfb_dsd_workspace_bytes", "sfb_fused_sdd_softmax",
     "sfb_split_softmax_scratch_bytes", "sfb_fused_sdd_softmax_split", "sfb_row_dot", "sfb_sdd_softmax_grad",
     "sfb_bias_act", "sfb_layernorm", "sfb_bias_residual_layernorm", "sfb_add_matrix", "sfb_transpose_0213", "sfb_embedding_lookup", "sfb_cast_f32_bf16",
     "sfb_pack_qkv", "sfb_gemm_release", "sfb_gemm", "sfb_gemm_bias", "sfb_gemm_bias_gelu", "sfb_gemm_bias_gelu_scaled", "sfb_encoder_layer_workspace_bytes", "sfb_encoder_layer_forward",
@@ -586,6 +588,30 @@ def bst_sgemm_xn(lut, a, b, ctx_blks_c, op=NN_OP, lut_heads=1, magic=1, shift=0,
                           C.c_uint32(ctx_blks_c), C.c_uint32(H), C.c_uint32(d), C.c_uint32(lut_heads),
                           C.c_uint32(ctx_blks_c + blocks), C.c_uint32(op), C.c_uint32(magic),
                           C.c_uint32(shift), C.c_uint32(max_lut)), "sfb_dsd_xn")
+    return c
+
+
+def dsd_workspace_bytes(sched, batch, heads, block_size, d):
+    return int(lib.sfb_dsd_workspace_bytes(C.c_uint32(sched["n_parts"]), C.c_uint32(batch), C.c_uint32(heads),
+                                           C.c_uint32(block_size), C.c_uint32(d)))
+
+
+def bst_sgemm_xn_scheduled(lut, a, b, ctx_blks_c, items, sched, workspace, op=NN_OP, lut_heads=1, c=None):
+    """sfb_dsd_xn_scheduled: bst_sgemm_xn launched over the work items of build_schedule(lut) (or
+    build_schedule_heads with a table per head); workspace: device bytes, dsd_workspace_bytes() of them, or None
+    when no line is cut."""
+    import torch
+    B, H, blocks, bs, _ = a.shape
+    _, Lb, _, d = b.shape
+    if c is None:
+        c = torch.empty((B, ctx_blks_c * bs, H, d), device=b.device, dtype=torch.float32)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _check(lib.sfb_dsd_xn_scheduled(_stream(), _dev(lut), _dev(a), _dev(b), _dev(c), _dtype_code(a), _dtype_code(b),
+                                    _dev(items), C.c_uint32(sched["n_items"]), C.c_uint32(sched["n_heavy"]),
+                                    C.c_uint32(sched["n_parts"]), _dev(workspace), C.c_size_t(ws_bytes),
+                                    C.c_uint32(bs), C.c_uint32(blocks), C.c_uint32(B), C.c_uint32(Lb // bs),
+                                    C.c_uint32(ctx_blks_c), C.c_uint32(H), C.c_uint32(d), C.c_uint32(lut_heads),
+                                    C.c_uint32(ctx_blks_c + blocks), C.c_uint32(op)), "sfb_dsd_xn_scheduled")
     return c
 
 

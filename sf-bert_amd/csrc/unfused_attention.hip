@@ -1183,9 +1183,65 @@ struct DsdParams {
     float* c;               // dense result
     uint32_t blocks, batch, heads, nb_b, nb_c, lut_stride, groups;
     uint32_t state;         // head size of the dense tensors (the kernels' D is the next multiple of 32)
+    // Scheduled launches (items != nullptr): one work-group per work item of sfb_build_schedule over `lut` instead of
+    // one per line.  A chunk of a split line leaves its sum in a record of `partials`
+    // ([batch * heads][n_parts][BS][D] floats); dsd_reduce_kernel adds the records of a line afterwards.
+    const sfb_work_item* items;
+    uint32_t item_stride, ranks, heavy, n_parts;
+    float* partials;
 };
 
-template <int BS, int D, typename TA, typename TB, bool RAGGED = false>
+// The line (block-row of an NN launch, block-column of a TN launch) of a work-group, or the part of it that a work
+// item of a scheduled launch covers.
+struct DsdLine {
+    uint32_t bh, line;
+    uint32_t off, count;    // the look-up entries lut[off .. off + count) of the head's table
+    uint32_t record;        // chunk of a split line: index + 1 of its record among the (batch, head)'s; else 0
+    bool valid;
+};
+
+template <bool ITEMS>
+__device__ __forceinline__ DsdLine decode_dsd_line(const DsdParams& p) {
+    DsdLine w;
+    if constexpr (ITEMS) {
+        const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.ranks, p.heavy);
+        w.valid = id.valid;
+        w.bh = id.bh;
+        const sfb_work_item it = p.items[(size_t)(id.valid ? id.bh % p.heads : 0u) * p.item_stride + id.rank];
+        if (it.row == SFB_WORK_ITEM_SKIP) w.valid = false;   // filler of a head whose list is shorter than the longest
+        w.line = __builtin_amdgcn_readfirstlane(it.row);
+        w.off = __builtin_amdgcn_readfirstlane(it.lut_first);
+        w.count = __builtin_amdgcn_readfirstlane(it.count);
+        w.record = __builtin_amdgcn_readfirstlane(it.nchunks > 1 ? it.part + it.chunk + 1 : 0u);
+        return w;
+    }
+    // Lines are taken from both ends of the context inwards, the last and the first one of every head before
+    // anything else: the long rows of causal layouts are the last ones (blocksparse.h:746-748), those of layouts
+    // with global tokens the first and the last; started late, a long line is the tail of the launch.
+    const WorkId id = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c, p.nb_c >= 2 ? 2 : 0);
+    w.valid = id.valid;
+    w.bh = id.bh;
+    w.line = (id.rank & 1u) ? id.rank / 2 : p.nb_c - 1 - id.rank / 2;
+    w.record = 0;
+    if (id.valid) {
+        const sfb_uint2 header = p.lut[(size_t)(id.bh % p.heads) * p.lut_stride + w.line];
+        w.off = __builtin_amdgcn_readfirstlane(header.x);
+        w.count = __builtin_amdgcn_readfirstlane(header.y);
+    } else {
+        w.off = w.count = 0;
+    }
+    return w;
+}
+
+// Where a lane's output row goes: the dense result, or the record of a split line's chunk (rows of D floats).
+template <int BS, int D, bool ITEMS>
+__device__ __forceinline__ float* dsd_output_row(const DsdParams& p, const DsdLine& w, uint32_t b, uint32_t h,
+                                                 uint32_t row_in_block, uint32_t hd) {
+    if (ITEMS && w.record) return p.partials + ((((size_t)w.bh * p.n_parts + (w.record - 1)) * BS) + row_in_block) * D;
+    return p.c + token_offset(b, w.line * BS + row_in_block, h, p.nb_c * BS, p.heads, hd);
+}
+
+template <int BS, int D, typename TA, typename TB, bool RAGGED = false, bool ITEMS = false>
 __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && sizeof(TB) == 2) ? 1 : 2) void dsd_tn_kernel(DsdParams p) {
     constexpr int NO = D / 32;
     constexpr bool kFast = sizeof(TA) == 2 && sizeof(TB) == 2 && BS == 64;
@@ -1195,20 +1251,18 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
     constexpr int LDS_BYTES = kFast ? 4 * TILE : BS * X_STRIDE * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
-    // block-columns from both ends of the context inwards, the last and the first one of every head before anything
-    // else (the columns of global tokens are the long ones; see dsd_nn_kernel)
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c, p.nb_c >= 2 ? 2 : 0);
+    // block-columns (the columns of global tokens are the long ones), or work items
+    const DsdLine work = decode_dsd_line<ITEMS>(p);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
-    const uint32_t col = (work.rank & 1u) ? work.rank / 2 : p.nb_c - 1 - work.rank / 2;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t kn = lane & 31, half = lane >> 5;
     const uint32_t key_in_block = wave * 32 + kn;
     const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
     const uint32_t row_stride = p.heads * hd;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
-    const uint32_t off = __builtin_amdgcn_readfirstlane(lut[col].x), count = __builtin_amdgcn_readfirstlane(lut[col].y);
-    float* c_row = p.c + token_offset(b, col * BS + key_in_block, h, p.nb_c * BS, p.heads, hd);
+    const uint32_t off = work.off, count = work.count;
+    float* c_row = dsd_output_row<BS, D, ITEMS>(p, work, b, h, key_in_block, hd);
     const TA* A = (const TA*)p.a + (size_t)work.bh * p.blocks * BS * BS;
     const TB* X = (const TB*)p.b;
 
@@ -1303,14 +1357,15 @@ __global__ __launch_bounds__(BS * 2, (D > 64 && BS == 64 && sizeof(TA) == 2 && s
 #pragma unroll
         for (int ig = 0; ig < 4; ++ig) {
             const f32x4 out = {acc[mt][ig * 4 + 0], acc[mt][ig * 4 + 1], acc[mt][ig * 4 + 2], acc[mt][ig * 4 + 3]};
-            if (!RAGGED || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(c_row + mt * 32 + ig * 8 + half * 4) = out;
+            // (the rows of a record are D wide; the reduction reads their first hd columns only)
+            if (!RAGGED || (ITEMS && work.record) || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(c_row + mt * 32 + ig * 8 + half * 4) = out;
         }
 }
 
 // ---------------------------------------------------------------------------------------------
 // dsd: one work-group per (batch, head, block-row), V staged through LDS, P read in operand layout
 // ---------------------------------------------------------------------------------------------
-template <int BS, int D, typename TP, typename TV, bool RAGGED = false>
+template <int BS, int D, typename TP, typename TV, bool RAGGED = false, bool ITEMS = false>
 __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int KT = BS / 32, NO = D / 32;
     constexpr bool kBf16 = sizeof(TV) == 2;
@@ -1320,21 +1375,18 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
     constexpr int LDS_BYTES = kBf16 ? (kRing ? 4 : 2) * TD::TILE_BYTES : TF::V_FLOATS * 4;
     __shared__ __attribute__((aligned(1024))) uint8_t smem[LDS_BYTES];
 
-    // Block-rows are taken from both ends of the context inwards, the last and the first one of every head before
-    // anything else: the long rows of causal layouts are the last ones (blocksparse.h:746-748), those of layouts
-    // with global tokens the first and the last; started late, a long row is the tail of the launch.
-    const WorkId work = decode_work(blockIdx.x, p.batch * p.heads, p.nb_c, p.nb_c >= 2 ? 2 : 0);
+    // block-rows, or work items
+    const DsdLine work = decode_dsd_line<ITEMS>(p);
     if (!work.valid) return;
     const uint32_t b = work.bh / p.heads, h = work.bh % p.heads;
-    const uint32_t r = (work.rank & 1u) ? work.rank / 2 : p.nb_c - 1 - work.rank / 2;
     const uint32_t t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t qn = lane & 31, half = lane >> 5;
     const uint32_t q_in_block = wave * 32 + qn;
     const uint32_t hd = RAGGED ? p.state : (uint32_t)D;
     const uint32_t row_stride = p.heads * hd;
     const sfb_uint2* lut = p.lut + (size_t)h * p.lut_stride;
-    const uint32_t off = __builtin_amdgcn_readfirstlane(lut[r].x), count = __builtin_amdgcn_readfirstlane(lut[r].y);
-    float* o_row = p.c + token_offset(b, r * BS + q_in_block, h, p.nb_c * BS, p.heads, hd);
+    const uint32_t off = work.off, count = work.count;
+    float* o_row = dsd_output_row<BS, D, ITEMS>(p, work, b, h, q_in_block, hd);
     const TP* P = (const TP*)p.a + (size_t)work.bh * p.blocks * BS * BS;
     const TV* V = (const TV*)p.b;
 
@@ -1531,8 +1583,27 @@ __global__ __launch_bounds__(BS * 2, 2) void dsd_nn_kernel(DsdParams p) {
         for (int ig = 0; ig < 4; ++ig) {
             const f32x4 out = {o_acc[mt][ig * 4 + 0], o_acc[mt][ig * 4 + 1], o_acc[mt][ig * 4 + 2],
                                o_acc[mt][ig * 4 + 3]};
-            if (!RAGGED || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
+            if (!RAGGED || (ITEMS && work.record) || mt * 32 + ig * 8 + half * 4 < hd) *(f32x4*)(o_row + mt * 32 + ig * 8 + half * 4) = out;
         }
+}
+
+// Sum of the records of the split lines of a scheduled dsd launch, in chunk order (so the result does not depend on
+// which chunk finished when), written to the lines' rows of the result.  grid (n_items, batch * heads): the
+// work-groups of the first chunk of a split line do the sums, all others leave at once.  The records are complete when
+// this kernel starts: nobody waits for anybody.
+__global__ __launch_bounds__(256) void dsd_reduce_kernel(DsdParams p, uint32_t bs, uint32_t dpad) {
+    const uint32_t bh = blockIdx.y, b = bh / p.heads, h = bh % p.heads;
+    const sfb_work_item it = p.items[(size_t)h * p.item_stride + blockIdx.x];
+    if (it.row == SFB_WORK_ITEM_SKIP || it.nchunks <= 1 || it.chunk != 0) return;
+    const uint32_t vecs_per_row = dpad / 4, vecs = bs * vecs_per_row;
+    for (uint32_t vec = threadIdx.x; vec < vecs; vec += 256) {
+        const uint32_t row = vec / vecs_per_row, c4 = vec % vecs_per_row;
+        if (c4 * 4 >= p.state) continue;
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (uint32_t ch = 0; ch < it.nchunks; ++ch)
+            sum += *(const f32x4*)(p.partials + (((size_t)bh * p.n_parts + it.part + ch) * bs + row) * dpad + c4 * 4);
+        *(f32x4*)(p.c + token_offset(b, it.row * bs + row, h, p.nb_c * bs, p.heads, p.state) + c4 * 4) = sum;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2005,12 +2076,21 @@ extern "C" int sfb_masked_softmax(sfb_stream_t stream, const sfb_uint2* lut, con
     return launch_status();
 }
 
-extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
-                          int a_dtype, int b_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
-                          uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim,
-                          uint32_t lut_heads, uint32_t lut_dim, uint32_t op, uint32_t magic, uint32_t shift,
-                          uint32_t max_lut) {
-    (void)magic; (void)shift; (void)max_lut;  // grid decomposition / smem sizing of the reference kernel
+extern "C" size_t sfb_dsd_workspace_bytes(uint32_t n_parts, uint32_t batch_dim, uint32_t head_dim, uint32_t block_size,
+                                          uint32_t state_dim) {
+    // records of the kernels' D floats a row
+    return (size_t)batch_dim * head_dim * n_parts * block_size * padded_head_state(state_dim) * sizeof(float);
+}
+
+// One launch of a dsd kernel: a work-group per line (items null) or per work item.
+static int dsd_launch(hipStream_t s, const DsdParams& p, int a_dtype, int b_dtype, uint32_t block_size, uint32_t state_dim,
+                      uint32_t op);
+
+static int dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c, int a_dtype,
+                  int b_dtype, const sfb_work_item* items, uint32_t n_items, uint32_t n_heavy, uint32_t n_parts,
+                  void* workspace, size_t workspace_bytes, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                  uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
+                  uint32_t lut_dim, uint32_t op) {
     if (!lut || !a || !b || !c) return SFB_ERR_NULL_POINTER;
     if (check_dtype(a_dtype) || check_dtype(b_dtype)) return SFB_ERR_DTYPE;
     if (op != SFB_NN_OP && op != SFB_TN_OP) return SFB_ERR_ARGUMENT;
@@ -2021,9 +2101,76 @@ extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void*
     if (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c) & 15u) return SFB_ERR_ALIGNMENT;
     DsdParams p = {lut, a, b, c, blocks, batch_dim, head_dim, ctx_blks_b, ctx_blks_c,
                    lut_heads > 1 ? lut_dim : 0, bh_groups(batch_dim * head_dim), state_dim};
-    const dim3 grid(p.groups * 8u * ctx_blks_c);
+    if (items) {
+        if (a_dtype != b_dtype) return SFB_ERR_DTYPE;
+        if (n_items == 0 || n_heavy >= n_items) return SFB_ERR_SHAPE;
+        if ((uint64_t)p.groups * 8u * n_items > 0x7fffffffull || (uint64_t)batch_dim * head_dim > 65535u) return SFB_ERR_SHAPE;
+        const size_t need = sfb_dsd_workspace_bytes(n_parts, batch_dim, head_dim, block_size, state_dim);
+        if (need && (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255u))) return SFB_ERR_WORKSPACE;
+        p.items = items;
+        p.item_stride = lut_heads > 1 ? n_items : 0;
+        p.ranks = n_items; p.heavy = n_heavy; p.n_parts = n_parts;
+        p.partials = (float*)workspace;
+    }
     hipStream_t s = (hipStream_t)stream;
     clear_stale_error();
+    const int rc = dsd_launch(s, p, a_dtype, b_dtype, block_size, state_dim, op);
+    if (rc != SFB_OK || !items || !n_parts) return rc;
+    dsd_reduce_kernel<<<dim3(n_items, batch_dim * head_dim), dim3(256), 0, s>>>(p, block_size, padded_head_state(state_dim));
+    return launch_status();
+}
+
+extern "C" int sfb_dsd_xn(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
+                          int a_dtype, int b_dtype, uint32_t block_size, uint32_t blocks, uint32_t batch_dim,
+                          uint32_t ctx_blks_b, uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim,
+                          uint32_t lut_heads, uint32_t lut_dim, uint32_t op, uint32_t magic, uint32_t shift,
+                          uint32_t max_lut) {
+    (void)magic; (void)shift; (void)max_lut;  // grid decomposition / smem sizing of the reference kernel
+    return dsd_xn(stream, lut, a, b, c, a_dtype, b_dtype, nullptr, 0, 0, 0, nullptr, 0, block_size, blocks, batch_dim,
+                  ctx_blks_b, ctx_blks_c, head_dim, state_dim, lut_heads, lut_dim, op);
+}
+
+extern "C" int sfb_dsd_xn_scheduled(sfb_stream_t stream, const sfb_uint2* lut, const void* a, const void* b, float* c,
+                                    int a_dtype, int b_dtype, const sfb_work_item* items, uint32_t n_items,
+                                    uint32_t n_heavy, uint32_t n_parts, void* workspace, size_t workspace_bytes,
+                                    uint32_t block_size, uint32_t blocks, uint32_t batch_dim, uint32_t ctx_blks_b,
+                                    uint32_t ctx_blks_c, uint32_t head_dim, uint32_t state_dim, uint32_t lut_heads,
+                                    uint32_t lut_dim, uint32_t op) {
+    if (!items) return SFB_ERR_NULL_POINTER;
+    return dsd_xn(stream, lut, a, b, c, a_dtype, b_dtype, items, n_items, n_heavy, n_parts, workspace, workspace_bytes,
+                  block_size, blocks, batch_dim, ctx_blks_b, ctx_blks_c, head_dim, state_dim, lut_heads, lut_dim, op);
+}
+
+static int dsd_launch(hipStream_t s, const DsdParams& p, int a_dtype, int b_dtype, uint32_t block_size, uint32_t state_dim,
+                      uint32_t op) {
+    const dim3 grid(p.groups * 8u * (p.items ? p.ranks : p.nb_c));
+    if (p.items) {
+        // work items: both operands of one type; the streaming kernels of bf16 operands with 64 x 64 blocks and 64
+        // features, otherwise the forms that take any head size
+        if (block_size == 64 && state_dim == 64 && b_dtype == SFB_BF16) {
+            if (op == SFB_TN_OP) dsd_tn_kernel<64, 64, __bf16, __bf16, false, true><<<grid, dim3(128), 0, s>>>(p);
+            else dsd_nn_kernel<64, 64, __bf16, __bf16, false, true><<<grid, dim3(128), 0, s>>>(p);
+            return launch_status();
+        }
+        const uint32_t pad = padded_head_state(state_dim);
+#define SFB_ITEMS(BSV, DV)                                                                                            \
+    do {                                                                                                              \
+        if (op == SFB_TN_OP) {                                                                                        \
+            if (b_dtype == SFB_BF16) dsd_tn_kernel<BSV, DV, __bf16, __bf16, true, true><<<grid, dim3(BSV * 2), 0, s>>>(p); \
+            else dsd_tn_kernel<BSV, DV, float, float, true, true><<<grid, dim3(BSV * 2), 0, s>>>(p);                  \
+        } else {                                                                                                      \
+            if (b_dtype == SFB_BF16) dsd_nn_kernel<BSV, DV, __bf16, __bf16, true, true><<<grid, dim3(BSV * 2), 0, s>>>(p); \
+            else dsd_nn_kernel<BSV, DV, float, float, true, true><<<grid, dim3(BSV * 2), 0, s>>>(p);                  \
+        }                                                                                                             \
+    } while (0)
+        if (block_size == 64) {
+            if (pad == 32) SFB_ITEMS(64, 32); else if (pad == 64) SFB_ITEMS(64, 64); else if (pad == 96) SFB_ITEMS(64, 96); else SFB_ITEMS(64, 128);
+        } else {
+            if (pad == 32) SFB_ITEMS(32, 32); else if (pad == 64) SFB_ITEMS(32, 64); else if (pad == 96) SFB_ITEMS(32, 96); else SFB_ITEMS(32, 128);
+        }
+#undef SFB_ITEMS
+        return launch_status();
+    }
     if (state_dim % 32 != 0) {
         const uint32_t pad = padded_head_state(state_dim);
 #define SFB_TN64(DV, TB, TA) dsd_tn_kernel<64, DV, TA, TB, true><<<grid, dim3(128), 0, s>>>(p)

@@ -47,6 +47,10 @@ def attention_forward(S, dev, zeros, fixture=FORWARD_FIXTURES[0]):
     scores = S.bst_sgemm_nt(nt, q, k, bs, blocks)
     p = S.BlocksparseMaskedSoftmax(nn, S.to_device(S.transpose_mask(mask, blocks, bs)), scores, nb, scale)
     assert rel_err(S.bst_sgemm_xn(nn, p, v, nb).cpu().numpy(), want) <= TOL
+    # the same product over work items, block-rows of more than 2 blocks cut
+    got = S.bst_sgemm_xn_scheduled(nn, p, v, nb, S.to_device(sched["items"]), sched,
+                                   zeros(S.dsd_workspace_bytes(sched, B, H, bs, d)))
+    assert rel_err(got.cpu().numpy(), want) <= TOL
     p2 = S.fusion_attention2(nn, q, k, bs, blocks, scale, mask=m)
     assert rel_err(S.bst_sgemm_xn(nn, p2, v, nb).cpu().numpy(), want) <= TOL
 

@@ -54,7 +54,7 @@ def test_bench_line_of_the_smallest_workload(workload, capsys):
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-12 and "traffic" in roof
     cpu = line["cpu_baseline"]
     assert cpu["kind"] in ("port", "reference") and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
-    for leg in ("streamed", "unfused", "backward_unfused", "backward_fused", "cpu_reference_single_thread"):
+    for leg in ("streamed", "unfused", "dsd_scheduled", "backward_unfused", "backward_fused", "cpu_reference_single_thread"):
         assert leg in line and "error" not in line[leg], (leg, line[leg])
 
 

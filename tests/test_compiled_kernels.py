@@ -74,15 +74,22 @@ def scratch_bytes(body):
     raise AssertionError("no ScratchSize line")
 
 
-def loop_lines(body):
-    """Lines inside any loop: the union of [label, backward branch to it] spans."""
+def loop_lines(body, innermost=False):
+    """Lines inside any loop: the union of [label, backward branch to it] spans.  innermost: the shortest such span
+    only (a block that the compiler laid out behind the loop and that jumps back to the code before it looks like a
+    span around the loop)."""
     labels = {m.group(1): i for i, line in enumerate(body) if (m := re.match(r"^(\.LBB\w+):", line))}
     inside = [False] * len(body)
+    spans = []
     for i, line in enumerate(body):
         m = re.match(r"^\s+s_c?branch\w*\s+(\.LBB\w+)", line)
         if m and labels.get(m.group(1), len(body)) < i:
+            spans.append((i - labels[m.group(1)], labels[m.group(1)], i))
             for k in range(labels[m.group(1)], i + 1):
                 inside[k] = True
+    if innermost:
+        _, first, last = min(spans)
+        return body[first:last + 1]
     return [line for line, keep in zip(body, inside) if keep]
 
 
@@ -163,11 +170,16 @@ def test_sdd_softmax_stream_step_issues_what_its_waits_count(kernels, elem, elem
                                                         {"lds": 3 * loads, "store": passes})
 
 
-def test_dsd_stream_steps_issue_what_their_wait_counts(kernels):
+# the streaming dsd kernel launched by block-rows and by work items
+DSD_STREAM = ["dsd_nn_kernelILi64ELi64EDF16bDF16bLb0ELb0EE", "dsd_nn_kernelILi64ELi64EDF16bDF16bLb0ELb1EE"]
+
+
+@pytest.mark.parametrize("name", DSD_STREAM)
+def test_dsd_stream_steps_issue_what_their_wait_counts(kernels, name):
     L = lib()
-    body = find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bLb0EE")
+    body = find(kernels, name)
     assert scratch_bytes(body) == 0
-    ev = events(loop_lines(body))
+    ev = events(loop_lines(body, innermost=True))
     spans = between_counted_waits(ev, L.ti_dsd_wait_count())
     assert len(spans) == L.ti_dsd_depth() // 2
     for span in spans:
@@ -216,11 +228,12 @@ def in_flight_violations(code, laxer_by=0):
     return loads_seen, touched
 
 
-def test_registers_of_loads_in_flight_are_left_alone(kernels):
+@pytest.mark.parametrize("name", DSD_STREAM)
+def test_registers_of_loads_in_flight_are_left_alone(kernels, name):
     """dsd (bf16): the P blocks are loaded into registers from inline assembly several blocks ahead and made valid by a
     counted wait, so the compiler believes them defined from the moment of issue: it must not read, copy or spill
     them before the wait that retires their loads.  Checked on the compiled loop (one straight-line block)."""
-    body = loop_lines(find(kernels, "dsd_nn_kernelILi64ELi64EDF16bDF16bLb0EE"))
+    body = loop_lines(find(kernels, name), innermost=True)
     code = [line.strip() for line in body if re.match(r"^\s+[a-z]", line)]
     assert not any(re.match(r"s_c?branch", c.split()[0]) for c in code[:-1]), "one straight-line block"
     loads_seen, touched = in_flight_violations(code)
