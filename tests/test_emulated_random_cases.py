@@ -154,6 +154,12 @@ def test_one_table_and_mask_per_head(E, seed):
     p2 = E.fusion_attention2(nnd, q, k, bs, blocks, scale, mask=md, valid_len=vd, out_dtype=code, lut_heads=H, mask_heads=mask_heads)
     check("two-stage fusion", p2.float().numpy(), P_want, tol, case)
     check("dsd", E.bst_sgemm_xn(nnd, p2, v, nb, lut_heads=H).numpy(), want, 2 * tol if bf16 else tol, case)
+    if p2.dtype == v.dtype:   # the same product over work items, lines cut at a random length
+        cut = int(rng.integers(1, 5))
+        sched = E.build_schedule_heads(nn, nb, H, cut) if H > 1 else E.build_schedule(nn, nb, cut)
+        ws = emu_lib.empty((max(E.dsd_workspace_bytes(sched, B, H, bs, d), 256),), torch.uint8, fill=0xFF)
+        got = E.bst_sgemm_xn_scheduled(nnd, p2, v, nb, E.to_device(sched["items"]), sched, ws, lut_heads=H)
+        check("dsd over work items", got.numpy(), want, 2 * tol if bf16 else tol, dict(case, cut=cut))
 
 
 @pytest.mark.parametrize("seed", range(8))

@@ -1,8 +1,9 @@
 """Do the tests on the host model notice mistakes in the real kernels?  Each case builds the host model with one
 deliberate mistake in a kernel source -- a wait or a barrier taken out of a tile pipeline, a swizzle dropped on the
 loading side, a merge that does not wait for its partial records, an arrival counter that is not reset, a counted wait
-one tile short -- and expects the corresponding test of test_emulated_kernels.py to FAIL under at least one of the
-lane orders / load timings it uses (and the unmodified build to pass, which the CPU suite checks anyway).
+one tile short, chunk sums of a cut line that overwrite one another or are left out of the reduction -- and expects
+the corresponding test of the CPU suite to FAIL under at least one of the lane orders / load timings it uses (and the
+unmodified build to pass, which the CPU suite checks anyway).
 A build per mistake: minutes.  Run with `pytest tests/test_host_model_mutants.py --mutants`."""
 import pytest
 import torch
@@ -33,9 +34,24 @@ MUTANTS = {
     "dsd_wait_one_tile_short": dict(
         source="unfused_attention.hip", old="do { emu::s_waitcnt_vmcnt((0)); } while (0)",
         new="do { emu::s_waitcnt_vmcnt((DsdStreamWait::V_LOADS)); } while (0)"),
+    "chunks_of_a_cut_line_share_a_record": dict(
+        source="unfused_attention.hip", old="it.nchunks > 1 ? it.part + it.chunk + 1 : 0u", new="it.nchunks > 1 ? it.part + 1 : 0u"),
+    "reduction_leaves_out_the_last_chunk": dict(
+        source="unfused_attention.hip", old="for (uint32_t ch = 0; ch < it.nchunks; ++ch)\n            sum +=",
+        new="for (uint32_t ch = 0; ch + 1 < it.nchunks; ++ch)\n            sum +="),
 }
 
+
+def scheduled_dsd(M, order, lazy):
+    import scheduled_dsd_cases
+    emu_lib.configure(order=order, lazy_loads=lazy)
+    poisoned = lambda n: emu_lib.empty((max(int(n), 256),), torch.uint8, fill=0xFF)   # noqa: E731
+    scheduled_dsd_cases.products(M, emu_lib.tensor, poisoned, 64, 64, True)
+
+
 CHECKS = {
+    "chunks_of_a_cut_line_share_a_record": scheduled_dsd,
+    "reduction_leaves_out_the_last_chunk": scheduled_dsd,
     "forward_tiles_read_without_the_wait": lambda M, o, l: T.test_fused_forward_plain_scheduled_streamed(M, 64, 64, True, o, l),
     "forward_tiles_read_without_the_barrier": lambda M, o, l: T.test_fused_forward_plain_scheduled_streamed(M, 64, 64, True, o, l),
     "loader_without_the_swizzle": lambda M, o, l: T.test_fused_forward_plain_scheduled_streamed(M, 64, 64, True, o, l),
