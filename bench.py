@@ -236,7 +236,10 @@ def time_backward(sfb, torch, luts, q, k, v, bs, blocks, scale, bf16):
     grad = _time(torch, lambda: sfb.BlocksparseMaskedSoftmaxGrad(ld["nn_lut"], dp, p, nb, scale, dx=ds), 200, 20)
     o = sfb.bst_sgemm_xn(ld["nn_lut"], p, v, nb)
     delta = sfb.row_dot(d_out, o)
+    schedules = sfb.dsd_schedules(luts, nb, B, H, bs, d)
     return {"ms_per_call": _time(torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale), 100, 20),
+            "ms_per_call_products_over_work_items": _time(
+                torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale, o=o, schedules=schedules), 100, 20),
             "ms_per_call_with_forward_output": _time(
                 torch, lambda: sfb.attention_backward(q, k, v, d_out, p, ld, bs, blocks, scale, o=o), 100, 20),
             "row_dot_ms": _time(torch, lambda: sfb.row_dot(d_out, o), 200, 20),

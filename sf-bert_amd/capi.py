@@ -683,28 +683,48 @@ def sdd_softmax_grad(nt_lut, d_out, v, p, delta, block_size, blocks, scale, lut_
     return ds
 
 
-def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None, o=None):
+def dsd_schedules(luts, nb, batch, heads, block_size, d, max_blocks=16):
+    """Work items and workspaces for the products of attention_backward launched over work items: one set over the
+    NN table (block-rows: dQ) and one over the TN table (block-columns: dV, dK).  luts: build_luts() of one layout."""
+    import torch
+    out = {}
+    for key in ("nn_lut", "tn_lut"):
+        sched = build_schedule(luts[key], nb, max_blocks)
+        nbytes = max(dsd_workspace_bytes(sched, batch, heads, block_size, d), 256)
+        out[key] = dict(items=to_device(sched["items"]), sched=sched,
+                        workspace=torch.empty(nbytes, dtype=torch.uint8, device="cuda"))
+    return out
+
+
+def attention_backward(q, k, v, d_out, p, luts_dev, block_size, blocks, scale, work_dtype=None, o=None, schedules=None):
     """Gradients of O = P V, P = masked softmax(scale * Q K^T) from the stored probabilities P, in the order of
     the reference's backward (transformer_attention_optimize.cu:924-965):
         dV = P^T dO (TN), dP = dO V^T (NT), dS = softmax grad, dK = dS^T Q (TN), dQ = dS K (NN).
     q, k, v, d_out [B, L, H, d]; p [B, H, blocks, bs, bs]; luts_dev: dict of device buffers nt_lut, nn_lut,
     tn_lut.  dP / dS use p's dtype unless work_dtype says otherwise.  o: the forward output O (fp32), optional; when
-    given, dP and the softmax gradient are computed by one kernel (sdd_softmax_grad).  Returns (dq, dk, dv) fp32."""
+    given, dP and the softmax gradient are computed by one kernel (sdd_softmax_grad).  schedules: dsd_schedules() of
+    the layout, optional; the three dsd products whose operands have one type are then launched over its work items
+    (long block-rows and block-columns cut).  Returns (dq, dk, dv) fp32."""
     nb = q.shape[1] // block_size
     code = _dtype_code(p) if work_dtype is None else work_dtype
-    dv = bst_sgemm_xn(luts_dev["tn_lut"], p, d_out, nb, op=TN_OP)
+
+    def product(key, sparse, dense, op):
+        if schedules is not None and sparse.dtype == dense.dtype:
+            s = schedules[key]
+            return bst_sgemm_xn_scheduled(luts_dev[key], sparse, dense, nb, s["items"], s["sched"], s["workspace"], op=op)
+        return bst_sgemm_xn(luts_dev[key], sparse, dense, nb, op=op)
+
+    dv = product("tn_lut", p, d_out, TN_OP)
     if o is not None:
         # with the forward output at hand the NT product and the softmax gradient are one kernel
         ds = sdd_softmax_grad(luts_dev["nt_lut"], d_out, v, p, row_dot(d_out, o), block_size, blocks, scale)
-        dk = bst_sgemm_xn(luts_dev["tn_lut"], ds, q, nb, op=TN_OP)
-        dq = bst_sgemm_xn(luts_dev["nn_lut"], ds, k, nb, op=NN_OP)
-        return dq, dk, dv
+        return product("nn_lut", ds, k, NN_OP), product("tn_lut", ds, q, TN_OP), dv
     dp = bst_sgemm_nt(luts_dev["nt_lut"], d_out, v, block_size, blocks, out_dtype=code)
     if dp.dtype != p.dtype:
         p = p.to(dp.dtype)
     ds = BlocksparseMaskedSoftmaxGrad(luts_dev["nn_lut"], dp, p, nb, scale, dx=dp)
-    dk = bst_sgemm_xn(luts_dev["tn_lut"], ds, q, nb, op=TN_OP)
-    dq = bst_sgemm_xn(luts_dev["nn_lut"], ds, k, nb, op=NN_OP)
+    dk = product("tn_lut", ds, q, TN_OP)
+    dq = product("nn_lut", ds, k, NN_OP)
     return dq, dk, dv
 
 

@@ -182,6 +182,13 @@ def test_attention_backward(pattern, bs, bf16):
     dq2, dk2, dv2 = sfb.attention_backward(q, k, v, do, p, luts_dev, bs, blocks, 0.125, o=o)
     for name, got, want in (("dq", dq2, dQ), ("dk", dk2, dK), ("dv", dv2, dV)):
         assert rel_err(got.cpu().numpy(), want) <= tol, name
+    # the three dsd products launched over work items, block-rows and block-columns of more than 3 blocks cut
+    schedules = sfb.dsd_schedules(luts, nb, B, H, bs, d, max_blocks=3)
+    for forward_output in (None, o):
+        dq3, dk3, dv3 = sfb.attention_backward(q, k, v, do, p, luts_dev, bs, blocks, 0.125, o=forward_output,
+                                               schedules=schedules)
+        for name, got, want in (("dq", dq3, dQ), ("dk", dk3, dK), ("dv", dv3, dV)):
+            assert rel_err(got.cpu().numpy(), want) <= tol, name
 
 
 @pytest.mark.parametrize("d", [32, 96, 128])
