@@ -273,6 +273,10 @@ def test_kernels_under_the_undefined_behaviour_sanitizer(E, request):
         test_unfused_sequence_bf16(S, bs, d, 0, True)
     test_unfused_sequence_fp32(S, 64, 36)
     test_scheduled_launch_with_one_table_per_head(S)
+    import scheduled_dsd_cases
+    poisoned = lambda n: emu_lib.empty((max(int(n), 256),), torch.uint8, fill=0xFF)   # noqa: E731
+    for bs, d, bf16, tables in ((64, 64, True, 1), (32, 40, True, 4), (64, 36, False, 1)):
+        scheduled_dsd_cases.products(S, emu_lib.tensor, poisoned, bs, d, bf16, tables)
 
 
 @pytest.mark.parametrize("name,args", [("attention_host_test", []),
