@@ -263,6 +263,37 @@ int main() {
         std::printf("fused backward: <dV,V> = %.5f, <dO,O> = %.5f; <dQ,Q> = %.5f, <dK,K> = %.5f\n", dv_v, do_o, dq_q, dk_k);
         if (!(std::fabs(dv_v - do_o) <= 2e-3 * abs_v)) ++failures;
         if (!(std::fabs(dq_q - dk_k) <= 2e-3 * abs_q)) ++failures;
+
+        // O = P V over the same work items (block-rows of more than 2 blocks cut, their chunk sums added by the
+        // library's second kernel) against the launch by block-rows, on the bf16 P of section 2 and the bf16 V
+        float *o_rows = nullptr, *o_items = nullptr;
+        void* dsd_ws = nullptr;
+        const size_t dsd_bytes = sfb_dsd_workspace_bytes(rows.parts, batch_dim, heads_, blk_size_, head_state_);
+        HIP_OK(hipMalloc((void**)&o_rows, n * sizeof(float)));
+        HIP_OK(hipMalloc((void**)&o_items, n * sizeof(float)));
+        HIP_OK(hipMalloc(&dsd_ws, dsd_bytes + 256));
+        rc = sfb_dsd_xn(stream, (const sfb_uint2*)d_nn, d_p, v16, o_rows, SFB_BF16, SFB_BF16, blk_size_, blocks, batch_dim,
+                        ctx_blks, ctx_blks, heads_, head_state_, 1, ctx_blks + blocks, SFB_NN_OP, magic, shift, nn_max);
+        rc = rc ? rc : sfb_dsd_xn_scheduled(stream, (const sfb_uint2*)d_nn, d_p, v16, o_items, SFB_BF16, SFB_BF16, rows.dev,
+                                            rows.n, rows.heavy, rows.parts, dsd_ws, dsd_bytes + 256, blk_size_, blocks,
+                                            batch_dim, ctx_blks, ctx_blks, heads_, head_state_, 1, ctx_blks + blocks,
+                                            SFB_NN_OP);
+        if (rc != SFB_OK) {
+            std::fprintf(stderr, "dsd over work items failed: %s\n", sfb_status_string(rc));
+            return 1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        std::vector<float> h_rows(n), h_items(n);
+        HIP_OK(hipMemcpy(h_rows.data(), o_rows, n * sizeof(float), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(h_items.data(), o_items, n * sizeof(float), hipMemcpyDeviceToHost));
+        double most = 0, apart = 0;
+        for (size_t i = 0; i < n; ++i) {
+            most = std::fmax(most, std::fabs((double)h_rows[i]));
+            apart = std::fmax(apart, std::fabs((double)h_rows[i] - h_items[i]));
+        }
+        std::printf("dsd over work items (%u items, %u chunk records) vs by block-rows: max |difference| %.3e of %.3e\n",
+                    rows.n, rows.parts, apart, most);
+        if (!(rows.parts > 0 && most > 0 && apart <= 1e-5 * most)) ++failures;
     }
 
     // ---- 5. a block size the kernels do not implement is an error, not a silent no-op ----
